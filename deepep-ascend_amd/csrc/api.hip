@@ -1,0 +1,384 @@
+// extern "C" entry points: argument validation, workspace carving, kernel sequencing.
+// The declarations (and the reference interfaces they stand in for) are in include/deep_ep_hip.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/deep_ep_hip.h"
+#include "common.cuh"
+#include "kernels.h"
+
+namespace deep_ep_hip {
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t err, const char* what) {
+    snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(err));
+    return int(err) > 0 ? int(err) : DEEP_EP_HIP_ERR_INVALID_ARGUMENT;
+}
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+#define REQUIRE(cond, ...)                                                     \
+    do {                                                                       \
+        if (!(cond)) return fail(DEEP_EP_HIP_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+int check_routing_shape(int T, int K, int E, int R) {
+    REQUIRE(T >= 0, "num_tokens must be >= 0 (got %d)", T);
+    REQUIRE(K >= 1 && K <= DEEP_EP_HIP_MAX_TOPK, "num_topk must be in [1, %d] (got %d)", DEEP_EP_HIP_MAX_TOPK, K);
+    REQUIRE(R >= 1 && R <= DEEP_EP_HIP_MAX_RANKS, "num_ranks must be in [1, %d] (got %d)", DEEP_EP_HIP_MAX_RANKS, R);
+    REQUIRE(E >= 1 && E <= DEEP_EP_HIP_MAX_EXPERTS, "num_experts must be in [1, %d] (got %d)", DEEP_EP_HIP_MAX_EXPERTS, E);
+    REQUIRE(E % R == 0, "num_experts (%d) must be divisible by num_ranks (%d)", E, R);
+    return DEEP_EP_HIP_OK;
+}
+
+}  // namespace
+
+WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_experts, int num_ranks) {
+    WorkspaceLayout w{};
+    const size_t n = size_t(num_ranks) + num_experts;
+    const size_t chunks = num_max_tokens > 0 ? (size_t(num_max_tokens) + kLayoutChunk - 1) / kLayoutChunk : 1;
+    const size_t lanes = size_t(num_max_tokens > 0 ? num_max_tokens : 1) * num_topk;
+    size_t off = 0;
+    w.status = off;
+    w.done_counter = off + 4;
+    w.totals = off + 8;
+    off = 256;
+    w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
+    w.chunk_counts = off;  off = align_up(off + chunks * n * 4, 256);
+    w.chunk_base = off;    off = align_up(off + chunks * n * 4, 256);
+    w.pos_rank = off;      off = align_up(off + lanes * 4, 256);
+    w.pos_expert = off;    off = align_up(off + lanes * 4, 256);
+    w.total_bytes = off;
+    return w;
+}
+
+}  // namespace deep_ep_hip
+
+using namespace deep_ep_hip;
+
+extern "C" {
+
+int deep_ep_hip_abi_version(void) { return DEEP_EP_HIP_ABI_VERSION; }
+
+const char* deep_ep_hip_last_error(void) { return g_last_error; }
+
+size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_experts, int num_ranks) {
+    if (num_max_tokens < 0 || num_topk < 1 || num_experts < 1 || num_ranks < 1) return 0;
+    return make_workspace_layout(num_max_tokens, num_topk, num_experts, num_ranks).total_bytes;
+}
+
+size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
+
+int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
+    REQUIRE(a->num_tokens == 0 || a->topk_idx != nullptr, "topk_idx is NULL");
+    REQUIRE(a->num_tokens_per_rank != nullptr && a->num_tokens_per_expert != nullptr, "count outputs are NULL");
+    REQUIRE(a->workspace != nullptr, "workspace is NULL");
+    const WorkspaceLayout w = make_workspace_layout(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks);
+    if (a->workspace_bytes < w.total_bytes)
+        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
+                    (unsigned long long)a->workspace_bytes, w.total_bytes);
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    LayoutParams p{};
+    p.topk_idx = a->topk_idx;
+    p.T = a->num_tokens; p.K = a->num_topk; p.E = a->num_experts; p.R = a->num_ranks;
+    p.E_l = p.E / p.R;
+    p.A = 1;
+    p.num_tokens_per_rank = a->num_tokens_per_rank;
+    p.num_tokens_per_expert = a->num_tokens_per_expert;
+    p.is_token_in_rank = a->is_token_in_rank;
+    p.status = reinterpret_cast<int32_t*>(ws + w.status);
+    p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
+    p.totals = reinterpret_cast<int32_t*>(ws + w.totals);
+    p.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
+    p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
+    p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
+    hipError_t err = launch_layout_kernel(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "layout launch");
+    return DEEP_EP_HIP_OK;
+}
+
+int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    REQUIRE(a != nullptr, "args is NULL");
+    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
+    const int T = a->num_tokens, H = a->hidden, K = a->num_topk, E = a->num_experts, R = a->num_ranks;
+    const bool do_layout = (a->phases & DEEP_EP_HIP_PHASE_LAYOUT) != 0;
+    const bool do_move = (a->phases & DEEP_EP_HIP_PHASE_MOVE) != 0;
+    REQUIRE(do_layout || do_move, "phases selects nothing");
+    REQUIRE(!(a->cached && do_layout), "a cached dispatch has no layout phase");
+    REQUIRE(a->rank_idx >= 0 && a->rank_idx < R, "rank_idx %d outside [0, %d)", a->rank_idx, R);
+    REQUIRE(T <= a->num_max_tokens_per_rank, "num_tokens (%d) exceeds num_max_tokens_per_rank (%d)", T,
+            a->num_max_tokens_per_rank);
+    REQUIRE(int64_t(a->num_max_tokens_per_rank) * R < (int64_t(1) << 31), "num_max_tokens_per_rank * num_ranks overflows int32");
+    REQUIRE(a->expert_alignment >= 1, "expert_alignment must be >= 1");
+    REQUIRE(!a->do_zero_padding || a->do_expand, "do_zero_padding requires do_expand");
+    REQUIRE(T == 0 || a->topk_idx != nullptr, "topk_idx is NULL");
+    REQUIRE(a->workspace != nullptr, "workspace is NULL");
+    REQUIRE(a->psum_num_recv_tokens_per_rank != nullptr && a->psum_num_recv_tokens_per_expert != nullptr &&
+            a->num_unaligned_recv_tokens_per_expert != nullptr, "handle prefix-sum tensors are NULL");
+    const WorkspaceLayout w = make_workspace_layout(T, K, E, R);
+    if (a->workspace_bytes < w.total_bytes)
+        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
+                    (unsigned long long)a->workspace_bytes, w.total_bytes);
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    int32_t* status = reinterpret_cast<int32_t*>(ws + w.status);
+
+    int elem_in = 2, elem_out = 2;
+    switch (a->payload) {
+        case DEEP_EP_HIP_PAYLOAD_BF16: break;
+        case DEEP_EP_HIP_PAYLOAD_FP8: elem_in = elem_out = 1; break;
+        case DEEP_EP_HIP_PAYLOAD_CAST_FP8: elem_out = 1; break;
+        default: return fail(DEEP_EP_HIP_ERR_INVALID_ARGUMENT, "unknown payload kind %d", a->payload);
+    }
+
+    if (do_move) {
+        REQUIRE(H >= 1, "hidden must be positive");
+        REQUIRE((int64_t(H) * elem_in) % 16 == 0, "a row of x must be a multiple of 16 bytes (hidden %d, %d-byte elements)", H, elem_in);
+        REQUIRE(int64_t(H) * elem_in < (int64_t(1) << 30), "row too large");
+        REQUIRE(T == 0 || a->x != nullptr, "x is NULL");
+        REQUIRE(a->recv_x != nullptr || (a->recv_capacity == 0 && a->expanded_capacity == 0), "recv_x is NULL");
+        REQUIRE(a->recv_src_metadata != nullptr || a->recv_capacity == 0, "recv_src_metadata is NULL");
+        REQUIRE(a->dst_buffer_slot_idx != nullptr || T == 0, "dst_buffer_slot_idx is NULL");
+        REQUIRE(a->recv_capacity >= 0 && a->expanded_capacity >= 0, "negative capacity");
+        REQUIRE(a->recv_capacity < (int64_t(1) << 31) && a->expanded_capacity < (int64_t(1) << 31), "capacity overflows int32 rows");
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8) {
+            REQUIRE(a->num_sf_packs >= 0, "num_sf_packs must be >= 0");
+            REQUIRE(a->num_sf_packs == 0 || (a->sf != nullptr && a->recv_sf != nullptr) || T == 0, "sf / recv_sf is NULL");
+        }
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
+            REQUIRE(H % 128 == 0, "the fused FP8 cast needs hidden %% 128 == 0 (got %d)", H);
+            REQUIRE(a->num_sf_packs == H / 128, "num_sf_packs must be hidden / 128 for the fused cast");
+            REQUIRE(a->recv_sf != nullptr || T == 0, "recv_sf is NULL");
+        }
+        REQUIRE(!(a->do_expand == 0 && a->recv_topk_idx == nullptr && a->recv_capacity > 0), "recv_topk_idx is NULL");
+    }
+
+    if (do_layout) {
+        LayoutParams p{};
+        p.topk_idx = a->topk_idx;
+        p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
+        p.A = a->expert_alignment;
+        p.do_expand = a->do_expand;
+        p.copied_topk_idx = a->copied_topk_idx;
+        p.psum_rank = a->psum_num_recv_tokens_per_rank;
+        p.psum_expert = a->psum_num_recv_tokens_per_expert;
+        p.num_unaligned = a->num_unaligned_recv_tokens_per_expert;
+        p.cumulative_stats = a->cumulative_local_expert_recv_stats;
+        p.host_counts = a->host_counts;
+        p.status = status;
+        p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
+        p.totals = reinterpret_cast<int32_t*>(ws + w.totals);
+        p.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
+        p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
+        p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
+        p.pos_rank = reinterpret_cast<int32_t*>(ws + w.pos_rank);
+        p.pos_expert = reinterpret_cast<int32_t*>(ws + w.pos_expert);
+        hipError_t err = launch_layout_kernel(p, stream);
+        if (err != hipSuccess) return hip_fail(err, "dispatch layout launch");
+    }
+
+    if (do_move) {
+        MoveParams m{};
+        m.x = static_cast<const uint8_t*>(a->x);
+        m.sf = static_cast<const uint32_t*>(a->sf);
+        m.sf_ts = a->sf_token_stride; m.sf_hs = a->sf_hidden_stride;
+        m.num_sf_packs = a->num_sf_packs;
+        m.topk_idx = a->topk_idx;
+        m.topk_weights = a->topk_weights;
+        m.pos_rank = reinterpret_cast<const int32_t*>(ws + w.pos_rank);
+        m.pos_expert = reinterpret_cast<const int32_t*>(ws + w.pos_expert);
+        m.chunk_base = reinterpret_cast<const int32_t*>(ws + w.chunk_base);
+        m.expert_start = reinterpret_cast<const int32_t*>(ws + w.expert_start);
+        m.cached_slot = a->dst_buffer_slot_idx;
+        m.dst_buffer_slot_idx = a->dst_buffer_slot_idx;
+        m.psum_rank = a->psum_num_recv_tokens_per_rank;
+        m.recv_src_metadata = a->recv_src_metadata;
+        m.recv_x = static_cast<uint8_t*>(a->recv_x);
+        m.recv_sf = static_cast<uint32_t*>(a->recv_sf);
+        m.rsf_ts = a->recv_sf_token_stride; m.rsf_hs = a->recv_sf_hidden_stride;
+        m.recv_topk_idx = a->recv_topk_idx;
+        m.recv_topk_weights = a->topk_weights != nullptr ? a->recv_topk_weights : nullptr;
+        m.recv_capacity = a->recv_capacity;
+        m.expanded_capacity = a->expanded_capacity;
+        m.T = T; m.H = H; m.K = K; m.E = E; m.R = R; m.E_l = E / R;
+        m.rank_idx = a->rank_idx; m.M = a->num_max_tokens_per_rank;
+        m.cached = a->cached ? 1 : 0;
+        m.do_expand = a->do_expand ? 1 : 0;
+        m.payload = a->payload;
+        m.row_bytes = H * elem_in;
+        m.status = status;
+        hipError_t err = launch_dispatch_move(m, stream);
+        if (err != hipSuccess) return hip_fail(err, "dispatch move launch");
+
+        if (a->do_zero_padding && a->expert_alignment > 1) {
+            PadParams z{};
+            z.recv_x = static_cast<uint8_t*>(a->recv_x);
+            z.recv_sf = (a->payload != DEEP_EP_HIP_PAYLOAD_BF16) ? static_cast<uint32_t*>(a->recv_sf) : nullptr;
+            z.rsf_ts = a->recv_sf_token_stride; z.rsf_hs = a->recv_sf_hidden_stride;
+            z.num_sf_packs = a->num_sf_packs;
+            z.recv_topk_weights = a->topk_weights != nullptr ? a->recv_topk_weights : nullptr;
+            z.psum_expert = a->psum_num_recv_tokens_per_expert;
+            z.num_unaligned = a->num_unaligned_recv_tokens_per_expert;
+            z.expanded_capacity = a->expanded_capacity;
+            z.E = E; z.A = a->expert_alignment;
+            z.out_row_bytes = H * elem_out;
+            err = launch_zero_padding(z, stream);
+            if (err != hipSuccess) return hip_fail(err, "zero padding launch");
+        }
+    }
+    return DEEP_EP_HIP_OK;
+}
+
+int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
+    REQUIRE(a->hidden >= 1 && (int64_t(a->hidden) * 2) % 16 == 0, "hidden (%d) must give rows that are multiples of 16 bytes", a->hidden);
+    REQUIRE(a->rank_idx >= 0 && a->rank_idx < a->num_ranks, "rank_idx %d outside [0, %d)", a->rank_idx, a->num_ranks);
+    REQUIRE(a->num_x_rows >= 0 && a->num_x_rows < (int64_t(1) << 31), "num_x_rows out of range");
+    const bool any = a->num_tokens > 0;
+    REQUIRE(!any || (a->topk_idx != nullptr && a->dst_buffer_slot_idx != nullptr && a->psum_num_recv_tokens_per_rank != nullptr),
+            "handle tensors are NULL");
+    REQUIRE(!any || a->combined_x != nullptr, "combined_x is NULL");
+    REQUIRE(!any || a->x != nullptr || a->num_x_rows == 0, "x is NULL");
+    REQUIRE(!(a->do_expand && any && a->recv_src_metadata == nullptr), "the expanded layout needs recv_src_metadata");
+    REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
+    CombineParams p{};
+    p.x = static_cast<const uint8_t*>(a->x);
+    p.num_x_rows = a->num_x_rows;
+    p.topk_weights = a->topk_weights;
+    p.bias0 = static_cast<const uint8_t*>(a->bias_0);
+    p.bias1 = static_cast<const uint8_t*>(a->bias_1);
+    p.topk_idx = a->topk_idx;
+    p.slot = a->dst_buffer_slot_idx;
+    p.meta = a->recv_src_metadata;
+    p.psum_rank = a->psum_num_recv_tokens_per_rank;
+    p.out = static_cast<uint8_t*>(a->combined_x);
+    p.out_w = a->combined_topk_weights;
+    p.T = a->num_tokens; p.H = a->hidden; p.K = a->num_topk; p.E = a->num_experts; p.R = a->num_ranks;
+    p.E_l = p.E / p.R;
+    p.rank_idx = a->rank_idx; p.M = a->num_max_tokens_per_rank;
+    p.do_expand = a->do_expand ? 1 : 0;
+    p.multi_red = a->allow_multiple_reduction ? 1 : 0;
+    p.status = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a->workspace));
+    hipError_t err = launch_combine_kernel(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "combine launch");
+    return DEEP_EP_HIP_OK;
+}
+
+size_t deep_ep_hip_ll_workspace_bytes(int num_src_ranks, int src_token_stride, int num_topk, int num_local_experts) {
+    if (num_src_ranks < 1 || src_token_stride < 1 || num_topk < 1 || num_local_experts < 1) return 0;
+    const size_t chunks = size_t(num_src_ranks) * ((size_t(src_token_stride) + kLayoutChunk - 1) / kLayoutChunk);
+    size_t off = 256;
+    off = align_up(off + chunks * num_local_experts * 4, 256) ;
+    off = align_up(off + chunks * num_local_experts * 4, 256);
+    off = align_up(off + size_t(num_src_ranks) * src_token_stride * num_topk * 4, 256);
+    return off;
+}
+
+int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    REQUIRE(a->num_src_ranks >= 1 && a->src_token_stride >= 1, "need at least one source rank and one token slot");
+    REQUIRE(a->num_topk >= 1 && a->num_topk <= DEEP_EP_HIP_MAX_TOPK, "num_topk must be in [1, %d]", DEEP_EP_HIP_MAX_TOPK);
+    REQUIRE(a->num_experts >= 1 && a->num_local_experts >= 1 && a->num_local_experts <= DEEP_EP_HIP_MAX_EXPERTS,
+            "bad expert counts");
+    REQUIRE(a->expert_begin >= 0 && a->expert_begin + a->num_local_experts <= a->num_experts, "local expert range outside [0, num_experts)");
+    REQUIRE(a->num_ranks >= 1 && a->src_rank_begin >= 0 && a->src_rank_begin + a->num_src_ranks <= a->num_ranks,
+            "source ranks outside [0, num_ranks)");
+    REQUIRE(a->num_max_dispatch_tokens_per_rank >= 1, "num_max_dispatch_tokens_per_rank must be positive");
+    REQUIRE(int64_t(a->num_ranks) * a->num_max_dispatch_tokens_per_rank < (int64_t(1) << 31), "rows per expert overflow int32");
+    REQUIRE(a->src_token_stride <= a->num_max_dispatch_tokens_per_rank, "src_token_stride exceeds num_max_dispatch_tokens_per_rank");
+    REQUIRE(a->hidden >= 16 && a->hidden % 16 == 0, "hidden must be a multiple of 16");
+    REQUIRE(!a->use_fp8 || a->hidden % 128 == 0, "FP8 needs hidden %% 128 == 0");
+    REQUIRE(!a->use_fp8 || a->packed_recv_x_scales != nullptr, "packed_recv_x_scales is NULL");
+    REQUIRE(a->x != nullptr && a->topk_idx != nullptr && a->packed_recv_x != nullptr && a->packed_recv_count != nullptr &&
+            a->packed_recv_src_info != nullptr && a->packed_recv_layout_range != nullptr, "NULL tensor");
+    const size_t need = deep_ep_hip_ll_workspace_bytes(a->num_src_ranks, a->src_token_stride, a->num_topk, a->num_local_experts);
+    REQUIRE(a->workspace != nullptr, "workspace is NULL");
+    if (a->workspace_bytes < need)
+        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
+                    (unsigned long long)a->workspace_bytes, need);
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    const size_t chunks = size_t(a->num_src_ranks) * ((size_t(a->src_token_stride) + kLayoutChunk - 1) / kLayoutChunk);
+    LLDispatchParams p{};
+    p.use_fp8 = a->use_fp8 ? 1 : 0;
+    p.S = a->num_src_ranks; p.src_rank_begin = a->src_rank_begin; p.src_token_stride = a->src_token_stride;
+    p.num_tokens_per_src = a->num_tokens_per_src;
+    p.H = a->hidden; p.K = a->num_topk; p.E = a->num_experts; p.expert_begin = a->expert_begin;
+    p.E_l = a->num_local_experts; p.R = a->num_ranks; p.M = a->num_max_dispatch_tokens_per_rank;
+    p.x = static_cast<const uint8_t*>(a->x);
+    p.topk_idx = a->topk_idx;
+    p.packed_x = static_cast<uint8_t*>(a->packed_recv_x);
+    p.packed_scales = a->packed_recv_x_scales;
+    p.packed_count = a->packed_recv_count;
+    p.packed_src_info = a->packed_recv_src_info;
+    p.packed_layout_range = a->packed_recv_layout_range;
+    p.cumulative_stats = a->cumulative_local_expert_recv_stats;
+    size_t off = 256;
+    p.status = reinterpret_cast<int32_t*>(ws);
+    p.done_counter = reinterpret_cast<uint32_t*>(ws + 4);
+    p.chunk_counts = reinterpret_cast<int32_t*>(ws + off); off = align_up(off + chunks * p.E_l * 4, 256);
+    p.chunk_base = reinterpret_cast<int32_t*>(ws + off);   off = align_up(off + chunks * p.E_l * 4, 256);
+    p.pos_expert = reinterpret_cast<int32_t*>(ws + off);
+    hipError_t err = launch_ll_dispatch(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "low-latency dispatch launch");
+    return DEEP_EP_HIP_OK;
+}
+
+int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    REQUIRE(a->num_src_ranks >= 1 && a->src_token_stride >= 1, "need at least one source rank and one token slot");
+    REQUIRE(a->num_topk >= 1 && a->num_topk <= DEEP_EP_HIP_MAX_TOPK, "num_topk must be in [1, %d]", DEEP_EP_HIP_MAX_TOPK);
+    REQUIRE(a->hidden >= 8 && (int64_t(a->hidden) * 2) % 16 == 0, "hidden must give rows that are multiples of 16 bytes");
+    REQUIRE(a->num_local_experts >= 1 && a->expert_begin >= 0 && a->expert_begin + a->num_local_experts <= a->num_experts,
+            "local expert range outside [0, num_experts)");
+    REQUIRE(a->num_ranks >= 1 && a->src_rank_begin >= 0 && a->src_rank_begin + a->num_src_ranks <= a->num_ranks,
+            "source ranks outside [0, num_ranks)");
+    REQUIRE(a->num_max_dispatch_tokens_per_rank >= 1, "num_max_dispatch_tokens_per_rank must be positive");
+    REQUIRE(a->x != nullptr && a->topk_idx != nullptr && a->topk_weights != nullptr &&
+            a->packed_recv_src_info != nullptr && a->packed_recv_layout_range != nullptr && a->combined_x != nullptr, "NULL tensor");
+    REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
+    LLCombineParams p{};
+    p.S = a->num_src_ranks; p.src_rank_begin = a->src_rank_begin; p.src_token_stride = a->src_token_stride;
+    p.num_tokens_per_src = a->num_tokens_per_src;
+    p.H = a->hidden; p.K = a->num_topk; p.E = a->num_experts;
+    p.expert_begin = a->expert_begin; p.E_l = a->num_local_experts; p.R = a->num_ranks;
+    p.M = a->num_max_dispatch_tokens_per_rank;
+    p.x = static_cast<const uint8_t*>(a->x);
+    p.topk_idx = a->topk_idx;
+    p.topk_weights = a->topk_weights;
+    p.src_info = a->packed_recv_src_info;
+    p.layout_range = a->packed_recv_layout_range;
+    p.out = static_cast<uint8_t*>(a->combined_x);
+    p.status = reinterpret_cast<int32_t*>(a->workspace);
+    hipError_t err = launch_ll_combine(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "low-latency combine launch");
+    return DEEP_EP_HIP_OK;
+}
+
+int deep_ep_hip_launch_cast_fp8(const deep_ep_hip_cast_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    REQUIRE(a->num_tokens >= 0 && a->hidden >= 1, "bad shape");
+    REQUIRE(a->num_tokens == 0 || (a->x != nullptr && a->out != nullptr && a->scales != nullptr), "NULL tensor");
+    CastParams p{static_cast<const uint8_t*>(a->x), static_cast<uint8_t*>(a->out), a->scales, a->num_tokens, a->hidden};
+    hipError_t err = launch_cast_kernel(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "cast launch");
+    return DEEP_EP_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,38 @@
+// Per-1x128 FP8 e4m3 quantisation of BF16 channels, as a wave-level building block.
+//
+// Follows deep_ep/utils/math.py:30-39: amax over 128 channels clamped below at 1e-4, payload =
+// e4m3(fp32(x) * (448 / amax)), stored scale = amax / 448, both divisions IEEE fp32.  (The
+// low-latency CUDA kernel multiplies by a precomputed 1/448 instead,
+// csrc/kernels/legacy/utils.cuh:477-503; that differs in the last bit of the scale for about
+// half of all amax values, so it is not used here.)
+#pragma once
+
+#include "common.cuh"
+
+namespace deep_ep_hip {
+
+// Each lane holds 16 consecutive BF16 channels in (a, b); 8 consecutive lanes form one group of
+// 128 channels.  Writes the 16 e4m3 bytes to `out` and returns the group's stored scale.
+__device__ __forceinline__ float cast_16_channels(const vec16& a, const vec16& b, vec16& out) {
+    const uint32_t wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    float f[16];
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        f[2 * i] = bf16_lo(wds[i]);
+        f[2 * i + 1] = bf16_hi(wds[i]);
+        amax = fmaxf(amax, fmaxf(fabsf(f[2 * i]), fabsf(f[2 * i + 1])));
+    }
+    amax = fmaxf(group8_max(amax), 1e-4f);
+    const float scale = 448.0f / amax;
+    const float scale_inv = amax / 448.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) f[i] = f[i] * scale;
+    out.x = pack_e4m3x4(f[0], f[1], f[2], f[3]);
+    out.y = pack_e4m3x4(f[4], f[5], f[6], f[7]);
+    out.z = pack_e4m3x4(f[8], f[9], f[10], f[11]);
+    out.w = pack_e4m3x4(f[12], f[13], f[14], f[15]);
+    return scale_inv;
+}
+
+}  // namespace deep_ep_hip

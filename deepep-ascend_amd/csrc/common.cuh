@@ -1,0 +1,129 @@
+// Device helpers shared by the gfx950 routing kernels: wave64 primitives, 16-byte vector
+// access, bf16 / e4m3 conversion.  Everything here is written for CDNA4 (64-wide wavefronts).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace deep_ep_hip {
+
+constexpr int kWaveSize = 64;
+constexpr int kLayoutChunk = 256;   // tokens per layout workgroup (= threads per workgroup)
+
+struct alignas(16) vec16 {
+    uint32_t x, y, z, w;
+};
+
+__device__ __forceinline__ int lane_id() {
+    return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+__device__ __forceinline__ uint64_t lanes_below(int lane) {
+    return (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+}
+
+// Broadcast the value held by `src_lane` (wave-uniform index) to every lane.
+__device__ __forceinline__ int read_lane(int v, int src_lane) {
+    return __builtin_amdgcn_readlane(v, src_lane);
+}
+__device__ __forceinline__ float read_lane(float v, int src_lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
+}
+
+__device__ __forceinline__ vec16 load16(const void* p) {
+    return *reinterpret_cast<const vec16*>(p);
+}
+__device__ __forceinline__ void store16(void* p, const vec16& v) {
+    *reinterpret_cast<vec16*>(p) = v;
+}
+// Streaming (non-temporal) forms for payload that is touched exactly once.
+__device__ __forceinline__ vec16 load16_stream(const void* p) {
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q));
+    return vec16{t.x, t.y, t.z, t.w};
+}
+__device__ __forceinline__ void store16_stream(void* p, const vec16& v) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+}
+
+// bf16 <-> fp32 on raw bits.
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+
+// Round-to-nearest-even fp32 -> bf16; NaN becomes the canonical quiet NaN 0x7fc0.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? 0x7fc0u : rounded;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// fp32 -> OCP e4m3fn, round-to-nearest-even, integer arithmetic only.  Magnitudes above 464
+// (the midpoint past the largest finite value 448; 464 itself ties to even = 448) and NaN give 0x7f.
+__device__ __forceinline__ uint32_t f32_to_e4m3_sw(float f) {
+    const uint32_t u = __float_as_uint(f);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    const uint32_t a = u & 0x7fffffffu;
+    uint32_t r;
+    if (a > 0x43e80000u) {                   // |f| > 464, inf, nan
+        r = 0x7fu;
+    } else if (a >= 0x3c800000u) {           // |f| >= 2^-6: normal e4m3, drop 20 mantissa bits
+        const uint32_t t = a + 0x7ffffu + ((a >> 20) & 1u);
+        r = (t >> 20) - (120u << 3);         // rebias 127 -> 7
+    } else if (a >= 0x3a800000u) {           // 2^-10 <= |f| < 2^-6: subnormal, unit 2^-9
+        const int shift = 20 + (121 - int(a >> 23));       // 21..24
+        const uint32_t m = (a & 0x7fffffu) | 0x800000u;
+        const uint32_t half = 1u << (shift - 1);
+        r = (m + half - 1u + ((m >> shift) & 1u)) >> shift;
+    } else {
+        r = 0u;                              // below half the smallest subnormal (2^-10 ties to even 0)
+    }
+    return sign | r;
+}
+
+#ifndef DEEP_EP_HIP_SOFTWARE_FP8
+#define DEEP_EP_HIP_SOFTWARE_FP8 0
+#endif
+
+// Four fp32 -> four e4m3 bytes packed little-endian (a in bits 0..7).
+__device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d) {
+#if DEEP_EP_HIP_SOFTWARE_FP8
+    return f32_to_e4m3_sw(a) | (f32_to_e4m3_sw(b) << 8) | (f32_to_e4m3_sw(c) << 16) | (f32_to_e4m3_sw(d) << 24);
+#else
+    int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+    return uint32_t(v);
+#endif
+}
+
+// Maximum over each aligned group of 8 consecutive lanes (butterfly over lane xor 1, 2, 4).
+__device__ __forceinline__ float group8_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 1, kWaveSize));
+    v = fmaxf(v, __shfl_xor(v, 2, kWaveSize));
+    v = fmaxf(v, __shfl_xor(v, 4, kWaveSize));
+    return v;
+}
+
+// Inclusive prefix sum across the wave.
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int off = 1; off < kWaveSize; off <<= 1) {
+        int o = __shfl_up(v, off, kWaveSize);
+        if (lane >= off) v += o;
+    }
+    return v;
+}
+
+// Agent-scope relaxed load/store that bypass the per-CU vector cache, for values another
+// workgroup of the same launch has just produced.
+__device__ __forceinline__ int load_agent(const int* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace deep_ep_hip

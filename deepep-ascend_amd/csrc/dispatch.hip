@@ -1,0 +1,344 @@
+// Dispatch payload movement for gfx950: every token row is read once from HBM and written once per
+// destination row (compact: one row per distinct destination rank; expanded: one row per valid
+// (token, lane)), with the optional BF16 -> FP8 e4m3 per-1x128 cast fused between the load and
+// the stores.
+//
+// Replaces the per-token warp loop of deep_ep/include/deep_ep/impls/dispatch.cuh:259-395 together
+// with the receive-side copy of deep_ep/include/deep_ep/impls/dispatch_copy_epilogue.cuh:70-208:
+// on one GPU the "send buffer -> peer recv buffer -> output tensor" chain collapses into a single
+// scatter.  Slot numbers come from the layout pass (scan based, deterministic) instead of atomics.
+//
+// Work decomposition: one wavefront owns one (token, column tile).  All 16-byte loads of the tile
+// are issued first, then the routing metadata is resolved while they are in flight, then the tile
+// is stored to each destination with 16-byte stores.  No LDS, no barriers.
+#include "common.cuh"
+#include "cast.cuh"
+#include "kernels.h"
+#include "../../include/deep_ep_hip.h"
+
+namespace deep_ep_hip {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerBlock = kThreads / kWaveSize;
+
+// Per-lane routing state of one token, lanes [0, K) meaningful.
+struct Route {
+    int e;        // expert id or -1
+    int d;        // destination rank or -1
+    int row_c;    // compact row, on master lanes only (else -1)
+    int my_row;   // compact row of this lane's destination (all valid lanes)
+    int erow;     // expanded row (expanded layout), else -1
+    float w;
+};
+
+__device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int lane, bool first_tile) {
+    Route r{-1, -1, -1, -1, -1, 0.f};
+    const int n = p.R + p.E;
+    const int chunk = t / kLayoutChunk;
+    int slot = -1;
+    if (lane < p.K) {
+        const int64_t raw = p.topk_idx[int64_t(t) * p.K + lane];
+        if (raw >= 0 && raw < p.E) r.e = int(raw);
+        if (p.topk_weights != nullptr) r.w = p.topk_weights[int64_t(t) * p.K + lane];
+        if (p.cached) {
+            const int v = p.cached_slot[int64_t(t) * p.K + lane];
+            slot = v >= 0 ? v - p.rank_idx * p.M : -1;
+        } else {
+            slot = p.pos_rank[int64_t(t) * p.K + lane];
+        }
+    }
+    if (r.e >= 0) {
+        r.d = r.e / p.E_l;
+        if (slot >= 0) {
+            if (!p.cached) slot += p.chunk_base[int64_t(chunk) * n + r.d];
+            r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
+        }
+    } else {
+        slot = -1;
+    }
+    if (first_tile && !p.cached && lane < p.K && p.dst_buffer_slot_idx != nullptr)
+        p.dst_buffer_slot_idx[int64_t(t) * p.K + lane] = (r.e >= 0 && slot >= 0) ? p.rank_idx * p.M + slot : -1;
+
+    // Every valid lane learns the compact row of its destination rank from that rank's master lane.
+    for (int j = 0; j < p.K; ++j) {
+        const int dj = read_lane(r.d, j);
+        const int rj = read_lane(r.row_c, j);
+        if (r.d >= 0 && dj == r.d && rj >= 0) r.my_row = rj;
+    }
+    if (p.do_expand && r.e >= 0) {
+        if (p.cached) {
+            if (r.my_row >= 0 && r.my_row < p.recv_capacity)
+                r.erow = p.recv_src_metadata[int64_t(r.my_row) * (p.K + 2) + 2 + lane];
+        } else {
+            r.erow = p.expert_start[r.e] + p.chunk_base[int64_t(chunk) * n + p.R + r.e] +
+                     p.pos_expert[int64_t(t) * p.K + lane];
+        }
+    }
+    return r;
+}
+
+// Token-level metadata, written once per token (by the wave that owns column tile 0).
+__device__ __forceinline__ void write_token_metadata(const MoveParams& p, const Route& r, int t, int lane) {
+    uint64_t masters = __ballot(r.row_c >= 0);
+    while (masters) {
+        const int j = __builtin_ctzll(masters);
+        masters &= masters - 1;
+        const int row = read_lane(r.row_c, j);
+        const int dj = read_lane(r.d, j);
+        if (row >= p.recv_capacity) {
+            if (lane == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
+            continue;
+        }
+        if (!p.do_expand && lane < p.K) {
+            if (p.recv_topk_idx != nullptr)
+                p.recv_topk_idx[int64_t(row) * p.K + lane] = (r.d == dj) ? int64_t(r.e - dj * p.E_l) : int64_t(-1);
+            if (p.recv_topk_weights != nullptr) p.recv_topk_weights[int64_t(row) * p.K + lane] = r.w;
+        }
+        if (!p.cached && lane < p.K + 2) {
+            int v;
+            if (lane < p.K) v = (p.do_expand && r.d == dj) ? r.erow : -1;
+            else if (lane == p.K) v = p.rank_idx * p.M + t;
+            else v = p.rank_idx * p.K + j;
+            const int col = lane < p.K ? 2 + lane : lane - p.K;
+            p.recv_src_metadata[int64_t(row) * (p.K + 2) + col] = v;
+        }
+    }
+    if (p.do_expand && p.recv_topk_weights != nullptr && r.erow >= 0 && r.erow < p.expanded_capacity)
+        p.recv_topk_weights[r.erow] = r.w;
+}
+
+// Bit mask of lanes that name a destination row, and the row each of them names.
+__device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const Route& r, int& row_of_lane) {
+    if (p.do_expand) {
+        row_of_lane = (r.erow >= 0 && r.erow < p.expanded_capacity) ? r.erow : -1;
+        if (r.erow >= p.expanded_capacity) atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
+    } else {
+        row_of_lane = (r.row_c >= 0 && r.row_c < p.recv_capacity) ? r.row_c : -1;
+    }
+    return __ballot(row_of_lane >= 0);
+}
+
+// ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
+template <int kVecs>
+__global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (work >= int64_t(p.T) * p.tiles) return;
+    const int t = int(work / p.tiles);
+    const int tile = int(work - int64_t(t) * p.tiles);
+
+    vec16 v[kVecs];
+    const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i) {
+        const int off = (tile * kVecs + i) * 1024 + lane * 16;
+        v[i] = vec16{0, 0, 0, 0};
+        if (off < p.row_bytes) v[i] = load16_stream(src + off);
+    }
+
+    const Route r = resolve_route(p, t, lane, tile == 0);
+    if (tile == 0) write_token_metadata(p, r, t, lane);
+
+    int row_of_lane;
+    uint64_t dests = destination_lanes(p, r, row_of_lane);
+    while (dests) {
+        const int j = __builtin_ctzll(dests);
+        dests &= dests - 1;
+        const int row = read_lane(row_of_lane, j);
+        uint8_t* dst = p.recv_x + int64_t(row) * p.row_bytes;
+#pragma unroll
+        for (int i = 0; i < kVecs; ++i) {
+            const int off = (tile * kVecs + i) * 1024 + lane * 16;
+            if (off < p.row_bytes) store16_stream(dst + off, v[i]);
+        }
+        if (tile == 0 && p.recv_sf != nullptr) {
+            for (int g = lane; g < p.num_sf_packs; g += kWaveSize)
+                p.recv_sf[int64_t(row) * p.rsf_ts + int64_t(g) * p.rsf_hs] =
+                    p.sf[int64_t(t) * p.sf_ts + int64_t(g) * p.sf_hs];
+        }
+    }
+}
+
+// ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
+template <int kPairs>
+__global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (work >= int64_t(p.T) * p.tiles) return;
+    const int t = int(work / p.tiles);
+    const int tile = int(work - int64_t(t) * p.tiles);
+
+    vec16 in[kPairs][2];
+    const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
+#pragma unroll
+    for (int q = 0; q < kPairs; ++q) {
+        const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+        in[q][0] = vec16{0, 0, 0, 0};
+        in[q][1] = vec16{0, 0, 0, 0};
+        if (elem < p.H) {
+            in[q][0] = load16_stream(src + int64_t(elem) * 2);
+            in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+        }
+    }
+
+    const Route r = resolve_route(p, t, lane, tile == 0);
+    if (tile == 0) write_token_metadata(p, r, t, lane);
+
+    vec16 out[kPairs];
+    float my_scale = 0.f;   // lane L < 8*kPairs ends up holding the scale of group (tile*kPairs*8 + L)
+#pragma unroll
+    for (int q = 0; q < kPairs; ++q) {
+        const float scale_inv = cast_16_channels(in[q][0], in[q][1], out[q]);
+        const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
+        if ((lane >> 3) == q) my_scale = gathered;
+    }
+    const int group = tile * kPairs * 8 + lane;
+    const bool owns_scale = lane < kPairs * 8 && group * 128 < p.H;
+
+    int row_of_lane;
+    uint64_t dests = destination_lanes(p, r, row_of_lane);
+    while (dests) {
+        const int j = __builtin_ctzll(dests);
+        dests &= dests - 1;
+        const int row = read_lane(row_of_lane, j);
+        uint8_t* dst = p.recv_x + int64_t(row) * p.H;
+#pragma unroll
+        for (int q = 0; q < kPairs; ++q) {
+            const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+            if (elem < p.H) store16_stream(dst + elem, out[q]);
+        }
+        if (owns_scale)
+            p.recv_sf[int64_t(row) * p.rsf_ts + int64_t(group) * p.rsf_hs] = __float_as_uint(my_scale);
+    }
+}
+
+// ---- zero the alignment padding rows of the expanded layout ----
+__global__ __launch_bounds__(kThreads) void zero_padding_kernel(const PadParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    const int pad_slots = p.A - 1;
+    if (work >= int64_t(p.E) * pad_slots) return;
+    const int e = int(work / pad_slots);
+    const int i = int(work - int64_t(e) * pad_slots);
+    const int cnt = p.num_unaligned[e];
+    const int aligned = (cnt + p.A - 1) / p.A * p.A;
+    if (i >= aligned - cnt) return;
+    const int64_t row = int64_t(p.psum_expert[e]) + i;      // start + actual count + i
+    if (row >= p.expanded_capacity) return;
+    uint8_t* dst = p.recv_x + row * p.out_row_bytes;
+    const vec16 zero{0, 0, 0, 0};
+    for (int off = lane * 16; off < p.out_row_bytes; off += kWaveSize * 16) store16(dst + off, zero);
+    if (p.recv_sf != nullptr)
+        for (int g = lane; g < p.num_sf_packs; g += kWaveSize) p.recv_sf[row * p.rsf_ts + int64_t(g) * p.rsf_hs] = 0u;
+    if (p.recv_topk_weights != nullptr && lane == 0) p.recv_topk_weights[row] = 0.f;
+}
+
+// ---- stand-alone per-token cast (identity routing) ----
+__global__ __launch_bounds__(kThreads) void cast_kernel(const CastParams p) {
+    const int lane = threadIdx.x & 63;
+    const int groups = (p.H + 127) / 128;
+    const int tiles = (p.H + 1023) / 1024;
+    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (work >= int64_t(p.T) * tiles) return;
+    const int t = int(work / tiles);
+    const int tile = int(work - int64_t(t) * tiles);
+    const int elem = tile * 1024 + lane * 16;
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(p.x) + int64_t(t) * p.H;
+    float f[16];
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        f[i] = (elem + i < p.H) ? __uint_as_float(uint32_t(src[elem + i]) << 16) : 0.f;
+        amax = fmaxf(amax, fabsf(f[i]));
+    }
+    amax = fmaxf(group8_max(amax), 1e-4f);
+    const float scale = 448.0f / amax;
+    const float scale_inv = amax / 448.0f;
+    uint8_t* dst = p.out + int64_t(t) * p.H;
+#pragma unroll
+    for (int i = 0; i < 16; i += 4) {
+        const uint32_t packed = pack_e4m3x4(f[i] * scale, f[i + 1] * scale, f[i + 2] * scale, f[i + 3] * scale);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            if (elem + i + b < p.H) dst[elem + i + b] = uint8_t(packed >> (8 * b));
+    }
+    const int group = elem / 128;
+    if ((lane & 7) == 0 && group < groups && elem < p.H) p.scales[int64_t(t) * groups + group] = scale_inv;
+}
+
+template <int kVecs>
+hipError_t launch_copy(MoveParams p, hipStream_t stream) {
+    p.tiles = (p.row_bytes + kVecs * 1024 - 1) / (kVecs * 1024);
+    const int64_t waves = int64_t(p.T) * p.tiles;
+    const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    hipLaunchKernelGGL(dispatch_copy_kernel<kVecs>, dim3(blocks), dim3(kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <int kPairs>
+hipError_t launch_cast(MoveParams p, hipStream_t stream) {
+    p.tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
+    const int64_t waves = int64_t(p.T) * p.tiles;
+    const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    hipLaunchKernelGGL(dispatch_cast_kernel<kPairs>, dim3(blocks), dim3(kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
+int tuning_override(const char* name) {
+    const char* v = getenv(name);
+    return v != nullptr ? atoi(v) : 0;
+}
+
+}  // namespace
+
+hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
+    if (p.T == 0) return hipSuccess;
+    if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
+        // Column tile = kPairs * 1024 channels per wavefront.
+        int pairs = tuning_override("DEEP_EP_HIP_CAST_PAIRS");
+        if (pairs == 0) {
+            const int segs = (p.H + 1023) / 1024;
+            pairs = segs <= 1 ? 1 : segs <= 2 ? 2 : segs <= 4 ? 4 : segs == 7 ? 7 : 4;
+        }
+        switch (pairs) {
+            case 1: return launch_cast<1>(p, stream);
+            case 2: return launch_cast<2>(p, stream);
+            case 7: return launch_cast<7>(p, stream);
+            case 8: return launch_cast<8>(p, stream);
+            default: return launch_cast<4>(p, stream);
+        }
+    }
+    int vecs = tuning_override("DEEP_EP_HIP_COPY_VECS");
+    if (vecs == 0) {
+        const int kb = (p.row_bytes + 1023) / 1024;
+        vecs = kb <= 1 ? 1 : kb <= 2 ? 2 : kb <= 4 ? 4 : (kb % 7 == 0) ? 7 : 8;
+    }
+    switch (vecs) {
+        case 1: return launch_copy<1>(p, stream);
+        case 2: return launch_copy<2>(p, stream);
+        case 4: return launch_copy<4>(p, stream);
+        case 7: return launch_copy<7>(p, stream);
+        default: return launch_copy<8>(p, stream);
+    }
+}
+
+hipError_t launch_zero_padding(const PadParams& p, hipStream_t stream) {
+    if (p.A <= 1 || p.E == 0) return hipSuccess;
+    const int64_t waves = int64_t(p.E) * (p.A - 1);
+    const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    hipLaunchKernelGGL(zero_padding_kernel, dim3(blocks), dim3(kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_cast_kernel(const CastParams& p, hipStream_t stream) {
+    if (p.T == 0) return hipSuccess;
+    const int tiles = (p.H + 1023) / 1024;
+    const int64_t waves = int64_t(p.T) * tiles;
+    const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    hipLaunchKernelGGL(cast_kernel, dim3(blocks), dim3(kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace deep_ep_hip

@@ -1,0 +1,164 @@
+// Internal interface between the C-ABI entry points (api.hip) and the kernel launchers.
+// Parameter blocks are plain structs passed to kernels by value.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace deep_ep_hip {
+
+// Byte offsets of the regions carved out of the caller's workspace.
+struct WorkspaceLayout {
+    size_t status;         // int32: device status bits
+    size_t done_counter;   // uint32: workgroups of the layout kernel that have finished
+    size_t totals;         // int32[2]: total compact rows, total expanded rows (incl. padding)
+    size_t expert_start;   // int32[E]: first expanded row of each expert
+    size_t chunk_counts;   // int32[C][R+E]
+    size_t chunk_base;     // int32[C][R+E]: exclusive prefix over chunks
+    size_t pos_rank;       // int32[Tmax*K]: slot of the token inside its chunk, on master lanes
+    size_t pos_expert;     // int32[Tmax*K]: position of (token, lane) inside its chunk, per expert
+    size_t total_bytes;
+};
+
+WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_experts, int num_ranks);
+
+struct LayoutParams {
+    const int64_t* topk_idx;
+    int T, K, E, R, E_l;
+    int A;            // expert alignment
+    int do_expand;
+    int32_t* num_tokens_per_rank;    // optional
+    int32_t* num_tokens_per_expert;  // optional
+    uint8_t* is_token_in_rank;       // optional
+    int64_t* copied_topk_idx;        // optional
+    int32_t* psum_rank;              // optional
+    int32_t* psum_expert;            // optional
+    int32_t* num_unaligned;          // optional
+    int32_t* cumulative_stats;       // optional
+    int32_t* host_counts;            // optional, host-mapped
+    int32_t* status;
+    uint32_t* done_counter;
+    int32_t* totals;
+    int32_t* expert_start;
+    int32_t* chunk_counts;
+    int32_t* chunk_base;
+    int32_t* pos_rank;               // optional (layout-only calls skip the per-lane positions)
+    int32_t* pos_expert;
+};
+
+hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream);
+
+struct MoveParams {
+    const uint8_t* x;
+    const uint32_t* sf;
+    int64_t sf_ts, sf_hs;
+    int num_sf_packs;
+    const int64_t* topk_idx;
+    const float* topk_weights;
+    const int32_t* pos_rank;
+    const int32_t* pos_expert;
+    const int32_t* chunk_base;
+    const int32_t* expert_start;
+    const int32_t* cached_slot;
+    int32_t* dst_buffer_slot_idx;
+    const int32_t* psum_rank;
+    int32_t* recv_src_metadata;
+    uint8_t* recv_x;
+    uint32_t* recv_sf;
+    int64_t rsf_ts, rsf_hs;
+    int64_t* recv_topk_idx;
+    float* recv_topk_weights;
+    int64_t recv_capacity, expanded_capacity;
+    int T, H, K, E, R, E_l, rank_idx, M;
+    int cached, do_expand;
+    int payload;         // DEEP_EP_HIP_PAYLOAD_*
+    int row_bytes;       // input row bytes
+    int tiles;           // column tiles per token
+    int32_t* status;
+};
+
+hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream);
+
+struct PadParams {
+    uint8_t* recv_x;
+    uint32_t* recv_sf;
+    int64_t rsf_ts, rsf_hs;
+    int num_sf_packs;
+    float* recv_topk_weights;
+    const int32_t* psum_expert;     // start + actual count (expanded convention)
+    const int32_t* num_unaligned;
+    int64_t expanded_capacity;
+    int E, A, out_row_bytes;
+};
+
+hipError_t launch_zero_padding(const PadParams& p, hipStream_t stream);
+
+struct CombineParams {
+    const uint8_t* x;
+    int64_t num_x_rows;
+    const float* topk_weights;
+    const uint8_t* bias0;
+    const uint8_t* bias1;
+    const int64_t* topk_idx;
+    const int32_t* slot;
+    const int32_t* meta;
+    const int32_t* psum_rank;
+    uint8_t* out;
+    float* out_w;
+    int T, H, K, E, R, E_l, rank_idx, M;
+    int do_expand, multi_red;
+    int tiles;
+    int32_t* status;
+};
+
+hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream);
+
+struct CastParams {
+    const uint8_t* x;
+    uint8_t* out;
+    float* scales;
+    int T, H;
+};
+
+hipError_t launch_cast_kernel(const CastParams& p, hipStream_t stream);
+
+struct LLDispatchParams {
+    int use_fp8;
+    int S, src_rank_begin, src_token_stride;
+    const int32_t* num_tokens_per_src;
+    int H, K, E, expert_begin, E_l, R, M;
+    const uint8_t* x;
+    const int64_t* topk_idx;
+    uint8_t* packed_x;
+    float* packed_scales;
+    int32_t* packed_count;
+    int32_t* packed_src_info;
+    int64_t* packed_layout_range;
+    int32_t* cumulative_stats;
+    // workspace
+    int32_t* status;
+    uint32_t* done_counter;
+    int32_t* chunk_counts;   // [C][E_l]
+    int32_t* chunk_base;     // [C][E_l]
+    int32_t* pos_expert;     // [S*stride*K]
+};
+
+hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream);
+
+struct LLCombineParams {
+    int S, src_rank_begin, src_token_stride;
+    const int32_t* num_tokens_per_src;
+    int H, K, E, expert_begin, E_l, R, M;
+    const uint8_t* x;
+    const int64_t* topk_idx;
+    const float* topk_weights;
+    const int32_t* src_info;
+    const int64_t* layout_range;
+    uint8_t* out;
+    int32_t* status;
+};
+
+hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream);
+
+}  // namespace deep_ep_hip

@@ -1,0 +1,204 @@
+// Dispatch layout for gfx950: one pass over topk_idx produces per-rank / per-expert counts, the
+// token->rank membership, and (for dispatch) the deterministic position of every (token, lane)
+// inside its destination bucket.
+//
+// Replaces csrc/kernels/legacy/layout.cu:10-122 (get_dispatch_layout, where every block rescans
+// the whole index array) and the notify warps of deep_ep/include/deep_ep/impls/dispatch.cuh:79-258
+// (per-rank / per-expert counts, aligned prefix sums, host mailbox).
+//
+// Design: a workgroup owns a chunk of 256 consecutive tokens (one lane per token).  Each wave sets
+// its lane bit in an LDS bitmap word per rank and per expert (ds_or_b64), so that
+//   count  = popcount(bitmap)                      and
+//   position of token t among chunk tokens routed to the same bucket = popcount(bitmap & lanes below t)
+// with no ordering-dependent atomics: placement is a pure function of the input.  Chunk totals go
+// to global memory; the last workgroup to finish turns them into exclusive chunk bases and into the
+// public prefix sums.
+#include "common.cuh"
+#include "kernels.h"
+#include "../../include/deep_ep_hip.h"
+
+namespace deep_ep_hip {
+
+namespace {
+
+constexpr int kThreads = kLayoutChunk;
+constexpr int kWaves = kThreads / kWaveSize;
+
+// In-place inclusive scan of a[0..n) in LDS by the whole workgroup.  tmp holds kWaves ints.
+__device__ void block_inclusive_scan(int* a, int n, int* tmp) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int per = (n + kThreads - 1) / kThreads;
+    const int begin = min(tid * per, n), end = min(begin + per, n);
+    int s = 0;
+    for (int i = begin; i < end; ++i) s += a[i];
+    const int inc = wave_inclusive_sum(s);
+    if (lane == kWaveSize - 1) tmp[wave] = inc;
+    __syncthreads();
+    int run = inc - s;
+    for (int w = 0; w < wave; ++w) run += tmp[w];
+    for (int i = begin; i < end; ++i) {
+        run += a[i];
+        a[i] = run;
+    }
+    __syncthreads();
+}
+
+template <int KMAX>
+__global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) {
+    extern __shared__ uint64_t bitmap[];   // [(R + E)][kWaves]
+    __shared__ int scan_tmp[kWaves];
+    __shared__ int is_last;
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int chunk = blockIdx.x;
+    const int t = chunk * kThreads + tid;
+    const int n = p.R + p.E;
+    const bool active = t < p.T;
+
+    for (int i = tid; i < n * kWaves; i += kThreads) bitmap[i] = 0ull;
+    __syncthreads();
+
+    int e[KMAX], d[KMAX];
+    int flags = 0;
+    const uint64_t my_bit = 1ull << lane;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        int ev = -1;
+        if (active && k < p.K) {
+            const int64_t raw = p.topk_idx[int64_t(t) * p.K + k];
+            if (p.copied_topk_idx != nullptr) p.copied_topk_idx[int64_t(t) * p.K + k] = raw;
+            if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+            else if (raw >= 0) ev = int(raw);
+        }
+        e[k] = ev;
+        d[k] = ev >= 0 ? ev / p.E_l : -1;
+        if (ev >= 0) {
+            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[(p.R + ev) * kWaves + wave]), my_bit);
+            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[d[k] * kWaves + wave]), my_bit);
+        }
+    }
+    __syncthreads();
+
+    const uint64_t below = lanes_below(lane);
+    auto rank_in_chunk = [&](int bucket) {
+        int pos = __popcll(bitmap[bucket * kWaves + wave] & below);
+        for (int w = 0; w < wave; ++w) pos += __popcll(bitmap[bucket * kWaves + w]);
+        return pos;
+    };
+
+    if (active) {
+        if (p.pos_rank != nullptr) {
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) {
+                if (k >= p.K) break;
+                int pr = -1, pe = -1;
+                if (e[k] >= 0) {
+                    bool master = true;
+#pragma unroll
+                    for (int j = 0; j < KMAX; ++j) {
+                        if (j > k && d[j] == d[k]) master = false;
+                        if (j != k && e[j] == e[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+                    }
+                    pe = rank_in_chunk(p.R + e[k]);
+                    if (master) pr = rank_in_chunk(d[k]);
+                }
+                p.pos_rank[int64_t(t) * p.K + k] = pr;
+                p.pos_expert[int64_t(t) * p.K + k] = pe;
+            }
+        }
+        if (p.is_token_in_rank != nullptr) {
+            for (int r = 0; r < p.R; ++r)
+                p.is_token_in_rank[int64_t(t) * p.R + r] = uint8_t((bitmap[r * kWaves + wave] >> lane) & 1ull);
+        }
+    }
+    if (flags != 0) atomicOr(p.status, flags);
+
+    for (int j = tid; j < n; j += kThreads) {
+        int c = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) c += __popcll(bitmap[j * kWaves + w]);
+        p.chunk_counts[int64_t(chunk) * n + j] = c;
+    }
+
+    // Hand the chunk totals to whichever workgroup finishes last.
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned ticket = atomicAdd(p.done_counter, 1u);
+        is_last = (ticket == gridDim.x - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+
+    // ---- last workgroup: chunk bases and public prefix sums ----
+    int* totals = reinterpret_cast<int*>(bitmap);          // [n]
+    int* aligned = totals + n;                             // [E] then scanned in place
+    const int num_chunks = gridDim.x;
+    for (int j = tid; j < n; j += kThreads) {
+        int running = 0;
+        for (int c = 0; c < num_chunks; ++c) {
+            const int v = load_agent(&p.chunk_counts[int64_t(c) * n + j]);
+            p.chunk_base[int64_t(c) * n + j] = running;
+            running += v;
+        }
+        totals[j] = running;
+    }
+    __syncthreads();
+
+    for (int j = tid; j < p.E; j += kThreads) {
+        const int cnt = totals[p.R + j];
+        aligned[j] = (cnt + p.A - 1) / p.A * p.A;
+        if (p.num_tokens_per_expert != nullptr) p.num_tokens_per_expert[j] = cnt;
+        if (p.num_unaligned != nullptr) p.num_unaligned[j] = cnt;
+        if (p.cumulative_stats != nullptr) p.cumulative_stats[j] += cnt;
+        if (p.host_counts != nullptr) p.host_counts[p.R + j] = -aligned[j] - 1;
+    }
+    for (int r = tid; r < p.R; r += kThreads) {
+        if (p.num_tokens_per_rank != nullptr) p.num_tokens_per_rank[r] = totals[r];
+        if (p.host_counts != nullptr) p.host_counts[r] = -totals[r] - 1;
+    }
+    __syncthreads();
+
+    int* aligned_incl = aligned + p.E;                     // [E]
+    for (int j = tid; j < p.E; j += kThreads) aligned_incl[j] = aligned[j];
+    __syncthreads();
+    block_inclusive_scan(aligned_incl, p.E, scan_tmp);
+    for (int j = tid; j < p.E; j += kThreads) {
+        const int start = aligned_incl[j] - aligned[j];
+        p.expert_start[j] = start;
+        if (p.psum_expert != nullptr) p.psum_expert[j] = p.do_expand ? start + totals[p.R + j] : aligned_incl[j];
+    }
+    const int total_expanded = p.E > 0 ? aligned_incl[p.E - 1] : 0;
+    __syncthreads();
+
+    block_inclusive_scan(totals, p.R, scan_tmp);           // ranks: inclusive prefix in place
+    for (int r = tid; r < p.R; r += kThreads)
+        if (p.psum_rank != nullptr) p.psum_rank[r] = totals[r];
+    if (tid == 0) {
+        p.totals[0] = totals[p.R - 1];
+        p.totals[1] = total_expanded;
+        *p.done_counter = 0u;                              // ready for the next launch
+    }
+    if (p.host_counts != nullptr) __threadfence_system();
+}
+
+}  // namespace
+
+hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream) {
+    const int num_chunks = p.T > 0 ? (p.T + kThreads - 1) / kThreads : 1;
+    const int n = p.R + p.E;
+    // bitmap words, reused by the last workgroup as 3 int arrays of at most n entries
+    const size_t lds = size_t(n) * kWaves * sizeof(uint64_t);
+    dim3 grid(num_chunks), block(kThreads);
+    if (p.K <= 8) {
+        hipLaunchKernelGGL(layout_kernel<8>, grid, block, lds, stream, p);
+    } else if (p.K <= 16) {
+        hipLaunchKernelGGL(layout_kernel<16>, grid, block, lds, stream, p);
+    } else {
+        hipLaunchKernelGGL(layout_kernel<32>, grid, block, lds, stream, p);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace deep_ep_hip

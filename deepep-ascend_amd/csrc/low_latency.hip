@@ -1,0 +1,326 @@
+// Low-latency packed per-expert layout for gfx950: dispatch into [local expert][slot][hidden]
+// buffers with counts, source info and per-source ranges, and the weighted combine back.
+//
+// Replaces csrc/kernels/legacy/internode_ll.cu:128-462 (dispatch: FP8 cast in the send phase,
+// per-(expert, source) packing in the receive phase) and :714-1138 (combine: BF16 branch,
+// weighted fp32 reduce :1072-1135).  Tensor contracts follow csrc/legacy/buffer.hpp:1515-1541.
+// With every logical source resident in local HBM the send/receive phases and the RDMA staging
+// buffers disappear; slots come from a scan, so the fill order is deterministic: source rank
+// ascending, then token ascending (the reference fills in arrival order).
+#include "common.cuh"
+#include "cast.cuh"
+#include "kernels.h"
+#include "../../include/deep_ep_hip.h"
+
+namespace deep_ep_hip {
+
+namespace {
+
+constexpr int kThreads = kLayoutChunk;
+constexpr int kWaves = kThreads / kWaveSize;
+
+__device__ __forceinline__ int tokens_of_source(const LLDispatchParams& p, int s) {
+    const int n = p.num_tokens_per_src != nullptr ? p.num_tokens_per_src[s] : p.src_token_stride;
+    return min(max(n, 0), p.src_token_stride);
+}
+
+// One workgroup per (source rank, chunk of 256 tokens).
+template <int KMAX>
+__global__ __launch_bounds__(kThreads) void ll_count_kernel(const LLDispatchParams p) {
+    extern __shared__ uint64_t bitmap[];   // [E_l][kWaves]
+    __shared__ int is_last;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int chunks_per_src = (p.src_token_stride + kThreads - 1) / kThreads;
+    const int s = blockIdx.x / chunks_per_src;
+    const int c = blockIdx.x - s * chunks_per_src;
+    const int t = c * kThreads + tid;
+    const bool active = t < tokens_of_source(p, s);
+    const int64_t g = int64_t(s) * p.src_token_stride + t;
+
+    for (int i = tid; i < p.E_l * kWaves; i += kThreads) bitmap[i] = 0ull;
+    __syncthreads();
+
+    int le[KMAX];
+    int flags = 0;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        le[k] = -1;
+        if (active && k < p.K) {
+            const int64_t raw = p.topk_idx[g * p.K + k];
+            if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+            else if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l) le[k] = int(raw) - p.expert_begin;
+        }
+        if (le[k] >= 0)
+            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[le[k] * kWaves + wave]), 1ull << lane);
+    }
+    __syncthreads();
+
+    if (active) {
+        const uint64_t below = lanes_below(lane);
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+            if (k >= p.K) break;
+            int pos = -1;
+            if (le[k] >= 0) {
+#pragma unroll
+                for (int j = 0; j < KMAX; ++j)
+                    if (j != k && le[j] == le[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+                pos = __popcll(bitmap[le[k] * kWaves + wave] & below);
+                for (int w = 0; w < wave; ++w) pos += __popcll(bitmap[le[k] * kWaves + w]);
+            }
+            p.pos_expert[g * p.K + k] = pos;
+        }
+    }
+    if (flags != 0) atomicOr(p.status, flags);
+
+    for (int j = tid; j < p.E_l; j += kThreads) {
+        int cnt = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) cnt += __popcll(bitmap[j * kWaves + w]);
+        p.chunk_counts[int64_t(blockIdx.x) * p.E_l + j] = cnt;
+    }
+
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned ticket = atomicAdd(p.done_counter, 1u);
+        is_last = (ticket == gridDim.x - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+
+    for (int j = tid; j < p.E_l; j += kThreads) {
+        int running = 0;
+        for (int src = 0; src < p.S; ++src) {
+            const int begin = running;
+            for (int cc = 0; cc < chunks_per_src; ++cc) {
+                const int64_t b = int64_t(src) * chunks_per_src + cc;
+                const int v = load_agent(&p.chunk_counts[b * p.E_l + j]);
+                p.chunk_base[b * p.E_l + j] = running;
+                running += v;
+            }
+            p.packed_layout_range[int64_t(j) * p.R + p.src_rank_begin + src] =
+                (int64_t(begin) << 32) | int64_t(running - begin);
+        }
+        p.packed_count[j] = running;
+        if (p.cumulative_stats != nullptr) p.cumulative_stats[j] += running;
+    }
+    if (tid == 0) *p.done_counter = 0u;
+}
+
+constexpr int kMoveThreads = 256;
+constexpr int kMoveWaves = kMoveThreads / kWaveSize;
+
+// One wavefront per (token, column tile of kPairs * 1024 channels).
+template <int kPairs, bool kFp8>
+__global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchParams p, const int tiles) {
+    const int lane = threadIdx.x & 63;
+    const int64_t work = int64_t(blockIdx.x) * kMoveWaves + (threadIdx.x >> 6);
+    const int64_t total_tokens = int64_t(p.S) * p.src_token_stride;
+    if (work >= total_tokens * tiles) return;
+    const int64_t g = work / tiles;
+    const int tile = int(work - g * tiles);
+    const int s = int(g / p.src_token_stride);
+    const int t = int(g - int64_t(s) * p.src_token_stride);
+    if (t >= tokens_of_source(p, s)) return;
+
+    const int rows_per_expert = p.R * p.M;
+    const int row_bytes = p.H * 2;
+    vec16 in[kPairs][2];
+    const uint8_t* src = p.x + g * row_bytes;
+#pragma unroll
+    for (int q = 0; q < kPairs; ++q) {
+        const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+        in[q][0] = vec16{0, 0, 0, 0};
+        in[q][1] = vec16{0, 0, 0, 0};
+        if (elem < p.H) {
+            in[q][0] = load16_stream(src + int64_t(elem) * 2);
+            in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+        }
+    }
+
+    // Destination (local expert, slot) of every lane of this token.
+    const int chunks_per_src = (p.src_token_stride + kLayoutChunk - 1) / kLayoutChunk;
+    const int64_t chunk = int64_t(s) * chunks_per_src + t / kLayoutChunk;
+    int le = -1, slot = -1;
+    if (lane < p.K) {
+        const int64_t raw = p.topk_idx[g * p.K + lane];
+        if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) {
+            le = int(raw) - p.expert_begin;
+            slot = p.chunk_base[chunk * p.E_l + le] + p.pos_expert[g * p.K + lane];
+            if (slot >= rows_per_expert) {
+                atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
+                slot = -1;
+            }
+        }
+    }
+    if (tile == 0 && slot >= 0) p.packed_src_info[int64_t(le) * rows_per_expert + slot] = t;
+
+    vec16 out[kPairs];
+    float my_scale = 0.f;
+    if constexpr (kFp8) {
+#pragma unroll
+        for (int q = 0; q < kPairs; ++q) {
+            const float scale_inv = cast_16_channels(in[q][0], in[q][1], out[q]);
+            const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
+            if ((lane >> 3) == q) my_scale = gathered;
+        }
+    }
+    const int group = tile * kPairs * 8 + lane;
+    const int num_groups = p.H / 128;
+    const bool owns_scale = kFp8 && lane < kPairs * 8 && group < num_groups;
+
+    uint64_t dests = __ballot(slot >= 0);
+    while (dests) {
+        const int j = __builtin_ctzll(dests);
+        dests &= dests - 1;
+        const int dle = read_lane(le, j);
+        const int dslot = read_lane(slot, j);
+        const int64_t row = int64_t(dle) * rows_per_expert + dslot;
+        if constexpr (kFp8) {
+            uint8_t* dst = p.packed_x + row * p.H;
+#pragma unroll
+            for (int q = 0; q < kPairs; ++q) {
+                const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+                if (elem < p.H) store16_stream(dst + elem, out[q]);
+            }
+            if (owns_scale)
+                p.packed_scales[(int64_t(dle) * num_groups + group) * rows_per_expert + dslot] = my_scale;
+        } else {
+            uint8_t* dst = p.packed_x + row * row_bytes;
+#pragma unroll
+            for (int q = 0; q < kPairs; ++q) {
+                const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+                if (elem < p.H) {
+                    store16_stream(dst + int64_t(elem) * 2, in[q][0]);
+                    store16_stream(dst + int64_t(elem) * 2 + 16, in[q][1]);
+                }
+            }
+        }
+    }
+}
+
+// Weighted reduce: one wavefront per (token, column tile of kVecs * 512 channels).
+template <int kVecs>
+__global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombineParams p, const int tiles) {
+    const int lane = threadIdx.x & 63;
+    const int64_t work = int64_t(blockIdx.x) * kMoveWaves + (threadIdx.x >> 6);
+    if (work >= int64_t(p.S) * p.src_token_stride * tiles) return;
+    const int64_t g = work / tiles;
+    const int tile = int(work - g * tiles);
+    const int s = int(g / p.src_token_stride);
+    const int t = int(g - int64_t(s) * p.src_token_stride);
+    const int n_s = p.num_tokens_per_src != nullptr ? p.num_tokens_per_src[s] : p.src_token_stride;
+    if (t >= n_s) return;
+    const int src_rank = p.src_rank_begin + s;
+    const int rows_per_expert = p.R * p.M;
+    const int row_bytes = p.H * 2;
+
+    int le = -1;
+    float w = 0.f;
+    if (lane < p.K) {
+        const int64_t raw = p.topk_idx[g * p.K + lane];
+        if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) le = int(raw) - p.expert_begin;
+        w = p.topk_weights[g * p.K + lane];
+    }
+
+    // Find the packed row of every lane: scan that expert's rows from this source for the token id.
+    int row_of_lane = -1;
+    for (int k = 0; k < p.K; ++k) {
+        const int kle = read_lane(le, k);
+        if (kle < 0) continue;
+        const int64_t range = p.layout_range[int64_t(kle) * p.R + src_rank];
+        const int begin = int(range >> 32), count = int(range & 0xffffffff);
+        int found = -1;
+        for (int base = 0; base < count; base += kWaveSize) {
+            const int i = base + lane;
+            const bool hit = i < count && begin + i < rows_per_expert &&
+                             p.src_info[int64_t(kle) * rows_per_expert + begin + i] == t;
+            const uint64_t m = __ballot(hit);
+            if (m) {
+                found = begin + base + __builtin_ctzll(m);
+                break;
+            }
+        }
+        if (lane == k) row_of_lane = found;
+    }
+
+    float acc[kVecs][8];
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[i][c] = 0.f;
+
+    uint64_t srcs = __ballot(row_of_lane >= 0);
+    while (srcs) {
+        const int j = __builtin_ctzll(srcs);
+        srcs &= srcs - 1;
+        const int64_t row = int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j);
+        const float wj = read_lane(w, j);
+        const uint8_t* src = p.x + row * row_bytes;
+#pragma unroll
+        for (int i = 0; i < kVecs; ++i) {
+            const int off = (tile * kVecs + i) * 1024 + lane * 16;
+            if (off < row_bytes) {
+                const vec16 v = load16_stream(src + off);
+                acc[i][0] += bf16_lo(v.x) * wj; acc[i][1] += bf16_hi(v.x) * wj;
+                acc[i][2] += bf16_lo(v.y) * wj; acc[i][3] += bf16_hi(v.y) * wj;
+                acc[i][4] += bf16_lo(v.z) * wj; acc[i][5] += bf16_hi(v.z) * wj;
+                acc[i][6] += bf16_lo(v.w) * wj; acc[i][7] += bf16_hi(v.w) * wj;
+            }
+        }
+    }
+
+    uint8_t* dst = p.out + g * row_bytes;
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i) {
+        const int off = (tile * kVecs + i) * 1024 + lane * 16;
+        if (off < row_bytes) {
+            vec16 o;
+            o.x = pack_bf16x2(acc[i][0], acc[i][1]);
+            o.y = pack_bf16x2(acc[i][2], acc[i][3]);
+            o.z = pack_bf16x2(acc[i][4], acc[i][5]);
+            o.w = pack_bf16x2(acc[i][6], acc[i][7]);
+            store16_stream(dst + off, o);
+        }
+    }
+}
+
+template <int kPairs>
+hipError_t launch_move(const LLDispatchParams& p, hipStream_t stream) {
+    const int tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
+    const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
+    const unsigned blocks = unsigned((waves + kMoveWaves - 1) / kMoveWaves);
+    if (p.use_fp8) hipLaunchKernelGGL((ll_move_kernel<kPairs, true>), dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    else hipLaunchKernelGGL((ll_move_kernel<kPairs, false>), dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
+    if (p.S <= 0 || p.src_token_stride <= 0) return hipSuccess;
+    const int chunks_per_src = (p.src_token_stride + kThreads - 1) / kThreads;
+    const unsigned blocks = unsigned(p.S) * chunks_per_src;
+    const size_t lds = size_t(p.E_l) * kWaves * sizeof(uint64_t);
+    if (p.K <= 8) hipLaunchKernelGGL(ll_count_kernel<8>, dim3(blocks), dim3(kThreads), lds, stream, p);
+    else if (p.K <= 16) hipLaunchKernelGGL(ll_count_kernel<16>, dim3(blocks), dim3(kThreads), lds, stream, p);
+    else hipLaunchKernelGGL(ll_count_kernel<32>, dim3(blocks), dim3(kThreads), lds, stream, p);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    // Small token counts: split rows finely so that more wavefronts share the work.
+    return (p.H > 2048) ? launch_move<1>(p, stream) : launch_move<2>(p, stream);
+}
+
+hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream) {
+    if (p.S <= 0 || p.src_token_stride <= 0) return hipSuccess;
+    constexpr int kVecs = 1;
+    const int tiles = (p.H * 2 + kVecs * 1024 - 1) / (kVecs * 1024);
+    const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
+    const unsigned blocks = unsigned((waves + kMoveWaves - 1) / kMoveWaves);
+    hipLaunchKernelGGL(ll_combine_kernel<kVecs>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    return hipGetLastError();
+}
+
+}  // namespace deep_ep_hip

@@ -1,0 +1,517 @@
+"""Host runtime of the HIP backend: the objects the reference exposes from its compiled
+`deep_ep._C` module (csrc/python_api.cpp:37-54, csrc/elastic/binding.hpp:9-44), written over the
+C ABI in include/deep_ep_hip.h.  PyTorch supplies device memory and streams only.
+
+Public names (same set as the reference's binding contract, tests/platform/api_contract.py):
+`get_platform`, `topk_idx_t`, `EventHandle`, `ElasticBuffer`, `calculate_elastic_buffer_size`,
+plus `get_elastic_buffer_alignment`.
+
+One GPU, logical ranks: `num_ranks` only decides which bucket (destination rank) an expert
+belongs to; every bucket lives in this GPU's HBM.  One call moves the tokens of the logical
+source rank `rank_idx`.
+"""
+import ctypes
+import os
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import _abi
+
+topk_idx_t = torch.int64          # EP_NUM_TOPK_IDX_BITS default (csrc/python_api.cpp:21-35)
+_ALIGNMENT_BYTES = 2 * 1024 * 1024  # symmetric::kNumAlignmentBytes (csrc/elastic/buffer.hpp:1363-1365)
+_TMA_ALIGN = 32                     # ptx::kNumTMAAlignBytes, used only by the size calculus
+
+
+def get_platform() -> str:
+    return "hip"
+
+
+def get_elastic_buffer_alignment() -> int:
+    return _ALIGNMENT_BYTES
+
+
+def _align(x: int, y: int) -> int:
+    return (x + y - 1) // y * y
+
+
+def _host_assert(cond: bool, what: str) -> None:
+    # EP_HOST_ASSERT raises EPException -> RuntimeError in Python (exception.cuh:11-34)
+    if not cond:
+        raise RuntimeError(f"Assertion failed: {what}")
+
+
+class EventHandle:
+    """An event recorded on a stream at construction (csrc/utils/event.hpp:10-42)."""
+
+    def __init__(self, stream: Optional[torch.cuda.Stream] = None):
+        self.event = torch.cuda.Event()
+        self.event.record(stream if stream is not None else torch.cuda.current_stream())
+        self.tensors_to_record: list = []
+
+    def __copy__(self):
+        other = EventHandle.__new__(EventHandle)
+        other.event = self.event
+        other.tensors_to_record = list(self.tensors_to_record)
+        return other
+
+    def current_stream_wait(self) -> None:
+        torch.cuda.current_stream().wait_event(self.event)
+
+
+def _token_record_bytes(hidden_bytes: int, sf_bytes: int, num_topk: int, with_metadata: bool) -> int:
+    # deep_ep/include/deep_ep/common/layout.cuh:187-208
+    meta = num_topk * 8 + ((1 + num_topk) * 4 if with_metadata else 0)
+    return _align(hidden_bytes, _TMA_ALIGN) + _align(sf_bytes, _TMA_ALIGN) + _align(meta, _TMA_ALIGN)
+
+
+def calculate_elastic_buffer_size(comm_handle, num_max_tokens_per_rank: int, hidden: int, num_topk: int,
+                                  use_fp8_dispatch: bool, allow_hybrid_mode: bool,
+                                  allow_multiple_reduction: bool, num_ranks: Optional[int] = None) -> int:
+    """Size the reference would ask for (csrc/elastic/buffer.hpp:588-688, direct mode, peers reachable
+    by load/store).  The HIP backend scatters straight into the output tensors and needs no staging
+    buffer; the number is kept so `num_bytes` / `get_buffer_size_hint` stay drop-in.
+    `comm_handle` is the logical rank count here (there is no communicator)."""
+    _host_assert(num_max_tokens_per_rank > 0 and hidden > 0, "num_max_tokens_per_rank > 0 and hidden > 0")
+    _host_assert(-(-hidden // 32) * 4 <= hidden, "ceil_div(hidden, 32) * sizeof(float) <= hidden")
+    ranks = int(num_ranks if num_ranks is not None else (comm_handle if comm_handle else 1))
+    topk = 32 if num_topk == 0 else num_topk
+    elem = 1 if use_fp8_dispatch else 2
+    sf_packs = -(-hidden // 32) if use_fp8_dispatch else 0
+    dispatch_record = _token_record_bytes(hidden * elem, sf_packs * 4, topk, True)
+    dispatch_bytes = ranks * num_max_tokens_per_rank * dispatch_record
+    combine_record = _token_record_bytes(hidden * 2, 0, topk, False)
+    tokens_in_layout = min(ranks, topk) if allow_multiple_reduction else topk
+    combine_bytes = tokens_in_layout * num_max_tokens_per_rank * combine_record
+    return _align(max(dispatch_bytes, combine_bytes), _ALIGNMENT_BYTES)
+
+
+class ElasticBuffer:
+    """Host side of dispatch / combine (the role of csrc/elastic/buffer.hpp:83-1345 on CUDA and of
+    csrc/backends/ascend/elastic_buffer.hpp on Ascend): checks arguments, allocates outputs,
+    sequences the kernels on the right stream and returns the reference's tuples."""
+
+    cpu_comm_t = list
+
+    def __init__(self, rank_idx: int, num_ranks: int, comm_handle: int, cpu_comm,
+                 num_buffer_bytes: int, num_cpu_buffer_bytes: int,
+                 allow_hybrid_mode: bool, allow_multiple_reduction: bool,
+                 prefer_overlap_with_compute: bool, sl_idx: int, num_allocated_qps: int,
+                 num_cpu_timeout_secs: int, num_gpu_timeout_secs: int, explicitly_destroy: bool):
+        _host_assert(0 <= rank_idx < num_ranks, "0 <= rank_idx < num_ranks")
+        _host_assert(num_ranks <= _abi.MAX_RANKS, f"num_ranks <= {_abi.MAX_RANKS}")
+        _host_assert(num_buffer_bytes > 0 and num_buffer_bytes % _ALIGNMENT_BYTES == 0,
+                     "num_buffer_bytes > 0 and num_buffer_bytes % kNumAlignmentBytes == 0")
+        _host_assert(num_cpu_buffer_bytes == 0, "CPU buffers are not supported by the HIP backend")
+        if not torch.cuda.is_available():
+            raise RuntimeError("DeepEP HIP backend: no GPU is visible")
+        self.rank_idx = rank_idx
+        self.num_ranks = num_ranks
+        self.num_buffer_bytes = num_buffer_bytes
+        self.allow_hybrid_mode = allow_hybrid_mode
+        self.allow_multiple_reduction = allow_multiple_reduction
+        self.prefer_overlap_with_compute = prefer_overlap_with_compute
+        self.num_cpu_timeout_secs = num_cpu_timeout_secs
+        self.explicitly_destroy = explicitly_destroy
+        self.device = torch.device("cuda", torch.cuda.current_device())
+        self.comm_stream = torch.cuda.Stream(device=self.device)
+        self._workspace: Optional[torch.Tensor] = None
+        self._destroyed = False
+
+    # ---- lifetime ----
+    def destroy(self) -> None:
+        _host_assert(self.explicitly_destroy, "explicitly_destroy")
+        _host_assert(not self._destroyed, "not destroyed")
+        torch.cuda.synchronize(self.device)
+        self._workspace = None
+        self._destroyed = True
+
+    def is_destroyed(self) -> bool:
+        return self._destroyed
+
+    def get_comm_stream(self) -> torch.cuda.Stream:
+        return self.comm_stream
+
+    def get_physical_domain_size(self) -> Tuple[int, int]:
+        # (RDMA ranks, load/store-reachable ranks): every logical rank is local
+        return 1, self.num_ranks
+
+    def get_logical_domain_size(self) -> Tuple[int, int]:
+        # (scale-out ranks, scale-up ranks)
+        return 1, self.num_ranks
+
+    def barrier(self, use_comm_stream: bool = True, with_cpu_sync: bool = False, sequential: bool = True) -> None:
+        # One process, one GPU: ordering between logical ranks is stream ordering.
+        if with_cpu_sync:
+            torch.cuda.synchronize(self.device)
+        if use_comm_stream:
+            self.comm_stream.wait_stream(torch.cuda.current_stream())
+            torch.cuda.current_stream().wait_stream(self.comm_stream)
+        if with_cpu_sync:
+            torch.cuda.synchronize(self.device)
+
+    # ---- helpers ----
+    def _get_workspace(self, num_tokens: int, num_topk: int, num_experts: int) -> torch.Tensor:
+        need = _abi.lib.deep_ep_hip_workspace_bytes(max(num_tokens, 1), num_topk, num_experts, self.num_ranks)
+        if self._workspace is None or self._workspace.numel() < need:
+            # grow geometrically so steady-state calls never allocate
+            size = max(need, 2 * (self._workspace.numel() if self._workspace is not None else 0))
+            self._workspace = torch.zeros(size, dtype=torch.uint8, device=self.device)
+        return self._workspace
+
+    def _read_and_clear_status(self, what: str) -> None:
+        ws = self._workspace
+        status = int(ws[:4].view(torch.int32).item())
+        if status != 0:
+            ws[:4].zero_()
+            reasons = []
+            if status & _abi.STATUS_EXPERT_OUT_OF_RANGE:
+                reasons.append("topk_idx holds an expert id >= num_experts")
+            if status & _abi.STATUS_DUPLICATE_EXPERT:
+                reasons.append("a token selects the same expert twice")
+            if status & _abi.STATUS_ROW_OVERFLOW:
+                reasons.append("a received row did not fit the output tensors")
+            raise RuntimeError(f"DeepEP HIP backend: {what}: " + "; ".join(reasons))
+
+    def _prologue(self, previous_event, allocate_on_comm_stream: bool, async_with_compute_stream: bool):
+        """Returns (compute_stream, run_stream).  The reference always runs on its comm stream
+        (csrc/elastic/buffer.hpp:528-551); when nothing asks for overlap the same ordering is had,
+        without two cross-stream waits, by running on the caller's stream."""
+        compute_stream = torch.cuda.current_stream()
+        if previous_event is not None:
+            _host_assert(allocate_on_comm_stream, "allocate_on_comm_stream")
+        overlap = previous_event is not None or allocate_on_comm_stream or async_with_compute_stream
+        if not overlap:
+            return compute_stream, compute_stream
+        if allocate_on_comm_stream:
+            torch.cuda.set_stream(self.comm_stream)
+        if previous_event is not None:
+            self.comm_stream.wait_event(previous_event.event)
+        else:
+            self.comm_stream.wait_stream(compute_stream)
+        return compute_stream, self.comm_stream
+
+    def _epilogue(self, tensors, compute_stream, run_stream, allocate_on_comm_stream: bool,
+                  async_with_compute_stream: bool) -> Optional[EventHandle]:
+        event = None
+        if run_stream is not compute_stream:
+            if async_with_compute_stream:
+                event = EventHandle(run_stream)
+                if int(os.environ.get("EP_AVOID_RECORD_STREAM", "0")):
+                    event.tensors_to_record = [t for t in tensors if t is not None]
+                else:
+                    for t in tensors:
+                        if t is not None and t.is_cuda:
+                            t.record_stream(compute_stream)
+                            t.record_stream(run_stream)
+            else:
+                compute_stream.wait_stream(run_stream)
+        elif async_with_compute_stream:
+            event = EventHandle(run_stream)
+        if allocate_on_comm_stream:
+            torch.cuda.set_stream(compute_stream)
+        return event
+
+    # ---- dispatch ----
+    def dispatch(self, x: torch.Tensor, sf: Optional[torch.Tensor],
+                 topk_idx: torch.Tensor, topk_weights: Optional[torch.Tensor],
+                 cumulative_local_expert_recv_stats: Optional[torch.Tensor],
+                 cached_num_recv_tokens: Optional[int],
+                 cached_num_expanded_tokens: Optional[int],
+                 cached_num_recv_tokens_per_expert_list: Optional[List[int]],
+                 cached_psum_num_recv_tokens_per_scaleup_rank: Optional[torch.Tensor],
+                 cached_psum_num_recv_tokens_per_expert: Optional[torch.Tensor],
+                 cached_num_unaligned_recv_tokens_per_expert: Optional[torch.Tensor],
+                 cached_dst_buffer_slot_idx: Optional[torch.Tensor],
+                 cached_token_metadata_at_forward: Optional[torch.Tensor],
+                 cached_recv_src_metadata: Optional[torch.Tensor],
+                 cached_channel_linked_list: Optional[torch.Tensor],
+                 num_max_tokens_per_rank: int, num_experts: int, expert_alignment: int,
+                 num_sms: int, num_qps: int,
+                 previous_event: Optional[EventHandle],
+                 previous_event_before_epilogue: Optional[EventHandle],
+                 async_with_compute_stream: bool, allocate_on_comm_stream: bool,
+                 do_handle_copy: bool, do_cpu_sync: bool, do_expand: bool, do_zero_padding: bool,
+                 use_tma_aligned_col_major_sf: bool, cast_to_fp8: bool = False):
+        """Argument order and the 16-tuple returned follow csrc/elastic/buffer.hpp:695-728,1166-1178.
+        `cast_to_fp8` (extension): `x` is BF16 and the FP8 e4m3 cast with per-1x128 fp32 scales is
+        fused into the scatter; the result equals casting first and dispatching the pair."""
+        _host_assert(not self._destroyed, "buffer is destroyed")
+        _host_assert(not do_zero_padding or do_expand, "not do_zero_padding or do_expand")
+        cached_mode = cached_num_recv_tokens is not None
+        if cached_mode:
+            _host_assert(cached_num_recv_tokens_per_expert_list is not None, "cached_num_recv_tokens_per_expert_list")
+            _host_assert(cached_num_expanded_tokens is not None, "cached_num_expanded_tokens")
+            _host_assert(cached_psum_num_recv_tokens_per_scaleup_rank is not None, "cached psum per rank")
+            _host_assert(cached_psum_num_recv_tokens_per_expert is not None, "cached psum per expert")
+            _host_assert(cached_dst_buffer_slot_idx is not None, "cached_dst_buffer_slot_idx")
+            _host_assert(cached_recv_src_metadata is not None, "cached_recv_src_metadata")
+            _host_assert(not do_cpu_sync, "Cannot do CPU sync with cached mode")
+            _host_assert(cumulative_local_expert_recv_stats is None, "statistics need a non-cached dispatch")
+
+        _host_assert(x.dim() == 2 and x.is_cuda and x.is_contiguous(), "x is a contiguous 2-D device tensor")
+        num_tokens, hidden = x.shape
+        _host_assert((hidden * x.element_size()) % 16 == 0, "(x.size(1) * x.element_size()) % sizeof(int4) == 0")
+        _host_assert(num_tokens <= num_max_tokens_per_rank, "num_tokens <= num_max_tokens_per_rank")
+        R = self.num_ranks
+        _host_assert(num_experts % R == 0, "num_experts % num_ranks == 0")
+        _host_assert(num_experts <= _abi.MAX_EXPERTS, f"num_experts <= {_abi.MAX_EXPERTS}")
+
+        if cast_to_fp8:
+            _host_assert(sf is None and x.dtype == torch.bfloat16, "cast_to_fp8 takes a BF16 tensor without scales")
+            _host_assert(hidden % 128 == 0, "cast_to_fp8 needs hidden % 128 == 0")
+            payload = _abi.PAYLOAD_CAST_FP8
+            num_sf_packs = hidden // 128
+            out_dtype, sf_dtype = torch.float8_e4m3fn, torch.float32
+            sf_ts = sf_hs = 0
+        elif sf is not None:
+            _host_assert(x.element_size() == 1, "x with scale factors must be a 1-byte type")
+            _host_assert(sf.dim() == 2 and sf.is_cuda and sf.shape[0] == num_tokens, "sf is [num_tokens, num_sf_packs] on device")
+            _host_assert(sf.element_size() == 4, "sf.element_size() == sizeof(sf_pack_t)")
+            payload = _abi.PAYLOAD_FP8
+            num_sf_packs = sf.shape[1]
+            out_dtype, sf_dtype = x.dtype, sf.dtype
+            sf_ts, sf_hs = sf.stride(0), sf.stride(1)
+        else:
+            _host_assert(x.dtype == torch.bfloat16, "x without scale factors must be BF16")
+            payload = _abi.PAYLOAD_BF16
+            num_sf_packs = 0
+            out_dtype, sf_dtype = x.dtype, None
+            sf_ts = sf_hs = 0
+
+        _host_assert(topk_idx is not None and topk_idx.dim() == 2 and topk_idx.shape[0] == num_tokens,
+                     "topk_idx is [num_tokens, num_topk]")
+        num_topk = topk_idx.shape[1]
+        _host_assert(1 <= num_topk <= _abi.MAX_TOPK, f"1 <= num_topk <= {_abi.MAX_TOPK}")
+        _host_assert(topk_idx.dtype == topk_idx_t, "topk_idx.scalar_type() == topk_idx_t")
+        _host_assert(topk_idx.is_cuda and topk_idx.is_contiguous(), "topk_idx is contiguous on device")
+        if topk_weights is not None:
+            _host_assert(tuple(topk_weights.shape) == (num_tokens, num_topk), "topk_weights is [num_tokens, num_topk]")
+            _host_assert(topk_weights.is_cuda and topk_weights.is_contiguous() and topk_weights.dtype == torch.float32,
+                         "topk_weights is contiguous FP32 on device")
+        if cumulative_local_expert_recv_stats is not None:
+            s = cumulative_local_expert_recv_stats
+            _host_assert(s.dim() == 1 and s.shape[0] == num_experts and s.dtype == torch.int32 and s.is_cuda and
+                         s.is_contiguous(), "cumulative_local_expert_recv_stats is int32 [num_experts] on device")
+
+        compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_with_compute_stream)
+        dev = self.device
+        i32 = dict(dtype=torch.int32, device=dev)
+        workspace = self._get_workspace(num_tokens, num_topk, num_experts)
+
+        with torch.cuda.stream(run_stream):
+            if cached_mode:
+                psum_rank = cached_psum_num_recv_tokens_per_scaleup_rank
+                psum_expert = cached_psum_num_recv_tokens_per_expert
+                num_unaligned = cached_num_unaligned_recv_tokens_per_expert
+                _host_assert(psum_rank.shape == (R,) and psum_rank.dtype == torch.int32 and psum_rank.is_cuda,
+                             "cached psum per rank is int32 [num_ranks]")
+                _host_assert(psum_expert.shape == (num_experts,) and psum_expert.dtype == torch.int32,
+                             "cached psum per expert is int32 [num_experts]")
+                _host_assert(num_unaligned is not None and num_unaligned.shape == (num_experts,),
+                             "cached unaligned counts are int32 [num_experts]")
+                dst_slot = cached_dst_buffer_slot_idx
+                _host_assert(tuple(dst_slot.shape) == (num_tokens, num_topk) and dst_slot.dtype == torch.int32 and
+                             dst_slot.is_contiguous(), "cached dst_buffer_slot_idx is int32 [num_tokens, num_topk]")
+                copied_topk_idx = None
+            else:
+                counts = torch.empty(R + 2 * num_experts, **i32)   # one allocation, one D2H copy when syncing
+                psum_rank = counts[:R]
+                psum_expert = counts[R:R + num_experts]
+                num_unaligned = counts[R + num_experts:]
+                dst_slot = torch.empty((num_tokens, num_topk), **i32)
+                copied_topk_idx = torch.empty_like(topk_idx) if do_handle_copy else None
+
+            args = _abi.DispatchArgs()
+            args.payload = payload
+            args.cached = int(cached_mode)
+            args.do_expand = int(do_expand)
+            args.do_zero_padding = int(do_zero_padding)
+            args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
+            args.num_experts, args.num_ranks, args.rank_idx = num_experts, R, self.rank_idx
+            args.num_max_tokens_per_rank = num_max_tokens_per_rank
+            args.expert_alignment = expert_alignment
+            args.x = _abi.ptr(x)
+            args.sf = _abi.ptr(sf)
+            args.sf_token_stride, args.sf_hidden_stride = sf_ts, sf_hs
+            args.num_sf_packs = num_sf_packs
+            args.topk_idx = _abi.ptr(topk_idx)
+            args.topk_weights = _abi.ptr(topk_weights)
+            args.copied_topk_idx = _abi.ptr(copied_topk_idx)
+            args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_rank)
+            args.psum_num_recv_tokens_per_expert = _abi.ptr(psum_expert)
+            args.num_unaligned_recv_tokens_per_expert = _abi.ptr(num_unaligned)
+            args.cumulative_local_expert_recv_stats = _abi.ptr(cumulative_local_expert_recv_stats)
+            args.host_counts = 0
+            args.dst_buffer_slot_idx = _abi.ptr(dst_slot)
+            args.workspace = _abi.ptr(workspace)
+            args.workspace_bytes = workspace.numel()
+            stream_ptr = run_stream.cuda_stream
+
+            # Sizes of the outputs
+            if cached_mode:
+                num_recv_tokens = cached_num_recv_tokens
+                num_expanded_tokens = cached_num_expanded_tokens
+                per_expert_list = list(cached_num_recv_tokens_per_expert_list)
+            elif do_cpu_sync:
+                args.phases = _abi.PHASE_LAYOUT
+                _abi.check(_abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(args), stream_ptr), "dispatch layout")
+                host = counts.cpu()                                  # waits for the layout kernel
+                self._read_and_clear_status("dispatch")
+                num_recv_tokens = int(host[R - 1])
+                unaligned = host[R + num_experts:]
+                aligned = (unaligned + (expert_alignment - 1)) // expert_alignment * expert_alignment
+                per_expert_list = aligned.tolist()
+                num_expanded_tokens = int(aligned.sum())
+            else:
+                num_recv_tokens = num_max_tokens_per_rank * R
+                num_expanded_tokens = num_max_tokens_per_rank * min(num_topk, num_experts) + \
+                    (expert_alignment - 1) * num_experts
+                num_expanded_tokens = _align(num_expanded_tokens, expert_alignment)
+                per_expert_list = []
+
+            num_allocated = num_expanded_tokens if do_expand else num_recv_tokens
+            recv_x = torch.empty((num_allocated, hidden), dtype=out_dtype, device=dev)
+            recv_src_metadata = cached_recv_src_metadata if cached_mode else \
+                torch.empty((num_recv_tokens, num_topk + 2), **i32)
+            recv_sf = None
+            rsf_ts = rsf_hs = 0
+            if sf_dtype is not None:
+                if not use_tma_aligned_col_major_sf:
+                    rsf_ts, rsf_hs = num_sf_packs, 1
+                else:
+                    rsf_ts, rsf_hs = 1, _align(num_allocated, 4)
+                recv_sf = torch.empty_strided((num_allocated, num_sf_packs), (rsf_ts, rsf_hs), dtype=sf_dtype, device=dev)
+            recv_topk_idx = torch.empty((num_allocated, num_topk), dtype=topk_idx.dtype, device=dev) if not do_expand else None
+            recv_topk_weights = None
+            if topk_weights is not None:
+                recv_topk_weights = torch.empty((num_allocated,) if do_expand else (num_allocated, num_topk),
+                                                dtype=torch.float32, device=dev)
+
+            if previous_event_before_epilogue is not None:
+                run_stream.wait_event(previous_event_before_epilogue.event)
+
+            args.phases = _abi.PHASE_MOVE if (cached_mode or do_cpu_sync) else (_abi.PHASE_LAYOUT | _abi.PHASE_MOVE)
+            args.recv_src_metadata = _abi.ptr(recv_src_metadata)
+            args.recv_x = _abi.ptr(recv_x)
+            args.recv_sf = _abi.ptr(recv_sf)
+            args.recv_sf_token_stride, args.recv_sf_hidden_stride = rsf_ts, rsf_hs
+            args.recv_topk_idx = _abi.ptr(recv_topk_idx)
+            args.recv_topk_weights = _abi.ptr(recv_topk_weights)
+            args.recv_capacity = recv_src_metadata.shape[0]
+            args.expanded_capacity = num_expanded_tokens if do_expand else 0
+            _abi.check(_abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(args), stream_ptr), "dispatch")
+
+        event = self._epilogue(
+            [x, sf, topk_idx, topk_weights, recv_x, recv_sf, recv_topk_idx, recv_topk_weights,
+             cumulative_local_expert_recv_stats, copied_topk_idx, psum_rank, psum_expert, num_unaligned,
+             recv_src_metadata, dst_slot, workspace],
+            compute_stream, run_stream, allocate_on_comm_stream, async_with_compute_stream)
+
+        return (recv_x, recv_sf, recv_topk_idx, recv_topk_weights, copied_topk_idx,
+                num_recv_tokens, num_expanded_tokens, per_expert_list,
+                psum_rank, psum_expert, num_unaligned, recv_src_metadata, dst_slot,
+                None, None, event)
+
+    # ---- combine ----
+    def combine(self, x: torch.Tensor, topk_weights: Optional[torch.Tensor],
+                bias_0: Optional[torch.Tensor], bias_1: Optional[torch.Tensor],
+                src_metadata: torch.Tensor, combined_topk_idx: torch.Tensor,
+                psum_num_recv_tokens_per_scaleup_rank: torch.Tensor,
+                token_metadata_at_forward: Optional[torch.Tensor],
+                channel_linked_list: Optional[torch.Tensor],
+                num_experts: int, num_max_tokens_per_rank: int,
+                num_sms: int, num_qps: int,
+                previous_event: Optional[EventHandle],
+                previous_event_before_epilogue: Optional[EventHandle],
+                async_with_compute_stream: bool, allocate_on_comm_stream: bool,
+                use_expanded_layout: bool, dst_buffer_slot_idx: Optional[torch.Tensor] = None):
+        """Argument order and the 3-tuple returned follow csrc/elastic/buffer.hpp:1181-1198,1344.
+        `dst_buffer_slot_idx` (the handle's token -> received-row map) is what lets a single GPU
+        gather instead of routing rows back through a buffer; the Python wrapper passes it."""
+        _host_assert(not self._destroyed, "buffer is destroyed")
+        _host_assert(dst_buffer_slot_idx is not None, "combine needs the handle's dst_buffer_slot_idx")
+        _host_assert(x.dim() == 2 and x.is_cuda and x.is_contiguous(), "x is a contiguous 2-D device tensor")
+        _host_assert(x.dtype == torch.bfloat16, "x.scalar_type() == torch::kBFloat16")
+        num_x_rows, hidden = x.shape
+        _host_assert((hidden * 2) % 16 == 0, "(hidden * sizeof(bf16)) % sizeof(int4) == 0")
+        num_tokens, num_topk = combined_topk_idx.shape
+        _host_assert(combined_topk_idx.dtype == topk_idx_t and combined_topk_idx.is_contiguous(), "handle topk_idx")
+        _host_assert(tuple(dst_buffer_slot_idx.shape) == (num_tokens, num_topk), "handle dst_buffer_slot_idx shape")
+        _host_assert(src_metadata.dim() == 2 and src_metadata.shape[1] == num_topk + 2, "handle recv_src_metadata shape")
+        if topk_weights is not None:
+            _host_assert(topk_weights.dtype == torch.float32 and topk_weights.is_cuda and topk_weights.is_contiguous(),
+                         "topk_weights is contiguous FP32 on device")
+            if use_expanded_layout:
+                _host_assert(topk_weights.dim() == 1 and topk_weights.shape[0] == num_x_rows, "expanded weights are [num_rows]")
+            else:
+                _host_assert(tuple(topk_weights.shape) == (num_x_rows, num_topk), "weights are [num_rows, num_topk]")
+        for b in (bias_0, bias_1):
+            if b is not None:
+                _host_assert(b.dtype == x.dtype and tuple(b.shape) == (num_tokens, hidden) and b.is_cuda and
+                             b.is_contiguous(), "bias is BF16 [num_combined_tokens, hidden]")
+        _host_assert(bias_0 is not None or bias_1 is None, "bias_1 needs bias_0")
+
+        compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_with_compute_stream)
+        workspace = self._get_workspace(num_tokens, num_topk, num_experts)
+        with torch.cuda.stream(run_stream):
+            combined_x = torch.empty((num_tokens, hidden), dtype=x.dtype, device=self.device)
+            combined_topk_weights = None
+            if topk_weights is not None:
+                combined_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
+            if previous_event_before_epilogue is not None:
+                run_stream.wait_event(previous_event_before_epilogue.event)
+            args = _abi.CombineArgs()
+            args.do_expand = int(use_expanded_layout)
+            args.allow_multiple_reduction = int(self.allow_multiple_reduction)
+            args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
+            args.num_experts, args.num_ranks = num_experts, self.num_ranks
+            args.rank_idx, args.num_max_tokens_per_rank = self.rank_idx, num_max_tokens_per_rank
+            args.x = _abi.ptr(x)
+            args.num_x_rows = num_x_rows
+            args.topk_weights = _abi.ptr(topk_weights)
+            args.bias_0, args.bias_1 = _abi.ptr(bias_0), _abi.ptr(bias_1)
+            args.topk_idx = _abi.ptr(combined_topk_idx)
+            args.dst_buffer_slot_idx = _abi.ptr(dst_buffer_slot_idx)
+            args.recv_src_metadata = _abi.ptr(src_metadata)
+            args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_num_recv_tokens_per_scaleup_rank)
+            args.combined_x = _abi.ptr(combined_x)
+            args.combined_topk_weights = _abi.ptr(combined_topk_weights)
+            args.workspace = _abi.ptr(workspace)
+            args.workspace_bytes = workspace.numel()
+            _abi.check(_abi.lib.deep_ep_hip_launch_combine(ctypes.byref(args), run_stream.cuda_stream), "combine")
+
+        event = self._epilogue(
+            [x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx,
+             psum_num_recv_tokens_per_scaleup_rank, dst_buffer_slot_idx, combined_x, combined_topk_weights, workspace],
+            compute_stream, run_stream, allocate_on_comm_stream, async_with_compute_stream)
+        return combined_x, combined_topk_weights, event
+
+    # ---- V1 surface kept on the same runtime ----
+    def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
+                            previous_event: Optional[EventHandle], async_finish: bool,
+                            allocate_on_comm_stream: bool):
+        """csrc/legacy/buffer.hpp:337-404: (num_tokens_per_rank, num_tokens_per_rdma_rank=None,
+        num_tokens_per_expert, is_token_in_rank, event)."""
+        _host_assert(topk_idx.dim() == 2 and topk_idx.is_contiguous() and topk_idx.is_cuda, "topk_idx is contiguous 2-D on device")
+        _host_assert(topk_idx.dtype == topk_idx_t, "topk_idx.scalar_type() == topk_idx_t")
+        _host_assert(num_experts > 0 and num_experts % self.num_ranks == 0, "num_experts % num_ranks == 0")
+        num_tokens, num_topk = topk_idx.shape
+        compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_finish)
+        workspace = self._get_workspace(num_tokens, num_topk, num_experts)
+        with torch.cuda.stream(run_stream):
+            num_tokens_per_rank = torch.empty((self.num_ranks,), dtype=torch.int32, device=self.device)
+            num_tokens_per_expert = torch.empty((num_experts,), dtype=torch.int32, device=self.device)
+            is_token_in_rank = torch.empty((num_tokens, self.num_ranks), dtype=torch.bool, device=self.device)
+            args = _abi.LayoutArgs()
+            args.topk_idx = _abi.ptr(topk_idx)
+            args.num_tokens, args.num_topk, args.num_experts, args.num_ranks = num_tokens, num_topk, num_experts, self.num_ranks
+            args.num_tokens_per_rank = _abi.ptr(num_tokens_per_rank)
+            args.num_tokens_per_expert = _abi.ptr(num_tokens_per_expert)
+            args.is_token_in_rank = _abi.ptr(is_token_in_rank)
+            args.workspace = _abi.ptr(workspace)
+            args.workspace_bytes = workspace.numel()
+            _abi.check(_abi.lib.deep_ep_hip_launch_layout(ctypes.byref(args), run_stream.cuda_stream), "get_dispatch_layout")
+        event = self._epilogue([topk_idx, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, workspace],
+                               compute_stream, run_stream, allocate_on_comm_stream, async_finish)
+        return num_tokens_per_rank, None, num_tokens_per_expert, is_token_in_rank, event

@@ -1,0 +1,316 @@
+"""`ElasticBuffer` / `EPHandle`: the V2 Python surface (reference deep_ep/buffers/elastic.py:40-113,
+331-553, 884-911, 1391-1712) over the single-GPU HIP runtime.
+
+Logical ranks.  `group.size()` is the logical expert-parallel width R and `group.rank()` the logical
+source rank of the tokens this process dispatches.  Destination rank d owns experts
+[d*E/R, (d+1)*E/R); all R destination buckets live in this GPU's HBM.  A dispatch returns the
+concatenation over d of "what d receives from this source": compact rows are ordered by
+(d, token); expanded rows are grouped by global expert id.  Per-expert handle tensors therefore
+have `num_experts` entries.  With R = 1 every shape and value equals the reference's at world
+size 1.  Placement is scan based, hence already deterministic: `deterministic=True` changes nothing.
+"""
+import os
+from typing import List, Optional, Tuple, Union
+
+import torch
+
+from .. import _C
+from .._C import EventHandle
+from ..platform import capture_event, unwrap_event
+from ..utils.event import EventOverlap
+from ..utils.semantic import value_or
+
+
+class LogicalGroup:
+    """Stand-in for a `torch.distributed` group when the ranks are logical: anything with
+    `rank()` and `size()` is accepted by `ElasticBuffer`."""
+
+    def __init__(self, rank: int, size: int):
+        assert 0 <= rank < size
+        self._rank, self._size = rank, size
+
+    def rank(self) -> int:
+        return self._rank
+
+    def size(self) -> int:
+        return self._size
+
+    def barrier(self) -> None:
+        pass
+
+
+class EPHandle:
+    """What `dispatch` returns for `combine` and for cached re-dispatch.
+
+    Attributes:
+        do_expand: whether the expanded (one row per (token, expert)) layout is used.
+        num_experts, expert_alignment, num_max_tokens_per_rank, num_sms: the dispatch settings.
+        topk_idx: the routing the handle was built from, `[num_tokens, num_topk]`.
+        psum_num_recv_tokens_per_scaleup_rank: inclusive prefix of rows per destination rank, `[num_ranks]`.
+        psum_num_recv_tokens_per_expert: per expert, inclusive prefix of aligned counts (compact) or
+            region start + actual count (expanded), `[num_experts]`.
+        num_unaligned_recv_tokens_per_expert: actual rows per expert, `[num_experts]`.
+        num_recv_tokens_per_expert_list: aligned rows per expert as a Python list (empty without CPU sync).
+        recv_src_metadata: `[num_recv_tokens, num_topk + 2]`: source token, source rank * num_topk + master
+            lane, then the expanded row of each lane (-1 if none).
+        dst_buffer_slot_idx: `[num_tokens, num_topk]`: rank_idx * num_max_tokens_per_rank + slot inside the
+            destination bucket on each destination's master (highest) lane, -1 elsewhere.
+        token_metadata_at_forward, channel_linked_list: hybrid-mode fields, always None here.
+        num_recv_tokens, num_expanded_tokens: row counts (upper bounds without CPU sync).
+    """
+
+    def __init__(self, do_expand: bool, num_experts: int, expert_alignment: int,
+                 num_max_tokens_per_rank: int, num_sms: int, topk_idx: torch.Tensor,
+                 num_recv_tokens: int, num_expanded_tokens: int,
+                 num_recv_tokens_per_expert_list: list,
+                 psum_num_recv_tokens_per_scaleup_rank: torch.Tensor,
+                 psum_num_recv_tokens_per_expert: torch.Tensor,
+                 num_unaligned_recv_tokens_per_expert: torch.Tensor,
+                 recv_src_metadata: torch.Tensor, dst_buffer_slot_idx: torch.Tensor,
+                 token_metadata_at_forward: Optional[torch.Tensor],
+                 channel_linked_list: Optional[torch.Tensor]):
+        assert topk_idx is not None
+        self.do_expand = do_expand
+        self.num_experts = num_experts
+        self.expert_alignment = expert_alignment
+        self.num_max_tokens_per_rank = num_max_tokens_per_rank
+        self.num_sms = num_sms
+        self.topk_idx = topk_idx
+        self.psum_num_recv_tokens_per_scaleup_rank = psum_num_recv_tokens_per_scaleup_rank
+        self.psum_num_recv_tokens_per_expert = psum_num_recv_tokens_per_expert
+        self.num_unaligned_recv_tokens_per_expert = num_unaligned_recv_tokens_per_expert
+        self.num_recv_tokens_per_expert_list = num_recv_tokens_per_expert_list
+        self.recv_src_metadata = recv_src_metadata
+        self.dst_buffer_slot_idx = dst_buffer_slot_idx
+        self.token_metadata_at_forward = token_metadata_at_forward
+        self.channel_linked_list = channel_linked_list
+        self.num_recv_tokens = num_recv_tokens
+        self.num_expanded_tokens = num_expanded_tokens
+        self.cached_recv_src_metadata_before_sort = None
+
+
+class ElasticBuffer:
+    """Expert-parallel dispatch / combine on one MI355X.
+
+    Attributes:
+        group, rank_idx, num_ranks: the (logical) communication group.
+        allow_hybrid_mode, allow_multiple_reduction, prefer_overlap_with_compute, deterministic: as given.
+        num_bytes: the buffer size the reference would reserve (kept for compatibility; unused).
+        num_max_tokens_per_rank: default capacity per rank.
+        num_scaleout_ranks / num_scaleup_ranks, scaleout_rank_idx / scaleup_rank_idx,
+        num_rdma_ranks / num_nvlink_ranks: domain sizes (everything is one scale-up domain).
+        runtime: the host runtime (`deep_ep._C.ElasticBuffer`).
+    """
+
+    def __init__(self, group, num_bytes: Optional[int] = None, num_cpu_bytes: int = 0,
+                 num_max_tokens_per_rank: int = 0, hidden: int = 0, num_topk: int = 0,
+                 use_fp8_dispatch: bool = False, deterministic: bool = False,
+                 allow_hybrid_mode: bool = True, allow_multiple_reduction: bool = True,
+                 prefer_overlap_with_compute: bool = True, sl_idx: int = 3, num_allocated_qps: int = 0,
+                 num_cpu_timeout_secs: int = 300, num_gpu_timeout_secs: int = 100,
+                 explicitly_destroy: bool = False):
+        self.group = group
+        self.rank_idx = group.rank()
+        self.num_ranks = group.size()
+        self.allow_hybrid_mode = allow_hybrid_mode
+        self.allow_multiple_reduction = allow_multiple_reduction
+        self.prefer_overlap_with_compute = prefer_overlap_with_compute
+        self.deterministic = deterministic
+        self.comm_handle = None
+
+        if num_bytes is None:
+            num_bytes = _C.calculate_elastic_buffer_size(
+                self.num_ranks, num_max_tokens_per_rank, hidden, num_topk, use_fp8_dispatch,
+                allow_hybrid_mode, allow_multiple_reduction)
+        if os.environ.get('EP_BUFFER_DEBUG', 0):
+            print(f'Initializing EP elastic buffer with {num_bytes} bytes '
+                  f'(cpu: {num_cpu_bytes}) at rank EP {self.rank_idx}/{self.num_ranks}')
+        self.num_bytes = num_bytes
+        self.num_max_tokens_per_rank = num_max_tokens_per_rank
+        self.num_allocated_qps = num_allocated_qps
+        self.explicitly_destroy = explicitly_destroy
+        self.runtime = _C.ElasticBuffer(self.rank_idx, self.num_ranks, 0, [], num_bytes, num_cpu_bytes,
+                                        allow_hybrid_mode, allow_multiple_reduction, prefer_overlap_with_compute,
+                                        sl_idx, num_allocated_qps, num_cpu_timeout_secs, num_gpu_timeout_secs,
+                                        explicitly_destroy)
+        self.num_scaleout_ranks, self.num_scaleup_ranks = self.get_logical_domain_size()
+        self.scaleout_rank_idx = self.rank_idx // self.num_scaleup_ranks
+        self.scaleup_rank_idx = self.rank_idx % self.num_scaleup_ranks
+        self.num_rdma_ranks, self.num_nvlink_ranks = self.get_physical_domain_size()
+
+    def destroy(self) -> None:
+        """Release the runtime. Requires `explicitly_destroy=True` at construction."""
+        assert self.explicitly_destroy
+        if self.runtime is not None:
+            self.runtime.destroy()
+            self.runtime = None
+
+    @staticmethod
+    def get_buffer_size_hint(group, num_max_tokens_per_rank: int, hidden: int, num_topk: int = 0,
+                             use_fp8_dispatch: bool = False, allow_hybrid_mode: bool = True,
+                             allow_multiple_reduction: bool = True) -> int:
+        """The 2 MB-aligned size the reference would recommend for these MoE settings."""
+        return _C.calculate_elastic_buffer_size(group.size(), num_max_tokens_per_rank, hidden, num_topk,
+                                                use_fp8_dispatch, allow_hybrid_mode, allow_multiple_reduction)
+
+    def barrier(self, use_comm_stream: bool = True, with_cpu_sync: bool = False, sequential: bool = True) -> None:
+        self.runtime.barrier(use_comm_stream, with_cpu_sync, sequential)
+
+    @staticmethod
+    def _unpack_handle(handle: Optional[EPHandle] = None):
+        if handle is None:
+            return (None,) * 10
+        return (handle.num_recv_tokens, handle.num_expanded_tokens, handle.num_recv_tokens_per_expert_list,
+                handle.psum_num_recv_tokens_per_scaleup_rank, handle.psum_num_recv_tokens_per_expert,
+                handle.num_unaligned_recv_tokens_per_expert, handle.dst_buffer_slot_idx,
+                handle.token_metadata_at_forward, handle.recv_src_metadata, handle.channel_linked_list)
+
+    @staticmethod
+    def capture() -> EventHandle:
+        """Record an event on the current stream."""
+        return capture_event()
+
+    def get_comm_stream(self) -> torch.cuda.Stream:
+        return self.runtime.get_comm_stream()
+
+    def get_physical_domain_size(self) -> Tuple[int, int]:
+        return self.runtime.get_physical_domain_size()
+
+    def get_logical_domain_size(self) -> Tuple[int, int]:
+        return self.runtime.get_logical_domain_size()
+
+    def get_theoretical_num_sms(self, num_experts: int, num_topk: int, *args, **kwargs) -> int:
+        """The routing kernels are bandwidth bound and always launched over the whole GPU."""
+        return torch.cuda.get_device_properties(self.runtime.device).multi_processor_count
+
+    def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
+                            previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
+                            allocate_on_comm_stream: bool = False):
+        """V1 `Buffer.get_dispatch_layout` (reference deep_ep/buffers/legacy.py:293-319) on this buffer:
+        returns (num_tokens_per_rank[R] int32, None, num_tokens_per_expert[E] int32,
+        is_token_in_rank[T, R] bool, EventOverlap)."""
+        a, b, c, d, event = self.runtime.get_dispatch_layout(topk_idx, num_experts, unwrap_event(previous_event),
+                                                             async_finish, allocate_on_comm_stream)
+        return a, b, c, d, EventOverlap(event)
+
+    def dispatch(self, x: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]],
+                 topk_idx: Optional[torch.Tensor] = None, topk_weights: Optional[torch.Tensor] = None,
+                 cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
+                 num_experts: Optional[int] = None, num_max_tokens_per_rank: Optional[int] = None,
+                 expert_alignment: Optional[int] = None, num_sms: int = 0, num_qps: int = 0,
+                 previous_event: Optional[EventHandle] = None,
+                 previous_event_before_epilogue: Optional[EventHandle] = None,
+                 async_with_compute_stream: bool = False, allocate_on_comm_stream: bool = False,
+                 handle: Optional[EPHandle] = None, do_handle_copy: bool = True,
+                 do_cpu_sync: Optional[bool] = None, do_expand: bool = False, do_zero_padding: bool = False,
+                 use_tma_aligned_col_major_sf: bool = False, cast_to_fp8: bool = False):
+        """Dispatch tokens to the logical destination ranks.
+
+        Arguments follow the reference (`deep_ep/buffers/elastic.py:1391-1412`):
+            x: BF16 `[num_tokens, hidden]`, or a pair (FP8 e4m3 `[num_tokens, hidden]`, scale factors).
+            topk_idx / topk_weights: `[num_tokens, num_topk]` (`deep_ep.topk_idx_t` / float); must be None with `handle`
+                (weights may still be given with a cached handle).
+            cumulative_local_expert_recv_stats: int32 `[num_experts]`, incremented by the per-expert counts.
+            num_experts, num_max_tokens_per_rank, expert_alignment: taken from `handle` / the constructor when None.
+            num_sms, num_qps: accepted and ignored (the kernels use the whole GPU; there are no queue pairs).
+            previous_event, previous_event_before_epilogue, async_with_compute_stream, allocate_on_comm_stream:
+                stream control, as in the reference.
+            handle: a cached `EPHandle` to skip the layout computation.
+            do_handle_copy: clone `topk_idx` into the handle.
+            do_cpu_sync: wait for exact counts and size the outputs exactly (default True unless cached);
+                otherwise outputs have worst-case sizes.
+            do_expand / do_zero_padding / use_tma_aligned_col_major_sf: output layout options.
+            cast_to_fp8 (extension): `x` is BF16; the per-1x128 FP8 e4m3 cast is fused into the scatter and
+                `recv_x` comes back as (FP8, fp32 scales).
+
+        Returns (recv_x or (recv_x, recv_sf), recv_topk_idx, recv_topk_weights, handle, event).
+        """
+        x, sf = x if isinstance(x, tuple) else (x, None)
+
+        if handle is not None:
+            assert topk_idx is None
+            assert do_cpu_sync is None or not do_cpu_sync, 'Cannot do CPU sync with cached handle'
+            topk_idx = handle.topk_idx
+            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, handle.num_max_tokens_per_rank)
+            num_experts = value_or(num_experts, handle.num_experts)
+            expert_alignment = value_or(expert_alignment, handle.expert_alignment)
+            do_cpu_sync = False
+            assert (num_experts, expert_alignment, num_max_tokens_per_rank) == \
+                   (handle.num_experts, handle.expert_alignment, handle.num_max_tokens_per_rank)
+            assert do_expand == handle.do_expand, 'The cached handle was built for the other layout'
+        cached = self._unpack_handle(handle)
+
+        num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
+        expert_alignment = value_or(expert_alignment, 1)
+        do_cpu_sync = value_or(do_cpu_sync, True)
+        assert num_experts is not None, '`num_experts` is required'
+        num_sms = self.get_theoretical_num_sms(num_experts, 0) if num_sms == 0 else num_sms
+
+        (recv_x, recv_sf, recv_topk_idx, recv_topk_weights, cloned_topk_idx,
+         num_recv_tokens, num_expanded_tokens, num_recv_tokens_per_expert_list,
+         psum_num_recv_tokens_per_scaleup_rank, psum_num_recv_tokens_per_expert,
+         num_unaligned_recv_tokens_per_expert, recv_src_metadata, dst_buffer_slot_idx,
+         token_metadata_at_forward, channel_linked_list, event) = self.runtime.dispatch(
+            x, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats,
+            *cached,
+            num_max_tokens_per_rank, num_experts, expert_alignment, num_sms, num_qps,
+            unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
+            async_with_compute_stream, allocate_on_comm_stream,
+            do_handle_copy, do_cpu_sync, do_expand, do_zero_padding, use_tma_aligned_col_major_sf,
+            cast_to_fp8)
+
+        if handle is None:
+            handle = EPHandle(do_expand, num_experts, expert_alignment, num_max_tokens_per_rank, num_sms,
+                              cloned_topk_idx if do_handle_copy else topk_idx,
+                              num_recv_tokens, num_expanded_tokens, num_recv_tokens_per_expert_list,
+                              psum_num_recv_tokens_per_scaleup_rank, psum_num_recv_tokens_per_expert,
+                              num_unaligned_recv_tokens_per_expert, recv_src_metadata, dst_buffer_slot_idx,
+                              token_metadata_at_forward, channel_linked_list)
+        recv_x = (recv_x, recv_sf) if recv_sf is not None else recv_x
+        return recv_x, recv_topk_idx, recv_topk_weights, handle, EventOverlap(event)
+
+    @staticmethod
+    def _unpack_bias(bias) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        bias_0, bias_1 = None, None
+        if isinstance(bias, torch.Tensor):
+            bias_0 = bias
+        elif isinstance(bias, tuple):
+            assert len(bias) == 2
+            bias_0, bias_1 = bias
+        return bias_0, bias_1
+
+    def combine(self, x: torch.Tensor, handle: EPHandle, topk_weights: Optional[torch.Tensor] = None,
+                bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]] = None,
+                num_sms: int = 0, num_qps: int = 0, previous_event: EventHandle = None,
+                previous_event_before_epilogue: Optional[EventHandle] = None,
+                async_with_compute_stream: bool = False, allocate_on_comm_stream: bool = False):
+        """Reduce received rows back to their origin tokens.
+
+        Arguments follow the reference (`deep_ep/buffers/elastic.py:1616-1626`):
+            x: BF16 `[num_recv_tokens, hidden]` (compact) or `[num_expanded_tokens, hidden]` (expanded).
+            handle: the handle `dispatch` returned.
+            topk_weights: float `[num_recv_tokens, num_topk]` (compact) or `[num_expanded_tokens]` (expanded);
+                routed back unchanged, never multiplied into `x`.
+            bias: zero, one or two BF16 `[num_tokens, hidden]` tensors added once to the output.
+
+        Returns (combined_x BF16 `[num_tokens, hidden]`, combined_topk_weights float `[num_tokens, num_topk]`
+        or None, event).  Accumulation is fp32 with one round-to-nearest-even BF16 store.
+        """
+        num_sms = handle.num_sms if num_sms == 0 else num_sms
+        bias_0, bias_1 = ElasticBuffer._unpack_bias(bias)
+        combined_x, combined_topk_weights, event = self.runtime.combine(
+            x, topk_weights, bias_0, bias_1, handle.recv_src_metadata, handle.topk_idx,
+            handle.psum_num_recv_tokens_per_scaleup_rank, handle.token_metadata_at_forward,
+            handle.channel_linked_list, handle.num_experts, handle.num_max_tokens_per_rank,
+            num_sms, num_qps, unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
+            async_with_compute_stream, allocate_on_comm_stream, handle.do_expand,
+            handle.dst_buffer_slot_idx)
+        return combined_x, combined_topk_weights, EventOverlap(event)
+
+    def check_device_status(self) -> None:
+        """Synchronise and raise if a kernel flagged bad routing input (an expert id outside
+        [0, num_experts), one expert named twice by a token) or a row that did not fit the outputs.
+        Calls with `do_cpu_sync=True` check this themselves."""
+        torch.cuda.synchronize()
+        if self.runtime._workspace is not None:
+            self.runtime._read_and_clear_status("routing")

@@ -1,0 +1,213 @@
+"""`Buffer`: the part of the V1 Python surface that sits on the routing hot path —
+`get_dispatch_layout` and the low-latency packed dispatch / combine (reference
+deep_ep/buffers/legacy.py:293-319, 553-670; host side csrc/legacy/buffer.hpp:337-404, 1463-1715).
+
+Logical ranks on one GPU.  `group.size()` = R logical ranks, `group.rank()` = this process's logical
+rank.  The packed buffers returned by `low_latency_dispatch` are those of destination rank
+`group.rank()` (experts [rank*E/R, (rank+1)*E/R)), shaped exactly as in the reference:
+`[E/R, R * num_max_dispatch_tokens_per_rank, hidden]`.  Two input forms are accepted:
+  * `x` `[T, H]`, `topk_idx` `[T, K]`: the tokens of logical source rank `group.rank()` only;
+  * `x` `[R, T, H]`, `topk_idx` `[R, T, K]` (extension): the tokens of all R logical source ranks,
+    i.e. everything destination rank `group.rank()` would receive in a real R-rank run.
+Rows of one expert are filled by source rank ascending, then token ascending.
+"""
+import ctypes
+from typing import Callable, Optional, Tuple
+
+import torch
+
+from .. import _C, _abi
+from ..platform import unwrap_event
+from ..utils.event import EventOverlap
+
+
+class Buffer:
+    num_sms: int = 20
+
+    def __init__(self, group, num_nvl_bytes: int = 0, num_rdma_bytes: int = 0, low_latency_mode: bool = False,
+                 num_qps_per_rank: int = 24, allow_nvlink_for_low_latency_mode: bool = True,
+                 allow_mnnvl: bool = False, explicitly_destroy: bool = False, enable_shrink: bool = False,
+                 comm=None) -> None:
+        self.group = group
+        self.rank = group.rank()
+        self.group_size = group.size()
+        self.num_nvl_bytes = num_nvl_bytes
+        self.num_rdma_bytes = num_rdma_bytes
+        self.low_latency_mode = low_latency_mode
+        self.explicitly_destroy = explicitly_destroy
+        self.runtime = _C.ElasticBuffer(self.rank, self.group_size, 0, [], _C.get_elastic_buffer_alignment(), 0,
+                                        False, True, True, 0, 0, 300, 100, explicitly_destroy)
+        self._ll_workspace: Optional[torch.Tensor] = None
+
+    def destroy(self) -> None:
+        assert self.explicitly_destroy, '`explicitly_destroy` flag must be set'
+        self.runtime.destroy()
+        self.runtime = None
+
+    @staticmethod
+    def capture() -> EventOverlap:
+        return EventOverlap(_C.EventHandle())
+
+    @staticmethod
+    def get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
+                                       num_experts: int) -> int:
+        """Bytes the reference would reserve (csrc/legacy/config.hpp:131-188); nothing is staged here."""
+        num_scales = hidden // 128
+        msg = 16 + max(hidden * 2, hidden + num_scales * 4)
+        combine_msg = num_scales * 4 + hidden * 2
+        send = max(num_max_dispatch_tokens_per_rank * msg, num_experts * num_max_dispatch_tokens_per_rank * combine_msg)
+        recv = num_experts * num_max_dispatch_tokens_per_rank * max(msg, combine_msg)
+        signal = num_experts * 4
+        total = 2 * (send + recv + signal)
+        return (total + 127) // 128 * 128
+
+    def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
+                            previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
+                            allocate_on_comm_stream: bool = False):
+        """Counts a dispatch needs.
+
+        Returns:
+            num_tokens_per_rank: `[num_ranks]` int32, tokens that go to each rank (once per rank).
+            num_tokens_per_rdma_rank: None (single scale-up domain).
+            num_tokens_per_expert: `[num_experts]` int32.
+            is_token_in_rank: `[num_tokens, num_ranks]` bool.
+            event: valid if `async_finish`.
+        """
+        a, b, c, d, event = self.runtime.get_dispatch_layout(topk_idx, num_experts, unwrap_event(previous_event),
+                                                             async_finish, allocate_on_comm_stream)
+        return a, b, c, d, EventOverlap(event)
+
+    def _workspace(self, num_bytes: int) -> torch.Tensor:
+        if self._ll_workspace is None or self._ll_workspace.numel() < num_bytes:
+            self._ll_workspace = torch.zeros(max(num_bytes, 4096), dtype=torch.uint8, device=self.runtime.device)
+        return self._ll_workspace
+
+    def low_latency_dispatch(self, x: torch.Tensor, topk_idx: torch.Tensor,
+                             num_max_dispatch_tokens_per_rank: int, num_experts: int,
+                             cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
+                             dispatch_wait_recv_cost_stats: Optional[torch.Tensor] = None,
+                             use_fp8: bool = True, round_scale: bool = False, use_ue8m0: bool = False,
+                             async_finish: bool = False, return_recv_hook: bool = False):
+        """Dispatch into packed per-local-expert buffers.
+
+        Returns (recv_x or (recv_x, recv_x_scales), recv_count, handle, event, hook) with
+            recv_x: `[E/R, R*M, hidden]` FP8 e4m3 (or BF16 with `use_fp8=False`); rows at or beyond
+                `recv_count[e]` are unspecified;
+            recv_x_scales: `[E/R, R*M, hidden // 128]` fp32, column-major in the last two dimensions;
+            recv_count: `[E/R]` int32;
+            handle: `(src_info [E/R, R*M] int32, layout_range [E/R, R] int64 = (begin << 32) | count,
+                      num_max_dispatch_tokens_per_rank, hidden, num_experts)`;
+            hook: None (there is no separate receive phase on one GPU).
+        FP8 scales follow the torch recipe (amax / 448 by IEEE division).
+        """
+        assert not (round_scale or use_ue8m0), 'power-of-two / UE8M0 scales are not implemented in the HIP backend'
+        assert not return_recv_hook, 'there is no separate receive phase on one GPU'
+        R, M = self.group_size, num_max_dispatch_tokens_per_rank
+        assert x.dtype == torch.bfloat16 and x.is_contiguous() and x.is_cuda
+        assert topk_idx.is_contiguous() and topk_idx.dtype == _C.topk_idx_t
+        assert num_experts % R == 0
+        if x.dim() == 3:
+            S, T, H = x.shape
+            assert S == R and tuple(topk_idx.shape[:2]) == (S, T), 'stacked input must cover all logical source ranks'
+            src_begin = 0
+        else:
+            assert x.dim() == 2 and topk_idx.dim() == 2 and x.shape[0] == topk_idx.shape[0]
+            (T, H), S, src_begin = x.shape, 1, self.rank
+        K = topk_idx.shape[-1]
+        assert T <= M and H % 16 == 0 and (not use_fp8 or H % 128 == 0)
+        assert (R * M) % 4 == 0, 'the number of rows per expert must be a multiple of 4'
+        E_l = num_experts // R
+        dev = x.device
+        rows = R * M
+
+        compute_stream, run_stream = self.runtime._prologue(None, False, async_finish)
+        with torch.cuda.stream(run_stream):
+            packed_recv_x = torch.empty((E_l, rows, H), dtype=torch.float8_e4m3fn if use_fp8 else torch.bfloat16, device=dev)
+            packed_recv_src_info = torch.empty((E_l, rows), dtype=torch.int32, device=dev)
+            # ranges of source ranks that do not send in this call stay (begin 0, count 0)
+            packed_recv_layout_range = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
+            packed_recv_count = torch.empty((E_l,), dtype=torch.int32, device=dev)
+            packed_recv_x_scales = None
+            if use_fp8:
+                packed_recv_x_scales = torch.empty((E_l, H // 128, rows), dtype=torch.float32, device=dev).transpose(1, 2)
+            if T > 0:
+                ws = self._workspace(_abi.lib.deep_ep_hip_ll_workspace_bytes(S, T, K, E_l))
+                args = _abi.LLDispatchArgs()
+                args.use_fp8 = int(use_fp8)
+                args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
+                args.num_tokens_per_src = 0
+                args.hidden, args.num_topk, args.num_experts = H, K, num_experts
+                args.expert_begin, args.num_local_experts = self.rank * E_l, E_l
+                args.num_ranks, args.num_max_dispatch_tokens_per_rank = R, M
+                args.x, args.topk_idx = _abi.ptr(x), _abi.ptr(topk_idx)
+                args.packed_recv_x = _abi.ptr(packed_recv_x)
+                args.packed_recv_x_scales = _abi.ptr(packed_recv_x_scales)
+                args.packed_recv_count = _abi.ptr(packed_recv_count)
+                args.packed_recv_src_info = _abi.ptr(packed_recv_src_info)
+                args.packed_recv_layout_range = _abi.ptr(packed_recv_layout_range)
+                args.cumulative_local_expert_recv_stats = _abi.ptr(cumulative_local_expert_recv_stats)
+                args.workspace, args.workspace_bytes = _abi.ptr(ws), ws.numel()
+                _abi.check(_abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(args), run_stream.cuda_stream),
+                           "low_latency_dispatch")
+            else:
+                packed_recv_count.zero_()
+        tensors = (x, topk_idx, packed_recv_x, packed_recv_x_scales, packed_recv_count, packed_recv_src_info,
+                   packed_recv_layout_range, cumulative_local_expert_recv_stats)
+        event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
+        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H, num_experts)
+        recv = (packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x
+        return recv, packed_recv_count, handle, EventOverlap(event, tensors if async_finish else None), None
+
+    def low_latency_combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
+                            handle: tuple, use_logfmt: bool = False, zero_copy: bool = False,
+                            async_finish: bool = False, return_recv_hook: bool = False,
+                            out: Optional[torch.Tensor] = None,
+                            combine_wait_recv_cost_stats: Optional[torch.Tensor] = None):
+        """Weighted reduce of expert outputs back to token order.
+
+        `x` is `[E/R, R*M, hidden]` BF16 laid out like the dispatched buffers; `topk_idx` / `topk_weights` are
+        those of the dispatched tokens (`[T, K]`, or `[R, T, K]` for the stacked form).  Each token sums, in lane
+        order and in fp32, `weight * row` over its lanes whose expert lives on this rank, then rounds once to
+        BF16.  Returns (combined_x, event, hook=None).
+        """
+        assert not use_logfmt, 'LogFMT is not implemented in the HIP backend'
+        assert not return_recv_hook, 'there is no separate receive phase on one GPU'
+        src_info, layout_range, M, H, num_experts = handle
+        R = self.group_size
+        E_l = num_experts // R
+        assert x.dtype == torch.bfloat16 and x.is_contiguous() and tuple(x.shape) == (E_l, R * M, H)
+        assert topk_idx.is_contiguous() and topk_idx.dtype == _C.topk_idx_t
+        assert topk_weights.is_contiguous() and topk_weights.dtype == torch.float32
+        assert topk_idx.shape == topk_weights.shape
+        if topk_idx.dim() == 3:
+            S, T, K = topk_idx.shape
+            assert S == R
+            src_begin, out_shape = 0, (S, T, H)
+        else:
+            T, K = topk_idx.shape
+            S, src_begin, out_shape = 1, self.rank, (T, H)
+        compute_stream, run_stream = self.runtime._prologue(None, False, async_finish)
+        with torch.cuda.stream(run_stream):
+            if out is None:
+                combined_x = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)
+            else:
+                assert tuple(out.shape) == out_shape and out.dtype == torch.bfloat16 and out.is_contiguous()
+                combined_x = out
+            if T > 0:
+                ws = self._workspace(4096)
+                args = _abi.LLCombineArgs()
+                args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
+                args.num_tokens_per_src = 0
+                args.hidden, args.num_topk, args.num_experts = H, K, num_experts
+                args.expert_begin, args.num_local_experts, args.num_ranks = self.rank * E_l, E_l, R
+                args.num_max_dispatch_tokens_per_rank = M
+                args.x, args.topk_idx, args.topk_weights = _abi.ptr(x), _abi.ptr(topk_idx), _abi.ptr(topk_weights)
+                args.packed_recv_src_info = _abi.ptr(src_info)
+                args.packed_recv_layout_range = _abi.ptr(layout_range)
+                args.combined_x = _abi.ptr(combined_x)
+                args.workspace, args.workspace_bytes = _abi.ptr(ws), ws.numel()
+                _abi.check(_abi.lib.deep_ep_hip_launch_ll_combine(ctypes.byref(args), run_stream.cuda_stream),
+                           "low_latency_combine")
+        tensors = (x, topk_idx, topk_weights, src_info, layout_range, combined_x)
+        event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
+        return combined_x, EventOverlap(event, tensors if async_finish else None), None

@@ -1,0 +1,239 @@
+/*
+ * C ABI of the MI355X (gfx950) MoE token-routing library: dispatch layout, dispatch
+ * (BF16 / FP8 pass-through / fused BF16->FP8 e4m3 cast), combine, and the low-latency
+ * packed per-expert layout.
+ *
+ * Conventions
+ *   - Every entry point takes a pointer to a plain-old-data argument block and the HIP stream
+ *     (hipStream_t passed as void*; NULL = the default stream).  All pointers inside an
+ *     argument block are device pointers unless a field says otherwise.  Nothing is allocated
+ *     or freed by the library; the caller owns every buffer, including the workspace.
+ *   - Return value: 0 on success, a negative DEEP_EP_HIP_ERR_* for rejected arguments, or a
+ *     positive hipError_t if a launch failed.  deep_ep_hip_last_error() returns the message of
+ *     the last failure on the calling thread.
+ *   - Launches are asynchronous on the given stream.  Calls that share one workspace must be
+ *     ordered on one stream (the workspace is not re-entrant), mirroring the reference's
+ *     "one workspace per buffer" rule (csrc/elastic/buffer.hpp:118-121).
+ *   - num_ranks is a logical bucketing parameter: destination rank d owns experts
+ *     [d*E/R, (d+1)*E/R).  All destination buckets live in the caller's own HBM.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   deep_ep_hip_launch_layout       csrc/kernels/legacy/layout.cu:124-150 (get_dispatch_layout)
+ *   deep_ep_hip_launch_dispatch     csrc/kernels/elastic/dispatch.hpp:141,293 (launch_dispatch +
+ *                                   launch_dispatch_copy_epilogue), ABI style of
+ *                                   csrc/backends/ascend/elastic/kernels.hpp:274-288
+ *   deep_ep_hip_launch_combine      csrc/kernels/elastic/combine.hpp:114,248 (launch_combine +
+ *                                   launch_combine_reduce_epilogue)
+ *   deep_ep_hip_launch_ll_dispatch  csrc/kernels/legacy/internode_ll.cu:464-554
+ *   deep_ep_hip_launch_ll_combine   csrc/kernels/legacy/internode_ll.cu:1140-1238
+ *   deep_ep_hip_launch_cast_fp8     deep_ep/utils/math.py:30-39 (per_token_cast_to_fp8)
+ */
+#ifndef DEEP_EP_HIP_H_
+#define DEEP_EP_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DEEP_EP_HIP_ABI_VERSION 1
+
+#define DEEP_EP_HIP_OK 0
+#define DEEP_EP_HIP_ERR_INVALID_ARGUMENT (-1)
+#define DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL (-2)
+#define DEEP_EP_HIP_ERR_UNSUPPORTED (-3)
+
+/* Limits checked by every entry point. */
+#define DEEP_EP_HIP_MAX_TOPK 32
+#define DEEP_EP_HIP_MAX_EXPERTS 1024
+#define DEEP_EP_HIP_MAX_RANKS 512
+
+/* Bits of the device-side status word (first int32 of the workspace, see
+ * deep_ep_hip_workspace_status_offset).  Kernels OR bits in; they never trap. */
+#define DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE 1  /* topk_idx >= num_experts (entry ignored) */
+#define DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT 2     /* one token names an expert twice */
+#define DEEP_EP_HIP_STATUS_ROW_OVERFLOW 4         /* a row fell outside the caller's capacity (row dropped) */
+
+int deep_ep_hip_abi_version(void);
+const char* deep_ep_hip_last_error(void);
+
+/* Bytes of workspace needed for dispatches of up to num_max_tokens tokens.  The workspace must
+ * be zero-filled once before its first use; the kernels leave it ready for the next call. */
+size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_experts, int num_ranks);
+/* Byte offset, inside the workspace, of the int32 status word. */
+size_t deep_ep_hip_workspace_status_offset(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Dispatch layout (V1 `Buffer.get_dispatch_layout`): counts only.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    const int64_t* topk_idx;        /* [num_tokens, num_topk], -1 = no selection */
+    int32_t num_tokens, num_topk, num_experts, num_ranks;
+    int32_t* num_tokens_per_rank;   /* [num_ranks] out */
+    int32_t* num_tokens_per_expert; /* [num_experts] out */
+    uint8_t* is_token_in_rank;      /* [num_tokens, num_ranks] out (bool), may be NULL */
+    void* workspace;
+    uint64_t workspace_bytes;
+} deep_ep_hip_layout_args;
+
+int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dispatch (V2 `ElasticBuffer.dispatch`), one logical source rank.
+ *
+ * phases: bit 0 = count/scan (fills the handle tensors psum_*, num_unaligned, host_counts and
+ * the per-(token,lane) positions kept in the workspace); bit 1 = move payload and metadata.
+ * A caller that needs exact output sizes runs phase 1, waits for host_counts, allocates, then
+ * runs phase 2; otherwise both phases go in one call.  With cached != 0 only phase 2 is legal
+ * and dst_buffer_slot_idx / psum_rank / recv_src_metadata are inputs.
+ * ---------------------------------------------------------------------------------------- */
+#define DEEP_EP_HIP_PHASE_LAYOUT 1
+#define DEEP_EP_HIP_PHASE_MOVE 2
+
+#define DEEP_EP_HIP_PAYLOAD_BF16 0      /* x bf16 -> recv_x bf16 */
+#define DEEP_EP_HIP_PAYLOAD_FP8 1       /* x e4m3 + sf -> recv_x e4m3 + recv_sf (pass-through) */
+#define DEEP_EP_HIP_PAYLOAD_CAST_FP8 2  /* x bf16 -> recv_x e4m3 + recv_sf fp32 (fused cast) */
+
+typedef struct {
+    int32_t phases;
+    int32_t payload;                /* DEEP_EP_HIP_PAYLOAD_* */
+    int32_t cached;                 /* reuse handle tensors instead of recomputing the layout */
+    int32_t do_expand;              /* expert-major layout, one row per (token, lane) */
+    int32_t do_zero_padding;        /* zero alignment padding rows (expanded layout only) */
+    int32_t num_tokens, hidden, num_topk, num_experts, num_ranks;
+    int32_t rank_idx;               /* logical source rank of these tokens */
+    int32_t num_max_tokens_per_rank;
+    int32_t expert_alignment;
+
+    /* inputs */
+    const void* x;                  /* [num_tokens, hidden] bf16 or e4m3, contiguous */
+    const void* sf;                 /* payload FP8: [num_tokens, num_sf_packs] 4-byte packs */
+    int64_t sf_token_stride, sf_hidden_stride;   /* in 4-byte elements */
+    int32_t num_sf_packs;           /* payload FP8: packs per token; CAST_FP8: must be ceil(hidden/128) */
+    const int64_t* topk_idx;        /* [num_tokens, num_topk] */
+    const float* topk_weights;      /* [num_tokens, num_topk] or NULL */
+
+    /* handle tensors: outputs of phase 1 (inputs when cached) */
+    int64_t* copied_topk_idx;       /* [num_tokens, num_topk] or NULL */
+    int32_t* psum_num_recv_tokens_per_rank;     /* [num_ranks] inclusive */
+    int32_t* psum_num_recv_tokens_per_expert;   /* [num_experts] */
+    int32_t* num_unaligned_recv_tokens_per_expert; /* [num_experts] */
+    int32_t* cumulative_local_expert_recv_stats;   /* [num_experts] += actual counts, or NULL */
+    int32_t* host_counts;           /* host-mapped [num_ranks + num_experts] or NULL: per-rank counts
+                                       then aligned per-expert counts, value v published as -v-1 */
+    int32_t* dst_buffer_slot_idx;   /* [num_tokens, num_topk]: written by phase 2 (input when cached) */
+    int32_t* recv_src_metadata;     /* [recv_capacity, num_topk + 2]: written by phase 2 (input when cached) */
+
+    /* outputs of phase 2 */
+    void* recv_x;                   /* [recv_capacity or expanded_capacity, hidden] */
+    void* recv_sf;                  /* 4-byte packs, strides below; NULL for BF16 */
+    int64_t recv_sf_token_stride, recv_sf_hidden_stride;
+    int64_t* recv_topk_idx;         /* [recv_capacity, num_topk], compact layout only */
+    float* recv_topk_weights;       /* [recv_capacity, num_topk] or [expanded_capacity]; NULL if no weights */
+    int64_t recv_capacity;          /* rows the compact-indexed outputs can hold */
+    int64_t expanded_capacity;      /* rows the expanded outputs can hold (do_expand) */
+
+    void* workspace;
+    uint64_t workspace_bytes;
+} deep_ep_hip_dispatch_args;
+
+int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Combine (V2 `ElasticBuffer.combine`): per origin token, fp32 sum of bias_0, bias_1 and the
+ * rows that came back, in ascending master-lane order, one round-to-nearest-even BF16 store.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    int32_t do_expand;
+    int32_t allow_multiple_reduction;   /* expanded layout: first reduce each rank's rows to bf16 */
+    int32_t num_tokens, hidden, num_topk, num_experts, num_ranks;
+    int32_t rank_idx, num_max_tokens_per_rank;
+    const void* x;                      /* bf16 [num_x_rows, hidden] */
+    int64_t num_x_rows;
+    const float* topk_weights;          /* [num_recv, num_topk] or [num_expanded] or NULL */
+    const void* bias_0;                 /* bf16 [num_tokens, hidden] or NULL */
+    const void* bias_1;
+    const int64_t* topk_idx;            /* handle: [num_tokens, num_topk] */
+    const int32_t* dst_buffer_slot_idx; /* handle: [num_tokens, num_topk] */
+    const int32_t* recv_src_metadata;   /* handle: [num_recv, num_topk + 2] (expanded layout) */
+    const int32_t* psum_num_recv_tokens_per_rank; /* handle: [num_ranks] */
+    void* combined_x;                   /* bf16 [num_tokens, hidden] out */
+    float* combined_topk_weights;       /* [num_tokens, num_topk] out or NULL */
+    void* workspace;
+    uint64_t workspace_bytes;
+} deep_ep_hip_combine_args;
+
+int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Low-latency packed layout (V1 `Buffer.low_latency_dispatch/combine`) for one logical
+ * destination rank holding experts [expert_begin, expert_begin + num_local_experts).
+ * Source ranks src_rank_begin .. src_rank_begin + num_src_ranks - 1 send in one launch; the
+ * tokens of the i-th source are rows [i*src_token_stride, i*src_token_stride + n_i) of x.
+ * Fill order inside an expert buffer: source rank ascending, then token ascending.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    int32_t use_fp8;                    /* 1: e4m3 payload + fp32 scales; 0: bf16 payload */
+    int32_t num_src_ranks, src_rank_begin;
+    int32_t src_token_stride;           /* rows of x reserved per source rank */
+    const int32_t* num_tokens_per_src;  /* [num_src_ranks] device, or NULL = src_token_stride each */
+    int32_t hidden, num_topk, num_experts;
+    int32_t expert_begin, num_local_experts;
+    int32_t num_ranks;                  /* columns of packed_recv_layout_range */
+    int32_t num_max_dispatch_tokens_per_rank;   /* slots per (expert, source rank) budget; rows per
+                                                   expert buffer = num_ranks * this */
+    const void* x;                      /* bf16 [num_src_ranks * src_token_stride, hidden] */
+    const int64_t* topk_idx;            /* [num_src_ranks * src_token_stride, num_topk] */
+    void* packed_recv_x;                /* [num_local_experts, rows, hidden] */
+    float* packed_recv_x_scales;        /* fp8: element (e, row, g) at e*rows*G + g*rows + row */
+    int32_t* packed_recv_count;         /* [num_local_experts] out */
+    int32_t* packed_recv_src_info;      /* [num_local_experts, rows] out */
+    int64_t* packed_recv_layout_range;  /* [num_local_experts, num_ranks] out: (begin<<32)|count */
+    int32_t* cumulative_local_expert_recv_stats; /* [num_local_experts] += counts, or NULL */
+    void* workspace;
+    uint64_t workspace_bytes;
+} deep_ep_hip_ll_dispatch_args;
+
+/* Bytes of (zero-initialised, reusable) workspace a low-latency dispatch of this shape needs. */
+size_t deep_ep_hip_ll_workspace_bytes(int num_src_ranks, int src_token_stride, int num_topk, int num_local_experts);
+int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* args, void* stream);
+
+typedef struct {
+    int32_t num_src_ranks, src_rank_begin;  /* source ranks whose tokens are rebuilt in this launch */
+    int32_t src_token_stride;           /* rows of topk_idx / topk_weights / combined_x per source rank */
+    const int32_t* num_tokens_per_src;  /* [num_src_ranks] device, or NULL = src_token_stride each */
+    int32_t hidden, num_topk, num_experts;
+    int32_t expert_begin, num_local_experts, num_ranks;
+    int32_t num_max_dispatch_tokens_per_rank;
+    const void* x;                      /* bf16 [num_local_experts, rows, hidden] */
+    const int64_t* topk_idx;            /* [num_src_ranks * src_token_stride, num_topk] */
+    const float* topk_weights;          /* [num_src_ranks * src_token_stride, num_topk] */
+    const int32_t* packed_recv_src_info;
+    const int64_t* packed_recv_layout_range;
+    void* combined_x;                   /* bf16 [num_src_ranks * src_token_stride, hidden] out; rows past a
+                                           source's token count are left untouched */
+    void* workspace;
+    uint64_t workspace_bytes;
+} deep_ep_hip_ll_combine_args;
+
+int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Stand-alone per-token 1x128 FP8 cast: bf16 [num_tokens, hidden] -> e4m3 + fp32 scales
+ * (row-major [num_tokens, ceil(hidden/128)]).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    const void* x;
+    void* out;
+    float* scales;
+    int32_t num_tokens, hidden;
+} deep_ep_hip_cast_args;
+
+int deep_ep_hip_launch_cast_fp8(const deep_ep_hip_cast_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEP_EP_HIP_H_ */

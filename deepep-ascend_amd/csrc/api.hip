@@ -257,6 +257,7 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
     REQUIRE(!any || a->combined_x != nullptr, "combined_x is NULL");
     REQUIRE(!any || a->x != nullptr || a->num_x_rows == 0, "x is NULL");
     REQUIRE(!(a->do_expand && any && a->recv_src_metadata == nullptr), "the expanded layout needs recv_src_metadata");
+    REQUIRE(a->num_recv_rows >= 0, "num_recv_rows must be >= 0");
     REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
     CombineParams p{};
     p.x = static_cast<const uint8_t*>(a->x);
@@ -267,6 +268,7 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
     p.topk_idx = a->topk_idx;
     p.slot = a->dst_buffer_slot_idx;
     p.meta = a->recv_src_metadata;
+    p.num_meta_rows = a->num_recv_rows;
     p.psum_rank = a->psum_num_recv_tokens_per_rank;
     p.out = static_cast<uint8_t*>(a->combined_x);
     p.out_w = a->combined_topk_weights;

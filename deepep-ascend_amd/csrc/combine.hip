@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
         const int rj = read_lane(row_c, j);
         if (d >= 0 && dj == d && rj >= 0) my_row = rj;
     }
-    if (p.do_expand && my_row >= 0) {
+    if (p.do_expand && my_row >= 0 && my_row < p.num_meta_rows) {
         erow = p.meta[int64_t(my_row) * (p.K + 2) + 2 + lane];
         if (erow >= p.num_x_rows) {
             atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);

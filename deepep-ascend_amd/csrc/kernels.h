@@ -103,6 +103,7 @@ struct CombineParams {
     const int64_t* topk_idx;
     const int32_t* slot;
     const int32_t* meta;
+    int64_t num_meta_rows;
     const int32_t* psum_rank;
     uint8_t* out;
     float* out_w;

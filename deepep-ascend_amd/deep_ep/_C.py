@@ -474,6 +474,7 @@ class ElasticBuffer:
             args.topk_idx = _abi.ptr(combined_topk_idx)
             args.dst_buffer_slot_idx = _abi.ptr(dst_buffer_slot_idx)
             args.recv_src_metadata = _abi.ptr(src_metadata)
+            args.num_recv_rows = src_metadata.shape[0]
             args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_num_recv_tokens_per_scaleup_rank)
             args.combined_x = _abi.ptr(combined_x)
             args.combined_topk_weights = _abi.ptr(combined_topk_weights)

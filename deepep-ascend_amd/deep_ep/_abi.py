@@ -84,6 +84,7 @@ class CombineArgs(Structure):
         ("topk_idx", c_void_p),
         ("dst_buffer_slot_idx", c_void_p),
         ("recv_src_metadata", c_void_p),
+        ("num_recv_rows", c_int64),
         ("psum_num_recv_tokens_per_rank", c_void_p),
         ("combined_x", c_void_p),
         ("combined_topk_weights", c_void_p),

@@ -157,7 +157,8 @@ typedef struct {
     const void* bias_1;
     const int64_t* topk_idx;            /* handle: [num_tokens, num_topk] */
     const int32_t* dst_buffer_slot_idx; /* handle: [num_tokens, num_topk] */
-    const int32_t* recv_src_metadata;   /* handle: [num_recv, num_topk + 2] (expanded layout) */
+    const int32_t* recv_src_metadata;   /* handle: [num_recv_rows, num_topk + 2] (expanded layout) */
+    int64_t num_recv_rows;              /* rows of recv_src_metadata */
     const int32_t* psum_num_recv_tokens_per_rank; /* handle: [num_ranks] */
     void* combined_x;                   /* bf16 [num_tokens, hidden] out */
     float* combined_topk_weights;       /* [num_tokens, num_topk] out or NULL */

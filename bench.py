@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE token-routing hot path on one MI355X.
+
+One step = one pass of the hot path over one batch of synthetic tokens: dispatch (layout + fused
+BF16->FP8 e4m3 cast + scatter into the rank-major receive buffer) followed by combine (gather +
+fp32 reduce + BF16 store) at T=8192, H=7168, top-8 of 256 experts, 8 logical ranks, uniform-random
+routing.  Inputs are resident in HBM before the timed region; outputs are pre-sized for the worst
+case so no host synchronisation sits inside a step.  Calls go straight through the C ABI.
+
+Prints one JSON line: whole-step achieved HBM GB/s (algorithmic bytes / time), per-op us/call,
+a roofline object for the dominant kernel (combine) and a CPU baseline (the torch-CPU oracle timed
+on a bounded sample of the same workload).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "deepep-ascend_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=True, expanded=False):
+    """Bytes a perfect implementation must move (each payload byte read once, written once)."""
+    s_in = T * H * 2
+    b_row = H * (1 if fp8 else 2) + ((H // 128) * 4 if fp8 else 0)
+    meta = K * 8 + K * 4 + (K + 2) * 4
+    layout = T * K * 8 + T * R + (R + E) * 4
+    if expanded:
+        dispatch = s_in + T * K * 12 + N_e * (b_row + 4) + N_r * (K + 2) * 4
+    else:
+        dispatch = s_in + T * K * 12 + N_r * (b_row + meta)
+    n_in = N_e if expanded else N_r
+    combine = n_in * H * 2 + T * K * 8 + T * H * 2
+    return {"layout": layout, "dispatch": dispatch, "combine": combine}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4"])
+    ap.add_argument("--expanded", action="store_true", help="expert-major (expanded) receive layout")
+    ap.add_argument("--bf16", action="store_true", help="BF16 dispatch instead of the fused FP8 cast")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--l2-flush", action="store_true", help="zero a 256 MB buffer between per-kernel timings")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (logical ranks share its HBM); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import routing_cases as rc
+    from deep_ep import _abi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    case = {"C2": rc.c2, "C3": rc.c3, "C4": rc.c4}[args.workload]()
+    T, H, K, E, R, M = case.T, case.H, case.K, case.E, case.R, case.M
+    fp8 = not args.bf16
+    expanded = args.expanded
+    x, idx, w = case.x.to(dev), case.topk_idx.to(dev), case.topk_weights.to(dev)
+
+    # realised routing statistics (for the algorithmic bytes)
+    valid = case.topk_idx >= 0
+    N_e = int(valid.sum())
+    dst = torch.where(valid, case.topk_idx // (E // R), torch.full_like(case.topk_idx, -1))
+    N_r = int(sum(int((dst == r).any(dim=1).sum()) for r in range(R)))
+    ab = algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=fp8, expanded=expanded)
+
+    # ---- buffers (worst-case sized, allocated once) ----
+    i32 = dict(dtype=torch.int32, device=dev)
+    cap = M * R
+    ecap = M * min(K, E)
+    rows = ecap if expanded else cap
+    ws_bytes = _abi.lib.deep_ep_hip_workspace_bytes(T, K, E, R)
+    workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    psum_rank, psum_expert, unaligned = torch.empty(R, **i32), torch.empty(E, **i32), torch.empty(E, **i32)
+    slot = torch.empty((T, K), **i32)
+    meta = torch.empty((cap, K + 2), **i32)
+    recv_x = torch.empty((rows, H), dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16, device=dev)
+    recv_sf = torch.empty((rows, H // 128), dtype=torch.float32, device=dev) if fp8 else None
+    recv_idx = torch.empty((cap, K), dtype=torch.int64, device=dev) if not expanded else None
+    recv_w = torch.empty((rows,) if expanded else (cap, K), dtype=torch.float32, device=dev)
+    y = torch.randn((rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)   # "expert outputs"
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    out_w = torch.empty((T, K), dtype=torch.float32, device=dev)
+
+    d = _abi.DispatchArgs()
+    d.payload = _abi.PAYLOAD_CAST_FP8 if fp8 else _abi.PAYLOAD_BF16
+    d.do_expand = int(expanded)
+    d.num_tokens, d.hidden, d.num_topk, d.num_experts, d.num_ranks = T, H, K, E, R
+    d.rank_idx, d.num_max_tokens_per_rank, d.expert_alignment = 0, M, 1
+    d.x, d.topk_idx, d.topk_weights = x.data_ptr(), idx.data_ptr(), w.data_ptr()
+    d.num_sf_packs = H // 128 if fp8 else 0
+    d.psum_num_recv_tokens_per_rank = psum_rank.data_ptr()
+    d.psum_num_recv_tokens_per_expert = psum_expert.data_ptr()
+    d.num_unaligned_recv_tokens_per_expert = unaligned.data_ptr()
+    d.dst_buffer_slot_idx, d.recv_src_metadata = slot.data_ptr(), meta.data_ptr()
+    d.recv_x = recv_x.data_ptr()
+    d.recv_sf = recv_sf.data_ptr() if fp8 else 0
+    d.recv_sf_token_stride, d.recv_sf_hidden_stride = (H // 128, 1) if fp8 else (0, 0)
+    d.recv_topk_idx = recv_idx.data_ptr() if recv_idx is not None else 0
+    d.recv_topk_weights = recv_w.data_ptr()
+    d.recv_capacity, d.expanded_capacity = cap, (ecap if expanded else 0)
+    d.workspace, d.workspace_bytes = workspace.data_ptr(), ws_bytes
+
+    c = _abi.CombineArgs()
+    c.do_expand, c.allow_multiple_reduction = int(expanded), 1
+    c.num_tokens, c.hidden, c.num_topk, c.num_experts, c.num_ranks = T, H, K, E, R
+    c.rank_idx, c.num_max_tokens_per_rank = 0, M
+    c.x, c.num_x_rows = y.data_ptr(), rows
+    c.topk_weights = recv_w.data_ptr()
+    c.topk_idx, c.dst_buffer_slot_idx = idx.data_ptr(), slot.data_ptr()
+    c.recv_src_metadata, c.num_recv_rows = meta.data_ptr(), cap
+    c.psum_num_recv_tokens_per_rank = psum_rank.data_ptr()
+    c.combined_x, c.combined_topk_weights = out.data_ptr(), out_w.data_ptr()
+    c.workspace, c.workspace_bytes = workspace.data_ptr(), ws_bytes
+
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    lib = _abi.lib
+
+    def dispatch(phases):
+        d.phases = phases
+        _abi.check(lib.deep_ep_hip_launch_dispatch(ctypes.byref(d), sp), "dispatch")
+
+    def combine():
+        _abi.check(lib.deep_ep_hip_launch_combine(ctypes.byref(c), sp), "combine")
+
+    def step():
+        dispatch(_abi.PHASE_LAYOUT | _abi.PHASE_MOVE)
+        combine()
+
+    flush_buf = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev) if args.l2_flush else None
+
+    def timed(fn, iters, flush=False):
+        """Average duration in us of fn over iters launches, by HIP events on the launch stream."""
+        if flush:
+            total = 0.0
+            for _ in range(iters):
+                flush_buf.zero_()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream); fn(); e1.record(stream)
+                e1.synchronize()
+                total += e0.elapsed_time(e1)
+            return total * 1e3 / iters
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(iters):
+            fn()
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    status = int(workspace[:4].view(torch.int32).item())
+    if status != 0:
+        print(f"bench.py: device status {status} after warm-up (bad routing input or overflow)", file=sys.stderr)
+        sys.exit(1)
+
+    # ---- the timed region: exactly `steps` steps ----
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step_us = timed(step, args.steps)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+
+    # ---- per-kernel durations (same launches, one kind at a time) ----
+    k = max(args.steps, 10)
+    layout_us = timed(lambda: dispatch(_abi.PHASE_LAYOUT), k, args.l2_flush)
+    move_us = timed(lambda: dispatch(_abi.PHASE_MOVE), k, args.l2_flush)
+    dispatch_us = timed(lambda: dispatch(_abi.PHASE_LAYOUT | _abi.PHASE_MOVE), k, args.l2_flush)
+    combine_us = timed(combine, k, args.l2_flush)
+
+    def gbs(nbytes, us):
+        return nbytes / us * 1e-3
+
+    step_bytes = ab["layout"] + ab["dispatch"] + ab["combine"]
+    result = {
+        "metric": "dispatch+combine achieved HBM GB/s (algorithmic bytes / step time), 8192x7168 top-8 of 256, 8 logical ranks",
+        "value": round(gbs(step_bytes, step_us), 1),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_us * 1e-3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 dispatch (bf16 in) / bf16 combine (fp32 accumulate)" if fp8 else "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{case.name}: T={T} H={H} E={E} R={R} K={K} "
+                               f"{'expanded' if expanded else 'compact'} layout, N_r={N_r}, N_e={N_e}",
+                   "l2_flush": bool(args.l2_flush)},
+        "us_per_call": {"dispatch": round(dispatch_us, 2), "dispatch_layout": round(layout_us, 2),
+                        "dispatch_move": round(move_us, 2), "combine": round(combine_us, 2)},
+        "achieved_gbs": {"dispatch": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us), 1),
+                         "dispatch_move": round(gbs(ab["dispatch"], move_us), 1),
+                         "combine": round(gbs(ab["combine"], combine_us), 1)},
+        "frac_of_peak": {"dispatch": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us) / HBM_PEAK_GBS, 4),
+                         "combine": round(gbs(ab["combine"], combine_us) / HBM_PEAK_GBS, 4)},
+        "algorithmic_bytes": ab,
+        "roofline": {"kernel": "combine_kernel", "bound": "hbm",
+                     "achieved": round(gbs(ab["combine"], combine_us), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs(ab["combine"], combine_us) / HBM_PEAK_GBS, 4), "traffic": None},
+        "roofline_dispatch": {"kernel": "dispatch_cast_kernel" if fp8 else "dispatch_copy_kernel", "bound": "hbm",
+                              "achieved": round(gbs(ab["dispatch"], move_us), 1), "peak": HBM_PEAK_GBS,
+                              "unit": "GB/s", "frac": round(gbs(ab["dispatch"], move_us) / HBM_PEAK_GBS, 4),
+                              "traffic": None},
+        "wall_ms_timed_region": round(wall_ms, 3),
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens, fp8, expanded)
+    print(json.dumps(result))
+
+
+def cpu_baseline(case, sample_tokens, fp8, expanded):
+    """The torch-CPU oracle (the reference path restated) timed on the first `sample_tokens` tokens of
+    the same workload: layout + (FP8 cast +) dispatch + combine, all host cores."""
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import routing_oracle as oracle
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    n = min(sample_tokens, case.T)
+    x, idx, w = case.x[:n].contiguous(), case.topk_idx[:n].contiguous(), case.topk_weights[:n].contiguous()
+    T, H, K, E, R = n, case.H, case.K, case.E, case.R
+
+    def one_pass():
+        oracle.layout(idx, E, R)
+        payload = oracle.per_token_cast_to_fp8(x) if fp8 else x
+        r = oracle.dispatch(payload, idx, w, E, R, 0, n, do_expand=expanded)
+        rows = r.recv_x[0].shape[0] if isinstance(r.recv_x, tuple) else r.recv_x.shape[0]
+        y = torch.zeros((rows, H), dtype=torch.bfloat16)
+        oracle.combine(y, idx, r.recv_src_metadata, r.dst_buffer_slot_idx, r.psum_num_recv_tokens_per_scaleup_rank,
+                       E, R, 0, n, topk_weights=r.recv_topk_weights, do_expand=expanded)
+        return r
+
+    r = one_pass()   # warm-up
+    iters, t0 = 0, time.perf_counter()
+    while True:
+        one_pass()
+        iters += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed > 10.0 or iters >= 5:
+            break
+    per_pass = elapsed / iters
+    valid = idx >= 0
+    N_e = int(valid.sum())
+    N_r = r.num_recv_tokens
+    ab = algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=fp8, expanded=expanded)
+    total = ab["layout"] + ab["dispatch"] + ab["combine"]
+    return {"value": round(total / per_pass * 1e-9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"first {n} of {case.T} tokens of the same workload, 1 warm-up + {iters} timed passes of "
+                      f"layout+dispatch+combine (torch CPU, eager), {per_pass * 1e3:.1f} ms/pass",
+            "ms_per_pass": round(per_pass * 1e3, 2)}
+
+
+if __name__ == "__main__":
+    main()

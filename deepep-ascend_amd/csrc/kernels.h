@@ -28,6 +28,7 @@ struct LayoutParams {
     int T, K, E, R, E_l;
     int A;            // expert alignment
     int do_expand;
+    int slab_rows;    // chunk rows staged in LDS per pass of the final scan (set by the launcher)
     int32_t* num_tokens_per_rank;    // optional
     int32_t* num_tokens_per_expert;  // optional
     uint8_t* is_token_in_rank;       // optional

@@ -58,24 +58,30 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     for (int i = tid; i < n * kWaves; i += kThreads) bitmap[i] = 0ull;
     __syncthreads();
 
+    // All index loads are issued before anything that could alias them is stored.
+    int64_t raw[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) raw[k] = (active && k < p.K) ? p.topk_idx[int64_t(t) * p.K + k] : int64_t(-1);
+
     int e[KMAX], d[KMAX];
     int flags = 0;
     const uint64_t my_bit = 1ull << lane;
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
         int ev = -1;
-        if (active && k < p.K) {
-            const int64_t raw = p.topk_idx[int64_t(t) * p.K + k];
-            if (p.copied_topk_idx != nullptr) p.copied_topk_idx[int64_t(t) * p.K + k] = raw;
-            if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
-            else if (raw >= 0) ev = int(raw);
-        }
+        if (raw[k] >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+        else if (raw[k] >= 0) ev = int(raw[k]);
         e[k] = ev;
         d[k] = ev >= 0 ? ev / p.E_l : -1;
         if (ev >= 0) {
             atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[(p.R + ev) * kWaves + wave]), my_bit);
             atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[d[k] * kWaves + wave]), my_bit);
         }
+    }
+    if (p.copied_topk_idx != nullptr && active) {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+            if (k < p.K) p.copied_topk_idx[int64_t(t) * p.K + k] = raw[k];
     }
     __syncthreads();
 
@@ -132,19 +138,31 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     __threadfence();
 
     // ---- last workgroup: chunk bases and public prefix sums ----
-    int* totals = reinterpret_cast<int*>(bitmap);          // [n]
+    // LDS is re-carved as int arrays: a staging slab of chunk rows, then totals / aligned / scanned.
+    int* stage = reinterpret_cast<int*>(bitmap);           // [slab_rows][n]
+    int* totals = stage + size_t(p.slab_rows) * n;         // [n]
     int* aligned = totals + n;                             // [E] then scanned in place
     const int num_chunks = gridDim.x;
-    for (int j = tid; j < n; j += kThreads) {
-        int running = 0;
-        for (int c = 0; c < num_chunks; ++c) {
-            const int v = load_agent(&p.chunk_counts[int64_t(c) * n + j]);
-            p.chunk_base[int64_t(c) * n + j] = running;
-            running += v;
+    for (int j = tid; j < n; j += kThreads) totals[j] = 0;
+    for (int c0 = 0; c0 < num_chunks; c0 += p.slab_rows) {
+        const int rows = min(p.slab_rows, num_chunks - c0);
+        const int32_t* src = p.chunk_counts + int64_t(c0) * n;
+        for (int i = tid; i < rows * n; i += kThreads) stage[i] = src[i];       // coalesced, independent loads
+        __syncthreads();
+        for (int j = tid; j < n; j += kThreads) {                               // one column per thread
+            int running = totals[j];
+            for (int r = 0; r < rows; ++r) {
+                const int v = stage[r * n + j];
+                stage[r * n + j] = running;
+                running += v;
+            }
+            totals[j] = running;
         }
-        totals[j] = running;
+        __syncthreads();
+        int32_t* dstb = p.chunk_base + int64_t(c0) * n;
+        for (int i = tid; i < rows * n; i += kThreads) dstb[i] = stage[i];
+        __syncthreads();
     }
-    __syncthreads();
 
     for (int j = tid; j < p.E; j += kThreads) {
         const int cnt = totals[p.R + j];
@@ -188,15 +206,23 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
 hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream) {
     const int num_chunks = p.T > 0 ? (p.T + kThreads - 1) / kThreads : 1;
     const int n = p.R + p.E;
-    // bitmap words, reused by the last workgroup as 3 int arrays of at most n entries
-    const size_t lds = size_t(n) * kWaves * sizeof(uint64_t);
+    // LDS holds the bitmap words [n][kWaves] first; the last workgroup re-carves it as a staging slab of
+    // chunk rows plus three int arrays of at most n entries.
+    const size_t bitmap_bytes = size_t(n) * kWaves * sizeof(uint64_t);
+    const size_t budget = 60 * 1024;
+    int slab_rows = int((budget - 3 * size_t(n) * 4) / (size_t(n) * 4));
+    slab_rows = slab_rows < 1 ? 1 : (slab_rows > num_chunks ? num_chunks : slab_rows);
+    const size_t scan_bytes = (size_t(slab_rows) + 3) * n * 4;
+    const size_t lds = bitmap_bytes > scan_bytes ? bitmap_bytes : scan_bytes;
+    LayoutParams q = p;
+    q.slab_rows = slab_rows;
     dim3 grid(num_chunks), block(kThreads);
     if (p.K <= 8) {
-        hipLaunchKernelGGL(layout_kernel<8>, grid, block, lds, stream, p);
+        hipLaunchKernelGGL(layout_kernel<8>, grid, block, lds, stream, q);
     } else if (p.K <= 16) {
-        hipLaunchKernelGGL(layout_kernel<16>, grid, block, lds, stream, p);
+        hipLaunchKernelGGL(layout_kernel<16>, grid, block, lds, stream, q);
     } else {
-        hipLaunchKernelGGL(layout_kernel<32>, grid, block, lds, stream, p);
+        hipLaunchKernelGGL(layout_kernel<32>, grid, block, lds, stream, q);
     }
     return hipGetLastError();
 }

@@ -40,16 +40,17 @@ __global__ __launch_bounds__(kThreads) void ll_count_kernel(const LLDispatchPara
     for (int i = tid; i < p.E_l * kWaves; i += kThreads) bitmap[i] = 0ull;
     __syncthreads();
 
+    int64_t raw[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) raw[k] = (active && k < p.K) ? p.topk_idx[g * p.K + k] : int64_t(-1);
+
     int le[KMAX];
     int flags = 0;
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
         le[k] = -1;
-        if (active && k < p.K) {
-            const int64_t raw = p.topk_idx[g * p.K + k];
-            if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
-            else if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l) le[k] = int(raw) - p.expert_begin;
-        }
+        if (raw[k] >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+        else if (raw[k] >= p.expert_begin && raw[k] < p.expert_begin + p.E_l) le[k] = int(raw[k]) - p.expert_begin;
         if (le[k] >= 0)
             atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[le[k] * kWaves + wave]), 1ull << lane);
     }
@@ -90,18 +91,28 @@ __global__ __launch_bounds__(kThreads) void ll_count_kernel(const LLDispatchPara
     if (!is_last) return;
     __threadfence();
 
+    // Exclusive prefix over (source rank, chunk) per local expert.  Loads go in batches of 16 that are
+    // all issued before the batch's stores, so a decode-sized call needs a single memory round trip.
+    const int num_blocks = p.S * chunks_per_src;
     for (int j = tid; j < p.E_l; j += kThreads) {
-        int running = 0;
-        for (int src = 0; src < p.S; ++src) {
-            const int begin = running;
-            for (int cc = 0; cc < chunks_per_src; ++cc) {
-                const int64_t b = int64_t(src) * chunks_per_src + cc;
-                const int v = load_agent(&p.chunk_counts[b * p.E_l + j]);
-                p.chunk_base[b * p.E_l + j] = running;
-                running += v;
+        int running = 0, begin = 0;
+        for (int b0 = 0; b0 < num_blocks; b0 += 16) {
+            int v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                v[i] = (b0 + i < num_blocks) ? p.chunk_counts[int64_t(b0 + i) * p.E_l + j] : 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int b = b0 + i;
+                if (b < num_blocks) {
+                    if (b % chunks_per_src == 0) begin = running;
+                    p.chunk_base[int64_t(b) * p.E_l + j] = running;
+                    running += v[i];
+                    if (b % chunks_per_src == chunks_per_src - 1)
+                        p.packed_layout_range[int64_t(j) * p.R + p.src_rank_begin + b / chunks_per_src] =
+                            (int64_t(begin) << 32) | int64_t(running - begin);
+                }
             }
-            p.packed_layout_range[int64_t(j) * p.R + p.src_rank_begin + src] =
-                (int64_t(begin) << 32) | int64_t(running - begin);
         }
         p.packed_count[j] = running;
         if (p.cumulative_stats != nullptr) p.cumulative_stats[j] += running;

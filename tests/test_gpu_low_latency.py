@@ -1,0 +1,70 @@
+"""GPU parity of the low-latency packed layout against the CPU oracle, through the Buffer API."""
+import pytest
+import torch
+
+import routing_cases as rc
+import routing_oracle as oracle
+from test_gpu_parity import assert_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def _ranges(layout_range):
+    lr = layout_range.cpu()
+    return lr >> 32, lr & 0xFFFFFFFF
+
+
+@pytest.mark.parametrize("R,T,H,E,K,M", [(8, 128, 7168, 256, 8, 128), (2, 40, 1024, 8, 2, 64), (4, 300, 2048, 32, 6, 300),
+                                         (1, 17, 512, 4, 3, 20)])
+@pytest.mark.parametrize("use_fp8", [True, False])
+def test_ll_stacked_sources(R, T, H, E, K, M, use_fp8):
+    import deep_ep
+    x, idx, w = rc.c5_sources(seed=5, R=R, T=T, H=H, E=E, K=K)
+    # mask a few lanes
+    g = torch.Generator().manual_seed(9)
+    mask = torch.rand(idx.shape, generator=g) < 0.1
+    idx = idx.masked_fill(mask, -1)
+    for dst_rank in sorted({0, R - 1}):
+        buf = deep_ep.Buffer(deep_ep.LogicalGroup(dst_rank, R), low_latency_mode=True)
+        stats = torch.zeros(E // R, dtype=torch.int32, device="cuda")
+        recv, count, handle, _, hook = buf.low_latency_dispatch(x.cuda(), idx.cuda(), M, E, use_fp8=use_fp8,
+                                                                cumulative_local_expert_recv_stats=stats)
+        assert hook is None
+        ref_x, ref_s, ref_cnt, ref_info, ref_range = oracle.ll_dispatch(list(x), list(idx), M, E, R, dst_rank, use_fp8)
+        assert_equal(count, ref_cnt, "packed_recv_count")
+        assert_equal(stats, ref_cnt, "cumulative stats")
+        assert_equal(handle[1], ref_range, "packed_recv_layout_range")
+        px = recv[0] if use_fp8 else recv
+        assert px.shape == (E // R, R * M, H)
+        if use_fp8:
+            assert recv[1].shape == (E // R, R * M, H // 128) and recv[1].stride(1) == 1 and recv[1].stride(2) == R * M
+        for e in range(E // R):
+            n = int(ref_cnt[e])
+            assert_equal(px[e, :n], ref_x[e, :n], f"packed_recv_x[{e}]")
+            assert_equal(handle[0][e, :n], ref_info[e, :n], f"src_info[{e}]")
+            if use_fp8:
+                assert_equal(recv[1][e, :n], ref_s[e, :n], f"scales[{e}]")
+        # reference-test invariants (tests/legacy/test_low_latency.py:110-141)
+        begin, cnt = _ranges(handle[1])
+        assert torch.equal(cnt.sum(dim=1).to(torch.int32), ref_cnt)
+        assert torch.equal(begin, torch.cumsum(cnt, 1) - cnt)
+
+        # combine: expert outputs = dequantised/plain rows times (1 + local expert id / 8)
+        y = torch.zeros((E // R, R * M, H), dtype=torch.bfloat16)
+        for e in range(E // R):
+            n = int(ref_cnt[e])
+            rows = oracle.per_token_cast_back(ref_x[e, :n], ref_s[e, :n]) if use_fp8 else ref_x[e, :n]
+            y[e, :n] = (rows.float() * (1 + e / 8)).to(torch.bfloat16)
+        out, _, _ = buf.low_latency_combine(y.cuda(), idx.cuda(), w.cuda(), handle)
+        for s in range(R):
+            ref_out = oracle.ll_combine(y, idx[s], w[s], ref_info, ref_range, s, E, R, dst_rank)
+            assert_equal(out[s] + 0.0, ref_out + 0.0, f"ll combined_x from source {s}")
+        # single-source form gives the same rows for that source
+        if R > 1:
+            s = dst_rank
+            recv1, count1, handle1, _, _ = buf.low_latency_dispatch(x[s].cuda(), idx[s].cuda(), M, E, use_fp8=use_fp8)
+            r1 = oracle.ll_dispatch([x[i] if i == s else None for i in range(R)], list(idx), M, E, R, dst_rank, use_fp8)
+            assert_equal(count1, r1[2], "single-source count")
+            assert_equal(handle1[1], r1[4], "single-source layout_range")
+            out1, _, _ = buf.low_latency_combine(y.cuda() * 0 + 1, idx[s].cuda(), w[s].cuda(), handle1)
+            assert out1.shape == (T, H)

@@ -50,6 +50,8 @@ def main():
     ap.add_argument("--bf16", action="store_true", help="BF16 dispatch instead of the fused FP8 cast")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--routing", default="case", choices=["case", "sequential"],
+                    help="sequential: every token goes to ranks 0..4 (dest rows of consecutive tokens are adjacent)")
     ap.add_argument("--l2-flush", action="store_true", help="zero a 256 MB buffer between per-kernel timings")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -68,6 +70,10 @@ def main():
 
     case = {"C2": rc.c2, "C3": rc.c3, "C4": rc.c4}[args.workload]()
     T, H, K, E, R, M = case.T, case.H, case.K, case.E, case.R, case.M
+    if args.routing == "sequential":
+        E_l = E // R
+        base = torch.tensor([0, E_l, 2 * E_l, 3 * E_l, 4 * E_l, 1, E_l + 1, 2 * E_l + 1][:K], dtype=torch.int64)
+        case.topk_idx = base.unsqueeze(0).repeat(T, 1).contiguous()
     fp8 = not args.bf16
     expanded = args.expanded
     x, idx, w = case.x.to(dev), case.topk_idx.to(dev), case.topk_weights.to(dev)

@@ -60,8 +60,7 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
     w.chunk_counts = off;  off = align_up(off + chunks * n * 4, 256);
     w.chunk_base = off;    off = align_up(off + chunks * n * 4, 256);
-    w.pos_rank = off;      off = align_up(off + lanes * 4, 256);
-    w.pos_expert = off;    off = align_up(off + lanes * 4, 256);
+    w.pos = off;           off = align_up(off + lanes * 4, 256);
     w.total_bytes = off;
     return w;
 }
@@ -187,8 +186,7 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         p.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
         p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
         p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
-        p.pos_rank = reinterpret_cast<int32_t*>(ws + w.pos_rank);
-        p.pos_expert = reinterpret_cast<int32_t*>(ws + w.pos_expert);
+        p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
         hipError_t err = launch_layout_kernel(p, stream);
         if (err != hipSuccess) return hip_fail(err, "dispatch layout launch");
     }
@@ -201,8 +199,7 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         m.num_sf_packs = a->num_sf_packs;
         m.topk_idx = a->topk_idx;
         m.topk_weights = a->topk_weights;
-        m.pos_rank = reinterpret_cast<const int32_t*>(ws + w.pos_rank);
-        m.pos_expert = reinterpret_cast<const int32_t*>(ws + w.pos_expert);
+        m.pos = reinterpret_cast<const uint32_t*>(ws + w.pos);
         m.chunk_base = reinterpret_cast<const int32_t*>(ws + w.chunk_base);
         m.expert_start = reinterpret_cast<const int32_t*>(ws + w.expert_start);
         m.cached_slot = a->dst_buffer_slot_idx;

@@ -120,6 +120,16 @@ __device__ __forceinline__ int wave_inclusive_sum(int v) {
     return v;
 }
 
+// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin: workgroup i runs on XCD i % 8.
+// This renumbering gives every XCD one contiguous range of logical workgroups, so that neighbouring
+// work items (which write neighbouring output rows) share an L2 and their partial-line writes merge.
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned block, unsigned num_blocks) {
+    constexpr unsigned kXcds = 8;
+    const unsigned per = num_blocks / kXcds;
+    if (block >= per * kXcds) return block;          // ragged tail keeps its index
+    return (block % kXcds) * per + block / kXcds;
+}
+
 // Agent-scope relaxed load/store that bypass the per-CU vector cache, for values another
 // workgroup of the same launch has just produced.
 __device__ __forceinline__ int load_agent(const int* p) {

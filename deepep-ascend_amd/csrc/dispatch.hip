@@ -37,7 +37,7 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
     Route r{-1, -1, -1, -1, -1, 0.f};
     const int n = p.R + p.E;
     const int chunk = t / kLayoutChunk;
-    int slot = -1;
+    int slot = -1, epos = -1;
     if (lane < p.K) {
         const int64_t raw = p.topk_idx[int64_t(t) * p.K + lane];
         if (raw >= 0 && raw < p.E) r.e = int(raw);
@@ -46,7 +46,9 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
             const int v = p.cached_slot[int64_t(t) * p.K + lane];
             slot = v >= 0 ? v - p.rank_idx * p.M : -1;
         } else {
-            slot = p.pos_rank[int64_t(t) * p.K + lane];
+            const uint32_t packed = p.pos[int64_t(t) * p.K + lane];
+            slot = (packed & 0xffffu) == 0xffffu ? -1 : int(packed & 0xffffu);
+            epos = int(packed >> 16);
         }
     }
     if (r.e >= 0) {
@@ -72,8 +74,7 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
             if (r.my_row >= 0 && r.my_row < p.recv_capacity)
                 r.erow = p.recv_src_metadata[int64_t(r.my_row) * (p.K + 2) + 2 + lane];
         } else {
-            r.erow = p.expert_start[r.e] + p.chunk_base[int64_t(chunk) * n + p.R + r.e] +
-                     p.pos_expert[int64_t(t) * p.K + lane];
+            r.erow = p.expert_start[r.e] + p.chunk_base[int64_t(chunk) * n + p.R + r.e] + epos;
         }
     }
     return r;
@@ -124,7 +125,8 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
 template <int kVecs>
 __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
     const int lane = threadIdx.x & 63;
-    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+    const int64_t work = int64_t(block) * kWavesPerBlock + (threadIdx.x >> 6);
     if (work >= int64_t(p.T) * p.tiles) return;
     const int t = int(work / p.tiles);
     const int tile = int(work - int64_t(t) * p.tiles);
@@ -165,7 +167,8 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
 template <int kPairs>
 __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
     const int lane = threadIdx.x & 63;
-    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+    const int64_t work = int64_t(block) * kWavesPerBlock + (threadIdx.x >> 6);
     if (work >= int64_t(p.T) * p.tiles) return;
     const int t = int(work / p.tiles);
     const int tile = int(work - int64_t(t) * p.tiles);
@@ -295,6 +298,10 @@ int tuning_override(const char* name) {
 
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
+    {
+        const char* v = getenv("DEEP_EP_HIP_XCD_REMAP");
+        p.xcd_remap = v != nullptr ? atoi(v) : 1;
+    }
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
         // Column tile = kPairs * 1024 channels per wavefront.
         int pairs = tuning_override("DEEP_EP_HIP_CAST_PAIRS");

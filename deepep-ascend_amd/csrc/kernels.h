@@ -16,8 +16,7 @@ struct WorkspaceLayout {
     size_t expert_start;   // int32[E]: first expanded row of each expert
     size_t chunk_counts;   // int32[C][R+E]
     size_t chunk_base;     // int32[C][R+E]: exclusive prefix over chunks
-    size_t pos_rank;       // int32[Tmax*K]: slot of the token inside its chunk, on master lanes
-    size_t pos_expert;     // int32[Tmax*K]: position of (token, lane) inside its chunk, per expert
+    size_t pos;            // uint32[Tmax*K]: chunk-relative positions, rank slot | expert position << 16
     size_t total_bytes;
 };
 
@@ -44,8 +43,8 @@ struct LayoutParams {
     int32_t* expert_start;
     int32_t* chunk_counts;
     int32_t* chunk_base;
-    int32_t* pos_rank;               // optional (layout-only calls skip the per-lane positions)
-    int32_t* pos_expert;
+    uint32_t* pos;                   // optional (layout-only calls skip the per-lane positions)
+    int vec_idx;                     // topk_idx is 16-byte aligned (set by the launcher)
 };
 
 hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream);
@@ -57,8 +56,7 @@ struct MoveParams {
     int num_sf_packs;
     const int64_t* topk_idx;
     const float* topk_weights;
-    const int32_t* pos_rank;
-    const int32_t* pos_expert;
+    const uint32_t* pos;
     const int32_t* chunk_base;
     const int32_t* expert_start;
     const int32_t* cached_slot;
@@ -76,6 +74,7 @@ struct MoveParams {
     int payload;         // DEEP_EP_HIP_PAYLOAD_*
     int row_bytes;       // input row bytes
     int tiles;           // column tiles per token
+    int xcd_remap;       // give each XCD a contiguous token range
     int32_t* status;
 };
 

@@ -60,8 +60,25 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
 
     // All index loads are issued before anything that could alias them is stored.
     int64_t raw[KMAX];
+    if (KMAX == 8 && p.K == 8 && p.vec_idx) {
+        if (active) {
+            const vec16* src = reinterpret_cast<const vec16*>(p.topk_idx + int64_t(t) * 8);
+            vec16 q[4];
 #pragma unroll
-    for (int k = 0; k < KMAX; ++k) raw[k] = (active && k < p.K) ? p.topk_idx[int64_t(t) * p.K + k] : int64_t(-1);
+            for (int i = 0; i < 4; ++i) q[i] = src[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                raw[2 * i] = int64_t(uint64_t(q[i].x) | (uint64_t(q[i].y) << 32));
+                raw[2 * i + 1] = int64_t(uint64_t(q[i].z) | (uint64_t(q[i].w) << 32));
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) raw[k] = -1;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) raw[k] = (active && k < p.K) ? p.topk_idx[int64_t(t) * p.K + k] : int64_t(-1);
+    }
 
     int e[KMAX], d[KMAX];
     int flags = 0;
@@ -93,11 +110,14 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     };
 
     if (active) {
-        if (p.pos_rank != nullptr) {
+        if (p.pos != nullptr) {
+            // One word per (token, lane): low 16 bits = slot of the token inside its chunk for the lane's
+            // destination rank (master lanes only), high 16 bits = position of the lane inside its chunk for
+            // its expert; 0xffff = none.
+            uint32_t packed[KMAX];
 #pragma unroll
             for (int k = 0; k < KMAX; ++k) {
-                if (k >= p.K) break;
-                int pr = -1, pe = -1;
+                uint32_t pr = 0xffffu, pe = 0xffffu;
                 if (e[k] >= 0) {
                     bool master = true;
 #pragma unroll
@@ -105,11 +125,19 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
                         if (j > k && d[j] == d[k]) master = false;
                         if (j != k && e[j] == e[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
                     }
-                    pe = rank_in_chunk(p.R + e[k]);
-                    if (master) pr = rank_in_chunk(d[k]);
+                    pe = uint32_t(rank_in_chunk(p.R + e[k]));
+                    if (master) pr = uint32_t(rank_in_chunk(d[k]));
                 }
-                p.pos_rank[int64_t(t) * p.K + k] = pr;
-                p.pos_expert[int64_t(t) * p.K + k] = pe;
+                packed[k] = pr | (pe << 16);
+            }
+            if (KMAX == 8 && p.K == 8) {
+                vec16* dst = reinterpret_cast<vec16*>(p.pos + int64_t(t) * 8);
+                dst[0] = vec16{packed[0], packed[1], packed[2], packed[3]};
+                dst[1] = vec16{packed[4], packed[5], packed[6], packed[7]};
+            } else {
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k)
+                    if (k < p.K) p.pos[int64_t(t) * p.K + k] = packed[k];
             }
         }
         if (p.is_token_in_rank != nullptr) {
@@ -126,8 +154,8 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
         p.chunk_counts[int64_t(chunk) * n + j] = c;
     }
 
-    // Hand the chunk totals to whichever workgroup finishes last.
-    __threadfence();
+    // Hand the chunk totals to whichever workgroup finishes last: release our stores, take a ticket.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     if (tid == 0) {
         const unsigned ticket = atomicAdd(p.done_counter, 1u);
@@ -135,7 +163,7 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     }
     __syncthreads();
     if (!is_last) return;
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
     // ---- last workgroup: chunk bases and public prefix sums ----
     // LDS is re-carved as int arrays: a staging slab of chunk rows, then totals / aligned / scanned.
@@ -147,20 +175,47 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     for (int c0 = 0; c0 < num_chunks; c0 += p.slab_rows) {
         const int rows = min(p.slab_rows, num_chunks - c0);
         const int32_t* src = p.chunk_counts + int64_t(c0) * n;
-        for (int i = tid; i < rows * n; i += kThreads) stage[i] = src[i];       // coalesced, independent loads
+        // 16-byte coalesced loads, all of a thread's loads in flight before its first LDS write (a plain
+        // copy loop would wait for each load in turn: one memory round trip per iteration).
+        const int total = rows * n;
+        const int total4 = (int64_t(c0) * n) % 4 == 0 ? total / 4 : 0;   // 16-byte path needs an aligned slab
+        const vec16* src4 = reinterpret_cast<const vec16*>(src);
+        vec16* stage4 = reinterpret_cast<vec16*>(stage);
+        for (int i0 = tid; i0 < total4; i0 += kThreads * 12) {
+            vec16 v[12];
+#pragma unroll
+            for (int u = 0; u < 12; ++u) {
+                const int i = i0 + u * kThreads;
+                v[u] = i < total4 ? src4[i] : vec16{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int u = 0; u < 12; ++u) {
+                const int i = i0 + u * kThreads;
+                if (i < total4) stage4[i] = v[u];
+            }
+        }
+        for (int i = total4 * 4 + tid; i < total; i += kThreads) stage[i] = src[i];
         __syncthreads();
-        for (int j = tid; j < n; j += kThreads) {                               // one column per thread
+        // Exclusive scan down each column, one column per thread, LDS reads batched by 8.
+        for (int j = tid; j < n; j += kThreads) {
             int running = totals[j];
-            for (int r = 0; r < rows; ++r) {
-                const int v = stage[r * n + j];
-                stage[r * n + j] = running;
-                running += v;
+            for (int r0 = 0; r0 < rows; r0 += 8) {
+                int v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = (r0 + u < rows) ? stage[(r0 + u) * n + j] : 0;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (r0 + u < rows) stage[(r0 + u) * n + j] = running;
+                    running += v[u];
+                }
             }
             totals[j] = running;
         }
         __syncthreads();
         int32_t* dstb = p.chunk_base + int64_t(c0) * n;
-        for (int i = tid; i < rows * n; i += kThreads) dstb[i] = stage[i];
+        vec16* dstb4 = reinterpret_cast<vec16*>(dstb);
+        for (int i = tid; i < total4; i += kThreads) dstb4[i] = stage4[i];
+        for (int i = total4 * 4 + tid; i < total; i += kThreads) dstb[i] = stage[i];
         __syncthreads();
     }
 
@@ -215,6 +270,7 @@ hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream) {
     const size_t scan_bytes = (size_t(slab_rows) + 3) * n * 4;
     const size_t lds = bitmap_bytes > scan_bytes ? bitmap_bytes : scan_bytes;
     LayoutParams q = p;
+    q.vec_idx = (reinterpret_cast<uintptr_t>(p.topk_idx) % 16 == 0) ? 1 : 0;
     q.slab_rows = slab_rows;
     dim3 grid(num_chunks), block(kThreads);
     if (p.K <= 8) {

@@ -51,6 +51,7 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     WorkspaceLayout w{};
     const size_t n = size_t(num_ranks) + num_experts;
     const size_t chunks = num_max_tokens > 0 ? (size_t(num_max_tokens) + kLayoutChunk - 1) / kLayoutChunk : 1;
+    const size_t chunks_padded = (chunks + 3) / 4 * 4;
     const size_t lanes = size_t(num_max_tokens > 0 ? num_max_tokens : 1) * num_topk;
     size_t off = 0;
     w.status = off;
@@ -58,7 +59,7 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.totals = off + 8;
     off = 256;
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
-    w.chunk_counts = off;  off = align_up(off + chunks * n * 4, 256);
+    w.chunk_counts = off;  off = align_up(off + chunks_padded * n * 4, 256);
     w.chunk_base = off;    off = align_up(off + chunks * n * 4, 256);
     w.pos = off;           off = align_up(off + lanes * 4, 256);
     w.total_bytes = off;
@@ -97,14 +98,14 @@ int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
     p.topk_idx = a->topk_idx;
     p.T = a->num_tokens; p.K = a->num_topk; p.E = a->num_experts; p.R = a->num_ranks;
     p.E_l = p.E / p.R;
-    p.A = 1;
-    p.num_tokens_per_rank = a->num_tokens_per_rank;
-    p.num_tokens_per_expert = a->num_tokens_per_expert;
     p.is_token_in_rank = a->is_token_in_rank;
+    p.pub.R = p.R; p.pub.E = p.E; p.pub.A = 1;
+    p.pub.num_tokens_per_rank = a->num_tokens_per_rank;
+    p.pub.num_tokens_per_expert = a->num_tokens_per_expert;
+    p.pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
+    p.pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
     p.status = reinterpret_cast<int32_t*>(ws + w.status);
     p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
-    p.totals = reinterpret_cast<int32_t*>(ws + w.totals);
-    p.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
     p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
     hipError_t err = launch_layout_kernel(p, static_cast<hipStream_t>(stream));
@@ -168,22 +169,38 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         REQUIRE(!(a->do_expand == 0 && a->recv_topk_idx == nullptr && a->recv_capacity > 0), "recv_topk_idx is NULL");
     }
 
+    // Publishing targets of the layout results (shared by the layout kernel and, in light mode, the move kernel).
+    PublishParams pub{};
+    pub.R = R; pub.E = E; pub.A = a->expert_alignment; pub.do_expand = a->do_expand ? 1 : 0;
+    pub.psum_rank = a->psum_num_recv_tokens_per_rank;
+    pub.psum_expert = a->psum_num_recv_tokens_per_expert;
+    pub.num_unaligned = a->num_unaligned_recv_tokens_per_expert;
+    pub.cumulative_stats = a->cumulative_local_expert_recv_stats;
+    pub.host_counts = a->host_counts;
+    pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
+    pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
+
+    // Light mode: when layout and move run in one call on the compact layout, the layout kernel only
+    // counts; every wavefront of the move kernel prefix-sums the (small) per-rank part of the chunk
+    // counts itself and workgroup 0 publishes the handle tensors.  That removes the serial tail of the
+    // layout kernel (ticket, fences, scan by the last workgroup) from the critical path.
+    const int chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
+    const int chunks_padded = (chunks + 3) / 4 * 4;
+    const int flat = R * chunks_padded;
+    const int flat_per = flat <= 256 ? 4 : flat <= 512 ? 8 : 16;
+    const bool light = do_layout && do_move && !a->do_expand && T > 0 && flat <= 1024 && (R + E) <= 512 &&
+                       getenv("DEEP_EP_HIP_NO_LIGHT_LAYOUT") == nullptr;
+
     if (do_layout) {
         LayoutParams p{};
         p.topk_idx = a->topk_idx;
         p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
-        p.A = a->expert_alignment;
-        p.do_expand = a->do_expand;
+        p.light = light ? 1 : 0;
+        p.chunks_padded = chunks_padded;
         p.copied_topk_idx = a->copied_topk_idx;
-        p.psum_rank = a->psum_num_recv_tokens_per_rank;
-        p.psum_expert = a->psum_num_recv_tokens_per_expert;
-        p.num_unaligned = a->num_unaligned_recv_tokens_per_expert;
-        p.cumulative_stats = a->cumulative_local_expert_recv_stats;
-        p.host_counts = a->host_counts;
+        p.pub = pub;
         p.status = status;
         p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
-        p.totals = reinterpret_cast<int32_t*>(ws + w.totals);
-        p.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
         p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
         p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
         p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
@@ -219,6 +236,11 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         m.do_expand = a->do_expand ? 1 : 0;
         m.payload = a->payload;
         m.row_bytes = H * elem_in;
+        m.light = light ? 1 : 0;
+        m.chunks_padded = chunks_padded;
+        m.flat_per = flat_per;
+        m.chunk_counts_t = reinterpret_cast<const int32_t*>(ws + w.chunk_counts);
+        m.pub = pub;
         m.status = status;
         hipError_t err = launch_dispatch_move(m, stream);
         if (err != hipSuccess) return hip_fail(err, "dispatch move launch");

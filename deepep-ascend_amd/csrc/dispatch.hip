@@ -14,6 +14,7 @@
 #include "common.cuh"
 #include "cast.cuh"
 #include "kernels.h"
+#include "publish.cuh"
 #include "../../include/deep_ep_hip.h"
 
 namespace deep_ep_hip {
@@ -51,14 +52,53 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
             epos = int(packed >> 16);
         }
     }
-    if (r.e >= 0) {
-        r.d = r.e / p.E_l;
-        if (slot >= 0) {
-            if (!p.cached) slot += p.chunk_base[int64_t(chunk) * n + r.d];
-            r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
+    if (r.e >= 0) r.d = r.e / p.E_l;
+    else slot = -1;
+    if (p.light) {
+        // Exclusive prefix of the per-rank chunk counts in (rank, chunk) order: lane L scans entries
+        // [L * per, (L + 1) * per) of the flattened [R][chunks_padded] table, a wave scan joins the lanes.
+        // The prefix at (d, chunk) is at once the start of bucket d and the rows that earlier chunks put
+        // into it, so no other table is needed.
+        const int per = p.flat_per;
+        const int nflat = p.R * p.chunks_padded;
+        int ex[16];
+        int sum = 0;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            vec16 v{0, 0, 0, 0};
+            if (u * 4 < per && lane * per + u * 4 < nflat)
+                v = load16(p.chunk_counts_t + lane * per + u * 4);
+            ex[4 * u] = sum; sum += int(v.x);
+            ex[4 * u + 1] = sum; sum += int(v.y);
+            ex[4 * u + 2] = sum; sum += int(v.z);
+            ex[4 * u + 3] = sum; sum += int(v.w);
         }
-    } else {
-        slot = -1;
+        const int lane_base = wave_inclusive_sum(sum) - sum;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ex[i] += lane_base;
+        // prefix at flat position f: held by lane f / per as its entry f % per (every lane takes part)
+        auto prefix_at = [&](int f) {
+            const int owner = f / per, off = f - owner * per;
+            int got = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                if (i < per) {
+                    const int v = __shfl(ex[i], owner, kWaveSize);
+                    if (i == off) got = v;
+                }
+            }
+            return got;
+        };
+        const int fd = (r.d >= 0 ? r.d : 0) * p.chunks_padded;
+        const int bucket_start = prefix_at(fd);
+        const int before = prefix_at(fd + chunk);
+        if (r.d >= 0 && slot >= 0) {
+            r.row_c = before + slot;
+            slot = r.row_c - bucket_start;      // slot inside the destination bucket
+        }
+    } else if (r.e >= 0 && slot >= 0) {
+        if (!p.cached) slot += p.chunk_base[int64_t(chunk) * n + r.d];
+        r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
     }
     if (first_tile && !p.cached && lane < p.K && p.dst_buffer_slot_idx != nullptr)
         p.dst_buffer_slot_idx[int64_t(t) * p.K + lane] = (r.e >= 0 && slot >= 0) ? p.rank_idx * p.M + slot : -1;
@@ -121,9 +161,31 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
     return __ballot(row_of_lane >= 0);
 }
 
+// Light mode: workgroup 0 sums the transposed chunk counts and publishes the handle tensors.  Every thread
+// of the workgroup must call this before any early exit.
+__device__ __forceinline__ void publish_from_chunk_counts(const MoveParams& p) {
+    extern __shared__ int publish_lds[];          // [R + E] totals, [2 * E] scratch, then per-wave scan slots
+    const int n = p.R + p.E;
+    int* totals = publish_lds;
+    int* scratch = totals + n;
+    int* scan_tmp = scratch + 2 * p.E;
+    for (int j = threadIdx.x; j < n; j += kThreads) {
+        const int32_t* row = p.chunk_counts_t + int64_t(j) * p.chunks_padded;
+        int sum = 0;
+        for (int c = 0; c < p.chunks_padded; c += 4) {
+            const vec16 v = load16(row + c);
+            sum += int(v.x) + int(v.y) + int(v.z) + int(v.w);
+        }
+        totals[j] = sum;
+    }
+    __syncthreads();
+    publish_counts<kThreads>(p.pub, totals, scratch, scan_tmp);
+}
+
 // ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
 template <int kVecs>
 __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
+    if (p.light && blockIdx.x == 0) publish_from_chunk_counts(p);
     const int lane = threadIdx.x & 63;
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
     const int64_t work = int64_t(block) * kWavesPerBlock + (threadIdx.x >> 6);
@@ -166,6 +228,7 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
 template <int kPairs>
 __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
+    if (p.light && blockIdx.x == 0) publish_from_chunk_counts(p);
     const int lane = threadIdx.x & 63;
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
     const int64_t work = int64_t(block) * kWavesPerBlock + (threadIdx.x >> 6);
@@ -271,12 +334,16 @@ __global__ __launch_bounds__(kThreads) void cast_kernel(const CastParams p) {
     if ((lane & 7) == 0 && group < groups && elem < p.H) p.scales[int64_t(t) * groups + group] = scale_inv;
 }
 
+size_t publish_lds_bytes(const MoveParams& p) {
+    return p.light ? size_t(p.R + 3 * p.E + kWavesPerBlock) * sizeof(int) : 0;
+}
+
 template <int kVecs>
 hipError_t launch_copy(MoveParams p, hipStream_t stream) {
     p.tiles = (p.row_bytes + kVecs * 1024 - 1) / (kVecs * 1024);
     const int64_t waves = int64_t(p.T) * p.tiles;
     const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(dispatch_copy_kernel<kVecs>, dim3(blocks), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL(dispatch_copy_kernel<kVecs>, dim3(blocks), dim3(kThreads), publish_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 
@@ -285,7 +352,7 @@ hipError_t launch_cast(MoveParams p, hipStream_t stream) {
     p.tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
     const int64_t waves = int64_t(p.T) * p.tiles;
     const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(dispatch_cast_kernel<kPairs>, dim3(blocks), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL(dispatch_cast_kernel<kPairs>, dim3(blocks), dim3(kThreads), publish_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 
@@ -300,7 +367,7 @@ hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
     {
         const char* v = getenv("DEEP_EP_HIP_XCD_REMAP");
-        p.xcd_remap = v != nullptr ? atoi(v) : 1;
+        p.xcd_remap = v != nullptr ? atoi(v) : 0;
     }
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
         // Column tile = kPairs * 1024 channels per wavefront.

@@ -22,29 +22,37 @@ struct WorkspaceLayout {
 
 WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_experts, int num_ranks);
 
+// Where the public results of the layout computation go (any pointer may be NULL).
+struct PublishParams {
+    int R, E;
+    int A;            // expert alignment
+    int do_expand;
+    int32_t* num_tokens_per_rank;
+    int32_t* num_tokens_per_expert;
+    int32_t* psum_rank;
+    int32_t* psum_expert;
+    int32_t* num_unaligned;
+    int32_t* cumulative_stats;
+    int32_t* host_counts;            // host-mapped
+    int32_t* expert_start;           // workspace
+    int32_t* totals_out;             // workspace: total compact rows, total expanded rows
+};
+
 struct LayoutParams {
     const int64_t* topk_idx;
     int T, K, E, R, E_l;
-    int A;            // expert alignment
-    int do_expand;
-    int slab_rows;    // chunk rows staged in LDS per pass of the final scan (set by the launcher)
-    int32_t* num_tokens_per_rank;    // optional
-    int32_t* num_tokens_per_expert;  // optional
+    int light;            // 1: only count (transposed chunk counts); the move kernel finishes the job
+    int chunks_padded;    // row length of the transposed chunk counts (light mode)
+    int slab_rows;        // chunk rows staged in LDS per pass of the final scan (set by the launcher)
+    int vec_idx;          // topk_idx is 16-byte aligned (set by the launcher)
     uint8_t* is_token_in_rank;       // optional
     int64_t* copied_topk_idx;        // optional
-    int32_t* psum_rank;              // optional
-    int32_t* psum_expert;            // optional
-    int32_t* num_unaligned;          // optional
-    int32_t* cumulative_stats;       // optional
-    int32_t* host_counts;            // optional, host-mapped
+    PublishParams pub;
     int32_t* status;
     uint32_t* done_counter;
-    int32_t* totals;
-    int32_t* expert_start;
     int32_t* chunk_counts;
     int32_t* chunk_base;
     uint32_t* pos;                   // optional (layout-only calls skip the per-lane positions)
-    int vec_idx;                     // topk_idx is 16-byte aligned (set by the launcher)
 };
 
 hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream);
@@ -75,6 +83,12 @@ struct MoveParams {
     int row_bytes;       // input row bytes
     int tiles;           // column tiles per token
     int xcd_remap;       // give each XCD a contiguous token range
+    // light mode (compact layout, layout and move in one call): bases come from the transposed chunk counts
+    int light;
+    int chunks_padded;   // row length of chunk_counts_t
+    int flat_per;        // rank-part entries each lane scans (4, 8 or 16)
+    const int32_t* chunk_counts_t;   // [R + E][chunks_padded]
+    PublishParams pub;   // written by workgroup 0
     int32_t* status;
 };
 

@@ -15,6 +15,7 @@
 // public prefix sums.
 #include "common.cuh"
 #include "kernels.h"
+#include "publish.cuh"
 #include "../../include/deep_ep_hip.h"
 
 namespace deep_ep_hip {
@@ -23,25 +24,6 @@ namespace {
 
 constexpr int kThreads = kLayoutChunk;
 constexpr int kWaves = kThreads / kWaveSize;
-
-// In-place inclusive scan of a[0..n) in LDS by the whole workgroup.  tmp holds kWaves ints.
-__device__ void block_inclusive_scan(int* a, int n, int* tmp) {
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int per = (n + kThreads - 1) / kThreads;
-    const int begin = min(tid * per, n), end = min(begin + per, n);
-    int s = 0;
-    for (int i = begin; i < end; ++i) s += a[i];
-    const int inc = wave_inclusive_sum(s);
-    if (lane == kWaveSize - 1) tmp[wave] = inc;
-    __syncthreads();
-    int run = inc - s;
-    for (int w = 0; w < wave; ++w) run += tmp[w];
-    for (int i = begin; i < end; ++i) {
-        run += a[i];
-        a[i] = run;
-    }
-    __syncthreads();
-}
 
 template <int KMAX>
 __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) {
@@ -151,7 +133,17 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
         int c = 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) c += __popcll(bitmap[j * kWaves + w]);
-        p.chunk_counts[int64_t(chunk) * n + j] = c;
+        if (p.light) p.chunk_counts[int64_t(j) * p.chunks_padded + chunk] = c;   // [bucket][chunk]
+        else p.chunk_counts[int64_t(chunk) * n + j] = c;                         // [chunk][bucket]
+    }
+    if (p.light) {
+        // The consumer (the move kernel) prefix-sums the transposed counts itself; only the padding
+        // columns still have to be cleared.
+        const int pad = p.chunks_padded - int(gridDim.x);
+        if (chunk == 0)
+            for (int i = tid; i < n * pad; i += kThreads)
+                p.chunk_counts[int64_t(i / pad) * p.chunks_padded + gridDim.x + i % pad] = 0;
+        return;
     }
 
     // Hand the chunk totals to whichever workgroup finishes last: release our stores, take a ticket.
@@ -219,41 +211,9 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
         __syncthreads();
     }
 
-    for (int j = tid; j < p.E; j += kThreads) {
-        const int cnt = totals[p.R + j];
-        aligned[j] = (cnt + p.A - 1) / p.A * p.A;
-        if (p.num_tokens_per_expert != nullptr) p.num_tokens_per_expert[j] = cnt;
-        if (p.num_unaligned != nullptr) p.num_unaligned[j] = cnt;
-        if (p.cumulative_stats != nullptr) p.cumulative_stats[j] += cnt;
-        if (p.host_counts != nullptr) p.host_counts[p.R + j] = -aligned[j] - 1;
-    }
-    for (int r = tid; r < p.R; r += kThreads) {
-        if (p.num_tokens_per_rank != nullptr) p.num_tokens_per_rank[r] = totals[r];
-        if (p.host_counts != nullptr) p.host_counts[r] = -totals[r] - 1;
-    }
     __syncthreads();
-
-    int* aligned_incl = aligned + p.E;                     // [E]
-    for (int j = tid; j < p.E; j += kThreads) aligned_incl[j] = aligned[j];
-    __syncthreads();
-    block_inclusive_scan(aligned_incl, p.E, scan_tmp);
-    for (int j = tid; j < p.E; j += kThreads) {
-        const int start = aligned_incl[j] - aligned[j];
-        p.expert_start[j] = start;
-        if (p.psum_expert != nullptr) p.psum_expert[j] = p.do_expand ? start + totals[p.R + j] : aligned_incl[j];
-    }
-    const int total_expanded = p.E > 0 ? aligned_incl[p.E - 1] : 0;
-    __syncthreads();
-
-    block_inclusive_scan(totals, p.R, scan_tmp);           // ranks: inclusive prefix in place
-    for (int r = tid; r < p.R; r += kThreads)
-        if (p.psum_rank != nullptr) p.psum_rank[r] = totals[r];
-    if (tid == 0) {
-        p.totals[0] = totals[p.R - 1];
-        p.totals[1] = total_expanded;
-        *p.done_counter = 0u;                              // ready for the next launch
-    }
-    if (p.host_counts != nullptr) __threadfence_system();
+    publish_counts<kThreads>(p.pub, totals, aligned, scan_tmp);
+    if (tid == 0) *p.done_counter = 0u;                    // ready for the next launch
 }
 
 }  // namespace

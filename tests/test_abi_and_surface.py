@@ -1,0 +1,230 @@
+"""CPU-side checks of the boundary: the C ABI exports what include/deep_ep_hip.h declares, the ctypes
+mirrors have the header's struct layouts, arguments are validated before anything is launched, and
+the Python surface has the reference's names and signatures.  No GPU work happens here."""
+import ctypes
+import inspect
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "deep_ep_hip.h")
+
+import deep_ep
+from deep_ep import _C, _abi
+
+
+def header_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(deep_ep_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = header_functions()
+    assert len(names) >= 11
+    for name in names:
+        assert hasattr(_abi.lib, name), f"{name} is declared in the header but not exported"
+    assert sorted(_abi.EXPORTS) == names, "ctypes binding table and header disagree"
+    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 1
+
+
+def test_ctypes_structs_match_the_header_layout():
+    structs = {"deep_ep_hip_layout_args": _abi.LayoutArgs, "deep_ep_hip_dispatch_args": _abi.DispatchArgs,
+               "deep_ep_hip_combine_args": _abi.CombineArgs, "deep_ep_hip_ll_dispatch_args": _abi.LLDispatchArgs,
+               "deep_ep_hip_ll_combine_args": _abi.LLCombineArgs, "deep_ep_hip_cast_args": _abi.CastArgs}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {"]
+    for cname, cls in structs.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for field, _ in cls._fields_:
+            lines.append(f'  printf("{cname}.{field} %zu\\n", offsetof({cname}, {field}));')
+    lines += ["  return 0;", "}"]
+    with tempfile.TemporaryDirectory() as tmp:
+        src, exe = os.path.join(tmp, "layout.c"), os.path.join(tmp, "layout")
+        open(src, "w").write("\n".join(lines))
+        subprocess.run(["gcc", "-std=c11", "-o", exe, src], check=True, capture_output=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    got = dict(line.split() for line in out.strip().splitlines())
+    for cname, cls in structs.items():
+        assert int(got[cname]) == ctypes.sizeof(cls), cname
+        for field, _ in cls._fields_:
+            assert int(got[f"{cname}.{field}"]) == getattr(cls, field).offset, f"{cname}.{field}"
+
+
+def test_header_limits_match_python_constants():
+    text = open(HEADER).read()
+    for name, value in (("DEEP_EP_HIP_MAX_TOPK", _abi.MAX_TOPK), ("DEEP_EP_HIP_MAX_EXPERTS", _abi.MAX_EXPERTS),
+                        ("DEEP_EP_HIP_MAX_RANKS", _abi.MAX_RANKS), ("DEEP_EP_HIP_PHASE_LAYOUT", _abi.PHASE_LAYOUT),
+                        ("DEEP_EP_HIP_PHASE_MOVE", _abi.PHASE_MOVE), ("DEEP_EP_HIP_PAYLOAD_CAST_FP8", _abi.PAYLOAD_CAST_FP8),
+                        ("DEEP_EP_HIP_STATUS_ROW_OVERFLOW", _abi.STATUS_ROW_OVERFLOW)):
+        assert re.search(rf"#define {name} {value}\b", text), name
+
+
+def _dispatch_args(**kw):
+    a = _abi.DispatchArgs()
+    a.phases = _abi.PHASE_LAYOUT
+    a.num_tokens, a.hidden, a.num_topk, a.num_experts, a.num_ranks = 16, 256, 2, 8, 2
+    a.num_max_tokens_per_rank, a.expert_alignment = 16, 1
+    # never dereferenced: every case below is rejected before a launch
+    a.topk_idx = a.workspace = a.psum_num_recv_tokens_per_rank = 0x1000
+    a.psum_num_recv_tokens_per_expert = a.num_unaligned_recv_tokens_per_expert = 0x1000
+    a.workspace_bytes = 1 << 30
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    (dict(num_topk=0), "num_topk"), (dict(num_topk=33), "num_topk"), (dict(num_experts=9), "divisible"),
+    (dict(num_ranks=0), "num_ranks"), (dict(num_tokens=17), "num_max_tokens_per_rank"), (dict(rank_idx=2), "rank_idx"),
+    (dict(phases=0), "phases"), (dict(cached=1), "cached"), (dict(do_zero_padding=1), "do_expand"),
+    (dict(expert_alignment=0), "expert_alignment"), (dict(payload=7), "payload"), (dict(workspace=0), "workspace"),
+    (dict(num_experts=2048, num_ranks=2), "num_experts"),
+    (dict(phases=_abi.PHASE_MOVE, hidden=100, payload=_abi.PAYLOAD_FP8), "16 bytes"),
+    (dict(phases=_abi.PHASE_MOVE, hidden=192, payload=_abi.PAYLOAD_CAST_FP8, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000,
+          dst_buffer_slot_idx=0x1000), "128"),
+])
+def test_dispatch_rejects_bad_arguments_before_launch(kw, fragment):
+    rc = _abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(_dispatch_args(**kw)), None)
+    assert rc == -1, kw
+    assert fragment in _abi.last_error(), _abi.last_error()
+
+
+def test_workspace_size_contract():
+    rc = _abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(_dispatch_args(workspace_bytes=64)), None)
+    assert rc == -2 and "needed" in _abi.last_error()
+    need = _abi.lib.deep_ep_hip_workspace_bytes
+    assert need(0, 2, 8, 2) > 0 and need(8192, 8, 256, 8) >= need(4096, 8, 256, 8) >= need(128, 2, 8, 2)
+    assert need(8192, 8, 256, 8) % 256 == 0 and need(8192, 8, 256, 8) < (1 << 21)
+    assert need(-1, 8, 256, 8) == 0 and _abi.lib.deep_ep_hip_ll_workspace_bytes(8, 128, 8, 32) > 0
+    with pytest.raises(RuntimeError, match="DeepEP HIP backend"):
+        _abi.check(-1, "probe")
+
+
+def test_other_entry_points_validate():
+    a = _abi.LayoutArgs()
+    a.num_tokens, a.num_topk, a.num_experts, a.num_ranks = 4, 2, 8, 3
+    assert _abi.lib.deep_ep_hip_launch_layout(ctypes.byref(a), None) == -1
+    c = _abi.CombineArgs()
+    c.num_tokens, c.hidden, c.num_topk, c.num_experts, c.num_ranks = 4, 100, 2, 8, 2       # 200-byte rows
+    assert _abi.lib.deep_ep_hip_launch_combine(ctypes.byref(c), None) == -1 and "16 bytes" in _abi.last_error()
+    l = _abi.LLDispatchArgs()
+    l.num_src_ranks, l.src_token_stride, l.num_topk, l.num_experts, l.num_local_experts = 1, 8, 2, 8, 4
+    l.expert_begin, l.num_ranks, l.num_max_dispatch_tokens_per_rank, l.hidden, l.use_fp8 = 6, 2, 8, 192, 1
+    assert _abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(l), None) == -1
+    assert _abi.lib.deep_ep_hip_launch_cast_fp8(None, None) == -1
+
+
+def test_missing_library_fails_loudly():
+    env = dict(os.environ, DEEP_EP_HIP_LIBRARY="/nonexistent/libdeep_ep_hip.so",
+               PYTHONPATH=os.path.join(ROOT, "deepep-ascend_amd"))
+    res = subprocess.run([sys.executable, "-c", "import deep_ep"], env=env, capture_output=True, text=True)
+    assert res.returncode != 0 and "ImportError" in res.stderr and "no fallback" in res.stderr
+
+
+def test_no_product_module_touches_the_oracle():
+    pkg = os.path.join(ROOT, "deepep-ascend_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cuh", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "routing_oracle" not in text and "fp8_ref" not in text and "/oracle" not in text, f
+
+
+# ---- Python surface (names and signatures of the reference: deep_ep/__init__.py:92-109,
+# deep_ep/buffers/elastic.py:331-349,1391-1412,1616-1626; binding contract tests/platform/api_contract.py:1-42)
+def test_module_surface():
+    for name in ("ElasticBuffer", "EPHandle", "EventOverlap", "EventHandle", "Buffer", "topk_idx_t", "__version__"):
+        assert hasattr(deep_ep, name)
+    assert deep_ep.topk_idx_t == torch.int64
+    for name in ("get_platform", "topk_idx_t", "EventHandle", "ElasticBuffer", "calculate_elastic_buffer_size"):
+        assert hasattr(_C, name)
+    assert _C.get_platform() == "hip"
+    for m in ("destroy", "get_comm_stream", "get_physical_domain_size", "get_logical_domain_size", "barrier", "dispatch", "combine"):
+        assert callable(getattr(_C.ElasticBuffer, m))
+    assert callable(_C.EventHandle.current_stream_wait) and hasattr(_C.EventHandle, "__copy__")
+    assert hasattr(_C.ElasticBuffer, "cpu_comm_t")
+
+
+def _params(fn):
+    return [p for p in inspect.signature(fn).parameters if p != "self"]
+
+
+def test_signatures_are_drop_in():
+    ctor = ["group", "num_bytes", "num_cpu_bytes", "num_max_tokens_per_rank", "hidden", "num_topk", "use_fp8_dispatch",
+            "deterministic", "allow_hybrid_mode", "allow_multiple_reduction", "prefer_overlap_with_compute", "sl_idx",
+            "num_allocated_qps", "num_cpu_timeout_secs", "num_gpu_timeout_secs", "explicitly_destroy"]
+    assert _params(deep_ep.ElasticBuffer.__init__) == ctor
+    dispatch = ["x", "topk_idx", "topk_weights", "cumulative_local_expert_recv_stats", "num_experts",
+                "num_max_tokens_per_rank", "expert_alignment", "num_sms", "num_qps", "previous_event",
+                "previous_event_before_epilogue", "async_with_compute_stream", "allocate_on_comm_stream", "handle",
+                "do_handle_copy", "do_cpu_sync", "do_expand", "do_zero_padding", "use_tma_aligned_col_major_sf"]
+    got = _params(deep_ep.ElasticBuffer.dispatch)
+    assert got[:len(dispatch)] == dispatch and got[len(dispatch):] == ["cast_to_fp8"]
+    combine = ["x", "handle", "topk_weights", "bias", "num_sms", "num_qps", "previous_event",
+               "previous_event_before_epilogue", "async_with_compute_stream", "allocate_on_comm_stream"]
+    assert _params(deep_ep.ElasticBuffer.combine) == combine
+    assert _params(deep_ep.ElasticBuffer.get_buffer_size_hint) == ["group", "num_max_tokens_per_rank", "hidden", "num_topk",
+                                                                  "use_fp8_dispatch", "allow_hybrid_mode",
+                                                                  "allow_multiple_reduction"]
+    assert _params(deep_ep.Buffer.get_dispatch_layout) == ["topk_idx", "num_experts", "previous_event", "async_finish",
+                                                           "allocate_on_comm_stream"]
+    assert _params(deep_ep.Buffer.low_latency_dispatch) == ["x", "topk_idx", "num_max_dispatch_tokens_per_rank", "num_experts",
+                                                            "cumulative_local_expert_recv_stats", "dispatch_wait_recv_cost_stats",
+                                                            "use_fp8", "round_scale", "use_ue8m0", "async_finish", "return_recv_hook"]
+    assert _params(deep_ep.Buffer.low_latency_combine) == ["x", "topk_idx", "topk_weights", "handle", "use_logfmt", "zero_copy",
+                                                           "async_finish", "return_recv_hook", "out", "combine_wait_recv_cost_stats"]
+    # the runtime keeps the positional order of the compiled binding (29 dispatch / 18 combine arguments, then extensions)
+    assert len(_params(_C.ElasticBuffer.dispatch)) == 30 and _params(_C.ElasticBuffer.dispatch)[-1] == "cast_to_fp8"
+    assert len(_params(_C.ElasticBuffer.combine)) == 19 and _params(_C.ElasticBuffer.combine)[-1] == "dst_buffer_slot_idx"
+    assert len(_params(_C.ElasticBuffer.__init__)) == 14
+
+
+def test_handle_fields():
+    idx = torch.zeros((2, 2), dtype=torch.int64)
+    h = deep_ep.EPHandle(False, 8, 1, 16, 4, idx, 3, 3, [1, 2], idx, idx, idx, idx, idx, None, None)
+    expected = {"do_expand", "num_experts", "expert_alignment", "num_max_tokens_per_rank", "num_sms", "topk_idx",
+                "psum_num_recv_tokens_per_scaleup_rank", "psum_num_recv_tokens_per_expert",
+                "num_unaligned_recv_tokens_per_expert", "num_recv_tokens_per_expert_list", "recv_src_metadata",
+                "dst_buffer_slot_idx", "token_metadata_at_forward", "channel_linked_list", "num_recv_tokens",
+                "num_expanded_tokens", "cached_recv_src_metadata_before_sort"}
+    assert set(vars(h)) == expected      # field set asserted by the reference at run_two_rank_dispatch.py:594-606
+
+
+def test_buffer_size_calculus_worked_numbers():
+    # T=8192 per rank, H=7168, K=8, R=8 (Appendix A of the reference's calculus): BF16 904 MiB, FP8 max(512, 900) MiB
+    mib = 1 << 20
+    assert _C.calculate_elastic_buffer_size(8, 8192, 7168, 8, False, True, True) == 904 * mib
+    assert _C.calculate_elastic_buffer_size(8, 8192, 7168, 8, True, True, True) == 900 * mib
+    assert _C.calculate_elastic_buffer_size(8, 128, 1024, 0, False, True, True) % _C.get_elastic_buffer_alignment() == 0
+    with pytest.raises(RuntimeError):
+        _C.calculate_elastic_buffer_size(8, 0, 7168, 8, False, True, True)
+    g = deep_ep.LogicalGroup(3, 8)
+    assert (g.rank(), g.size()) == (3, 8)
+    assert deep_ep.ElasticBuffer.get_buffer_size_hint(g, 8192, 7168, 8) == 904 * mib
+
+
+def test_event_overlap_hooks_without_gpu():
+    class FakeEvent:
+        waits = 0
+        def current_stream_wait(self):
+            FakeEvent.waits += 1
+    calls = []
+    ev = deep_ep.EventOverlap(FakeEvent())
+    ev.register_hook_after_wait(lambda: calls.append(1))
+    with pytest.raises(AssertionError):
+        ev.register_hook_after_wait(lambda: None)
+    with ev(release_handle=True):
+        pass
+    assert FakeEvent.waits == 1 and calls == [1] and ev.event is None and ev.hook_after_wait is None
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU failure mode")
+def test_runtime_fails_loudly_without_gpu():
+    with pytest.raises(RuntimeError, match="no GPU"):
+        deep_ep.ElasticBuffer(deep_ep.LogicalGroup(0, 2), num_max_tokens_per_rank=16, hidden=256, num_topk=2)

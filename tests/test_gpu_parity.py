@@ -215,3 +215,40 @@ def test_cached_dispatch_and_no_sync(name, do_expand):
     else:
         assert_equal(rw_c.cpu()[valid], ref2.recv_topk_weights[valid], "cached expanded weights")
     buf.check_device_status()
+
+
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("cast", [False, True])
+def test_dispatch_without_cpu_sync(name, cast):
+    """Layout and move in one call (no host round trip): worst-case sized outputs whose leading rows, and
+    every handle tensor, equal the oracle's."""
+    case = CASES[name]()
+    if cast and case.H % 128:
+        pytest.skip("hidden not a multiple of 128")
+    buf = _buffer(case, rank=case.R - 1)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    stats = torch.zeros(case.E, dtype=torch.int32, device="cuda")
+    for _ in range(2):   # twice: the workspace must be left clean for the next call
+        recv_x, recv_idx, recv_w, handle, _ = buf.dispatch(x, idx, w, num_experts=case.E, do_cpu_sync=False,
+                                                           cast_to_fp8=cast, cumulative_local_expert_recv_stats=stats)
+    payload = oracle.per_token_cast_to_fp8(case.x) if cast else case.x
+    ref = oracle.dispatch(payload, case.topk_idx, case.topk_weights, case.E, case.R, case.R - 1, case.M)
+    n = ref.num_recv_tokens
+    assert handle.num_recv_tokens == case.M * case.R and handle.num_recv_tokens_per_expert_list == []
+    if cast:
+        assert_equal(recv_x[0][:n], ref.recv_x, "recv_x")
+        assert_equal(recv_x[1][:n], ref.recv_sf, "recv_sf")
+    else:
+        assert_equal(recv_x[:n], ref.recv_x, "recv_x")
+    assert_equal(recv_idx[:n], ref.recv_topk_idx, "recv_topk_idx")
+    assert_equal(recv_w[:n], ref.recv_topk_weights, "recv_topk_weights")
+    _check_handle(handle, ref, case, False)
+    assert_equal(stats, 2 * ref.num_unaligned_recv_tokens_per_expert, "cumulative stats after two calls")
+    # combine straight from the worst-case sized buffers
+    y = torch.zeros((case.M * case.R, case.H), dtype=torch.bfloat16)
+    y[:n] = (ref.recv_x[0] if cast else ref.recv_x).to(torch.float32).to(torch.bfloat16)
+    out, out_w, _ = buf.combine(y.cuda(), handle, topk_weights=recv_w)
+    ref_out, _ = oracle.combine(y[:n], case.topk_idx, ref.recv_src_metadata, ref.dst_buffer_slot_idx,
+                                ref.psum_num_recv_tokens_per_scaleup_rank, case.E, case.R, case.R - 1, case.M)
+    assert_equal(out + 0.0, ref_out + 0.0, "combined_x")
+    buf.check_device_status()

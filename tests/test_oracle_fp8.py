@@ -1,0 +1,147 @@
+"""Pins the FP8 cast of the oracle (CPU only).
+
+Three independent statements of the same arithmetic must agree bit for bit:
+  * oracle.per_token_cast_to_fp8 (torch eager; the conversion itself is the torch library routine),
+  * oracle/fp8_ref.c (plain C: nearest-representable search, volatile fp32 arithmetic),
+  * closed-form facts of the format and of the recipe.
+A dropped clamp, a reciprocal-multiply instead of the division, truncation instead of round-to-nearest-even
+or a wrong subnormal boundary each fail at least one test below.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+import routing_oracle as oracle
+
+ORACLE_DIR = os.path.dirname(os.path.abspath(oracle.__file__))
+
+
+@pytest.fixture(scope="module")
+def cref():
+    lib = os.path.join(ORACLE_DIR, "libfp8_ref.so")
+    if not os.path.exists(lib):
+        subprocess.run(["make", "-C", ORACLE_DIR, lib], check=True, capture_output=True)
+    h = ctypes.CDLL(lib)
+    h.oracle_e4m3_from_f32.restype = ctypes.c_uint8
+    h.oracle_e4m3_from_f32.argtypes = [ctypes.c_float]
+    h.oracle_cast_1x128.restype = None
+    h.oracle_cast_1x128.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    h.oracle_ordered_sum_bf16.restype = None
+    h.oracle_ordered_sum_bf16.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    return h
+
+
+def c_cast(cref, x_bf16):
+    T, H = x_bf16.shape
+    xin = x_bf16.contiguous().view(torch.int16).numpy().copy()
+    out = np.zeros((T, H), dtype=np.uint8)
+    scales = np.zeros((T, (H + 127) // 128), dtype=np.float32)
+    cref.oracle_cast_1x128(xin.ctypes.data, T, H, out.ctypes.data, scales.ctypes.data)
+    return torch.from_numpy(out), torch.from_numpy(scales)
+
+
+def test_known_conversions(cref):
+    # (value, expected e4m3 byte): subnormal boundary, rounding to even, saturation edge
+    cases = [(2.0 ** -10, 0x00), (0.0014, 0x01), (2.0 ** -9, 0x01), (1.5 * 2.0 ** -9, 0x02), (17.0, 0x58), (19.0, 0x5a),
+             (448.0, 0x7e), (448.00003, 0x7e), (464.0, 0x7e), (464.00003, 0x7f), (float("inf"), 0x7f),
+             (-448.0, 0xfe), (0.0, 0x00), (1.0, 0x38), (-1.0, 0xb8), (2.0 ** -6, 0x08), (0.9375 * 2.0 ** -6, 0x08)]
+    for value, byte in cases:
+        t = torch.tensor([value], dtype=torch.float32)
+        assert int(t.to(torch.float8_e4m3fn).view(torch.uint8)) == byte, value
+        assert cref.oracle_e4m3_from_f32(float(t)) == byte, value
+    # 17 -> 16 and 19 -> 20 are the two directions of round-half-to-even at spacing 2
+    assert float(torch.tensor([0x58], dtype=torch.uint8).view(torch.float8_e4m3fn).float()) == 16.0
+    assert float(torch.tensor([0x5a], dtype=torch.uint8).view(torch.float8_e4m3fn).float()) == 20.0
+
+
+def test_c_encoder_matches_library_on_all_bf16_values(cref):
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    vals = bits.view(torch.bfloat16).to(torch.float32)
+    lib = vals.to(torch.float8_e4m3fn).view(torch.uint8)
+    got = torch.tensor([cref.oracle_e4m3_from_f32(float(v)) for v in vals.tolist()], dtype=torch.uint8)
+    nan = vals != vals
+    assert torch.equal(got[~nan], lib[~nan])
+    assert ((got[nan] & 0x7f) == 0x7f).all() and ((lib[nan] & 0x7f) == 0x7f).all()
+
+
+def test_c_encoder_matches_library_on_dense_fp32_sweep(cref):
+    g = torch.Generator().manual_seed(0)
+    mags = torch.cat([torch.rand(20000, generator=g) * 470.0, torch.rand(20000, generator=g) * 0.05,
+                      2.0 ** torch.randint(-12, 9, (5000,), generator=g).float() * (1 + torch.randint(0, 17, (5000,), generator=g).float() / 16)])
+    vals = mags * torch.where(torch.rand(mags.shape, generator=g) < 0.5, -1.0, 1.0)
+    lib = vals.to(torch.float8_e4m3fn).view(torch.uint8)
+    got = torch.tensor([cref.oracle_e4m3_from_f32(float(v)) for v in vals.tolist()], dtype=torch.uint8)
+    assert torch.equal(got, lib)
+
+
+@pytest.mark.parametrize("hidden", [128, 384, 7168, 200])
+def test_torch_oracle_matches_c_restatement(cref, hidden):
+    g = torch.Generator().manual_seed(hidden)
+    x = (torch.randn((24, hidden), generator=g) * torch.logspace(-6, 4, 24).unsqueeze(1)).to(torch.bfloat16)
+    x[3] = 0                      # all-zero groups: the 1e-4 clamp decides
+    x[4, ::7] = 0
+    q, s = oracle.per_token_cast_to_fp8(x)
+    cq, cs = c_cast(cref, x)
+    assert torch.equal(q.view(torch.uint8), cq)
+    assert torch.equal(s.view(torch.int32), cs.view(torch.int32))
+
+
+def test_every_bf16_pattern_as_payload(cref):
+    # all finite bf16 magnitudes, arranged so that each 128-group has its own amax
+    bits = torch.arange(0, 0x7f80, dtype=torch.int32)
+    vals = bits.to(torch.int16).view(torch.bfloat16)
+    x = torch.cat([vals, -vals]).view(-1, 128)
+    x = x[torch.randperm(x.shape[0], generator=torch.Generator().manual_seed(1))].view(-1, 256)   # 510 groups
+    q, s = oracle.per_token_cast_to_fp8(x)
+    cq, cs = c_cast(cref, x)
+    assert torch.equal(q.view(torch.uint8), cq)
+    assert torch.equal(s.view(torch.int32), cs.view(torch.int32))
+
+
+def test_recipe_identities():
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn((64, 1024), generator=g) * 3).to(torch.bfloat16)
+    x[0] = 0
+    q, s = oracle.per_token_cast_to_fp8(x)
+    qb = q.view(torch.uint8).view(64, 8, 128)
+    xg = x.float().view(64, 8, 128)
+    amax = xg.abs().amax(dim=2)
+    # the element that attains amax always encodes to +-448
+    pos = xg.abs().argmax(dim=2, keepdim=True)
+    enc = qb.gather(2, pos).squeeze(2) & 0x7f
+    assert (enc[amax >= 1e-4] == 0x7e).all()
+    # an all-zero group: payload 0, scale = 1e-4 / 448 in fp32
+    assert (qb[0] == 0).all()
+    expected = (torch.tensor(1e-4, dtype=torch.float32) / torch.tensor(448.0, dtype=torch.float32))
+    assert (s[0] == expected).all()
+    # scale is a true division, not a multiplication by the rounded reciprocal, wherever the two differ
+    by_recip = amax.clamp(min=1e-4) * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+    differs = by_recip != s
+    assert differs.any(), "sample too small to separate division from reciprocal-multiply"
+    assert torch.equal(s, amax.clamp(min=1e-4) / 448.0)
+    # nothing saturates: |x| * (448/amax) never reaches the NaN code
+    assert ((q.view(torch.uint8) & 0x7f) != 0x7f).all()
+    # dequantised values are within half an e4m3 step (relative 2^-4) of the input, or below the subnormal step
+    back = oracle.per_token_cast_back(q, s).float()
+    err = (back - x.float()).abs()
+    tol = torch.maximum(x.float().abs() * 2.0 ** -4, (s * 2.0 ** -9).repeat_interleave(128, dim=1)) + x.float().abs() * 2.0 ** -7
+    assert (err <= tol).all()
+
+
+def test_ordered_sum_matches_c_restatement(cref):
+    g = torch.Generator().manual_seed(3)
+    rows = (torch.randn((7, 96), generator=g) * torch.tensor([1e4, 1, 1e-3, -1e4, 5, 1e-2, 3]).unsqueeze(1)).to(torch.bfloat16)
+    init = torch.randn(96, generator=g)
+    want = oracle.ordered_accumulate(rows.unsqueeze(0), init.unsqueeze(0))[0]
+    rin = rows.view(torch.int16).numpy().copy()
+    out = np.zeros(96, dtype=np.uint16)
+    ini = init.numpy().copy()
+    cref.oracle_ordered_sum_bf16(rin.ctypes.data, 7, 96, ini.ctypes.data, out.ctypes.data)
+    assert torch.equal(want.view(torch.int16), torch.from_numpy(out.view(np.int16)))
+    # the reference's bf16 known answer: contributions are bf16 first (301 -> 300, 302 -> 302), sum 602 -> bf16 600
+    data = torch.tensor([[301.0], [302.0]]).to(torch.bfloat16)
+    assert float(oracle.ordered_accumulate(data.unsqueeze(0))[0, 0]) == 600.0

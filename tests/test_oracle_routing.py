@@ -1,0 +1,334 @@
+"""Pins the routing part of the oracle on the CPU: layout, dispatch placement, combine order, low latency.
+
+Evidence used: brute-force pure-Python restatements written as plain loops (no shared code with the
+oracle), the reference's literal two-rank cases and known answers (tests/golden/two_rank_cases.json),
+the reference's own host-compilable combine reduction (oracle/_ref, when built), and invariants.
+"""
+import ctypes
+import os
+
+import pytest
+import torch
+
+import routing_cases as rc
+import routing_oracle as oracle
+import world
+
+G = world.load_golden()
+E, R, H, M = G["num_experts"], G["num_ranks"], G["hidden"], G["capacity"]
+
+
+# ---------------------------------------------------------------- layout
+def brute_layout(idx, num_experts, num_ranks):
+    T, K = idx.shape
+    per = num_experts // num_ranks
+    per_rank, per_expert = [0] * num_ranks, [0] * num_experts
+    member = [[False] * num_ranks for _ in range(T)]
+    for t in range(T):
+        for k in range(K):
+            e = int(idx[t, k])
+            if e < 0:
+                continue
+            per_expert[e] += 1
+            member[t][e // per] = True
+        for r in range(num_ranks):
+            per_rank[r] += int(member[t][r])
+    return per_rank, per_expert, member
+
+
+@pytest.mark.parametrize("T,K,num_experts,num_ranks,masked", [(0, 2, 8, 2, 0.0), (1, 1, 4, 4, 0.0), (33, 4, 16, 4, 0.3),
+                                                             (70, 3, 12, 3, 0.1), (50, 8, 8, 8, 0.0), (9, 2, 6, 1, 0.5)])
+def test_layout_brute_force(T, K, num_experts, num_ranks, masked):
+    c = rc.small("l", max(T, 1), 8, num_experts, num_ranks, min(K, num_experts), seed=T + K, masked_ratio=masked)
+    idx = c.topk_idx[:T]
+    a, b, m = oracle.layout(idx, num_experts, num_ranks)
+    ra, rb, rm = brute_layout(idx, num_experts, num_ranks)
+    assert a.tolist() == ra and b.tolist() == rb and m.tolist() == rm
+    assert a.dtype == torch.int32 and b.dtype == torch.int32 and m.dtype == torch.bool
+
+
+def test_layout_literal_rows():
+    idx = torch.tensor([[-1, -1], [0, 1], [2, 3], [1, 2], [3, -1]])       # E=4, R=2
+    a, b, m = oracle.layout(idx, 4, 2)
+    assert a.tolist() == [2, 3]            # token 1 counts once for rank 0 although two experts live there
+    assert b.tolist() == [1, 2, 2, 2]
+    assert m.tolist() == [[False, False], [True, False], [False, True], [True, True], [False, True]]
+
+
+# ---------------------------------------------------------------- dispatch
+def brute_dispatch(x, idx, w, num_experts, num_ranks, rank, cap, A, expand):
+    """Loops only.  Returns dict of python lists."""
+    T, K = idx.shape
+    per = num_experts // num_ranks
+    rows = []                                  # (dst, token, master lane)
+    slots = [[-1] * K for _ in range(T)]
+    for d in range(num_ranks):
+        n = 0
+        for t in range(T):
+            lanes = [k for k in range(K) if int(idx[t, k]) >= 0 and int(idx[t, k]) // per == d]
+            if lanes:
+                slots[t][max(lanes)] = rank * cap + n
+                rows.append((d, t, max(lanes)))
+                n += 1
+    counts = [0] * num_experts
+    for t in range(T):
+        for k in range(K):
+            if int(idx[t, k]) >= 0:
+                counts[int(idx[t, k])] += 1
+    aligned = [(c + A - 1) // A * A for c in counts]
+    starts = [sum(aligned[:e]) for e in range(num_experts)]
+    meta = [[rank * cap + t, rank * K + ml] + [-1] * K for (d, t, ml) in rows]
+    out = {"slots": slots, "counts": counts, "aligned": aligned,
+           "psum_rank": [sum(1 for r in rows if r[0] <= d) for d in range(num_ranks)]}
+    if not expand:
+        out["recv_x"] = [x[t].tolist() for (d, t, ml) in rows]
+        out["recv_idx"] = [[(int(idx[t, k]) - d * per) if int(idx[t, k]) >= 0 and int(idx[t, k]) // per == d else -1
+                            for k in range(K)] for (d, t, ml) in rows]
+        out["recv_w"] = [w[t].tolist() for (d, t, ml) in rows]
+        out["psum_expert"] = [sum(aligned[:e + 1]) for e in range(num_experts)]
+    else:
+        total = sum(aligned)
+        ex, ew, valid = [None] * total, [None] * total, [False] * total
+        fill = [0] * num_experts
+        row_of = {(d, t): i for i, (d, t, ml) in enumerate(rows)}
+        for t in range(T):
+            for k in range(K):
+                e = int(idx[t, k])
+                if e < 0:
+                    continue
+                r = starts[e] + fill[e]
+                fill[e] += 1
+                ex[r], ew[r], valid[r] = x[t].tolist(), float(w[t, k]), True
+                meta[row_of[(e // per, t)]][2 + k] = r
+        out.update(ex=ex, ew=ew, valid=valid, psum_expert=[starts[e] + counts[e] for e in range(num_experts)])
+    out["meta"] = meta
+    return out
+
+
+@pytest.mark.parametrize("seed,T,K,num_experts,num_ranks,A,expand,rank", [
+    (1, 40, 3, 12, 3, 1, False, 0), (2, 40, 3, 12, 3, 4, True, 2), (3, 17, 8, 16, 8, 1, False, 5),
+    (4, 64, 4, 8, 2, 16, True, 1), (5, 5, 2, 4, 1, 1, True, 0), (6, 30, 6, 64, 8, 128, False, 7)])
+def test_dispatch_brute_force(seed, T, K, num_experts, num_ranks, A, expand, rank):
+    c = rc.small("d", T, 8, num_experts, num_ranks, K, seed=seed, masked_ratio=0.2, M=T + 3)
+    r = oracle.dispatch(c.x, c.topk_idx, c.topk_weights, num_experts, num_ranks, rank, c.M, expert_alignment=A, do_expand=expand)
+    b = brute_dispatch(c.x.float(), c.topk_idx, c.topk_weights, num_experts, num_ranks, rank, c.M, A, expand)
+    assert r.dst_buffer_slot_idx.tolist() == b["slots"]
+    assert r.num_unaligned_recv_tokens_per_expert.tolist() == b["counts"]
+    assert r.num_recv_tokens_per_expert_list == b["aligned"]
+    assert r.psum_num_recv_tokens_per_scaleup_rank.tolist() == b["psum_rank"]
+    assert r.psum_num_recv_tokens_per_expert.tolist() == b["psum_expert"]
+    assert r.recv_src_metadata.tolist() == b["meta"]
+    assert r.num_expanded_tokens == sum(b["aligned"])
+    if not expand:
+        assert r.recv_x.float().tolist() == b["recv_x"]
+        assert r.recv_topk_idx.tolist() == b["recv_idx"]
+        assert r.recv_topk_weights.tolist() == b["recv_w"]
+    else:
+        assert r.expanded_row_is_valid.tolist() == b["valid"]
+        for i, ok in enumerate(b["valid"]):
+            if ok:
+                assert r.recv_x[i].float().tolist() == b["ex"][i] and float(r.recv_topk_weights[i]) == b["ew"][i]
+            else:
+                assert float(r.recv_x[i].float().abs().sum()) == 0.0 and float(r.recv_topk_weights[i]) == 0.0
+    # permutation invariants: every (token, destination) exactly once; payload rows are copies
+    assert r.num_recv_tokens == int(oracle.layout(c.topk_idx, num_experts, num_ranks)[2].sum())
+
+
+def _case_tensors(case, K):
+    weights = case.get("weights")
+    x, idx, w = world.stack_world(case["payloads"], case["routes"], weights, M, H, K)
+    counts = [len(r) for r in case["routes"]]
+    return x, idx, w, counts
+
+
+@pytest.mark.parametrize("name", list(G["dispatch_cases"]))
+def test_single_source_calls_compose_into_the_reference_world(name):
+    """The padded one-call world equals the restated refs.dispatch for every destination rank."""
+    case = G["dispatch_cases"][name]
+    K = len(case["routes"][1][0]) if case["routes"][1] else 2
+    x, idx, w, counts = _case_tensors(case, K)
+    w_full = w if w is not None else torch.zeros(idx.shape, dtype=torch.float32)
+    r = oracle.dispatch(x, idx, w_full, E, R, 0, R * M)
+    xs, idxs, ws = world.per_source(x, idx, w_full, M, R, counts)
+    ref = oracle.world_dispatch(xs, idxs, ws, M, E)
+    for d, (lo, hi) in enumerate(world.bucket_bounds(r.psum_num_recv_tokens_per_scaleup_rank)):
+        rx, ridx, rw, rsrc, rcnt = ref[d]
+        assert torch.equal(r.recv_x[lo:hi], rx)
+        assert torch.equal(r.recv_topk_idx[lo:hi], ridx)
+        assert torch.equal(r.recv_topk_weights[lo:hi], rw)
+        assert torch.equal(r.recv_src_metadata[lo:hi, 0], rsrc)       # source rank * M + token
+        assert hi - lo == int(rcnt.sum())
+
+
+@pytest.mark.parametrize("name", list(G["expanded_layout_cases"]))
+def test_expanded_layout_known_answers(name):
+    case = G["expanded_layout_cases"][name]
+    K = len(case["routes"][0][0])
+    _, idx, _ = world.stack_world(None, case["routes"], None, M, H, K)
+    r = oracle.dispatch(torch.zeros((R * M, H), dtype=torch.bfloat16), idx, None, E, R, 0, R * M,
+                        expert_alignment=case["expert_alignment"], do_expand=True)
+    per = E // R
+    for d in range(R):
+        aligned = r.num_recv_tokens_per_expert_list[d * per:(d + 1) * per]
+        actual = r.num_unaligned_recv_tokens_per_expert[d * per:(d + 1) * per].tolist()
+        exp = case["expected"][f"rank{d}"]
+        assert sum(aligned) == exp["rows"] and sum(aligned) - sum(actual) == exp["padding"]
+
+
+# ---------------------------------------------------------------- combine
+def contribution(rank, token, lane, variant=None):
+    if variant is not None:
+        first, second = variant[lane]
+        ident = 1 + rank * 16 + token * 4 + lane * 2
+        return [first, second, float(ident), float(ident + 1)]
+    b = 1 + rank * 16 + token * 4 + lane * 2
+    return [float(b + c) for c in range(H)]
+
+
+def combine_world(routes, K, do_expand, multi_red, variant=None, weights=None, biases=None):
+    """Dispatch the world, build expert outputs by the reference's synthetic rule, combine, split per source."""
+    x, idx, w = world.stack_world(None, routes, weights, M, H, K)
+    r = oracle.dispatch(x, idx, w, E, R, 0, R * M, do_expand=do_expand)
+    per = E // R
+    if do_expand:
+        y = torch.zeros((r.num_expanded_tokens, H), dtype=torch.bfloat16)
+        for i in range(r.num_recv_tokens):
+            g = int(r.recv_src_metadata[i, 0])
+            for k in range(K):
+                row = int(r.recv_src_metadata[i, 2 + k])
+                if row >= 0:
+                    y[row] = torch.tensor(contribution(g // M, g % M, k, variant)).to(torch.bfloat16)
+    else:
+        y = torch.zeros((r.num_recv_tokens, H), dtype=torch.bfloat16)
+        bounds = world.bucket_bounds(r.psum_num_recv_tokens_per_scaleup_rank)
+        for d, (lo, hi) in enumerate(bounds):
+            for i in range(lo, hi):
+                g = int(r.recv_src_metadata[i, 0])
+                acc = torch.zeros(H)
+                for k in range(K):
+                    e = int(idx[g, k])
+                    if e >= 0 and e // per == d:
+                        acc = acc + torch.tensor(contribution(g // M, g % M, k, variant))
+                y[i] = acc.to(torch.bfloat16)
+    bias = None
+    if biases is not None:
+        bias = tuple(torch.tensor(b, dtype=torch.float32).to(torch.bfloat16).expand(R * M, H).contiguous() for b in biases)
+        bias = bias[0] if len(bias) == 1 else bias
+    out, out_w = oracle.combine(y, idx, r.recv_src_metadata, r.dst_buffer_slot_idx, r.psum_num_recv_tokens_per_scaleup_rank,
+                                E, R, 0, R * M, topk_weights=r.recv_topk_weights, bias=bias, do_expand=do_expand,
+                                allow_multiple_reduction=multi_red)
+    return out.float(), out_w
+
+
+def test_combine_reference_fixture():
+    fx = G["combine"]["reference_fixture"]
+    for do_expand, multi in ((False, True), (True, True), (True, False)):
+        out, _ = combine_world(fx["routes"], 2, do_expand, multi)
+        assert out[0:2].tolist() == fx["expected"]["rank0"]
+        assert out[M:M + 1].tolist() == fx["expected"]["rank1"]
+
+
+def test_combine_order_sensitive_fixture():
+    fx = G["combine"]["ordering"]
+    routes = [[fx["route"]], []]
+    out, _ = combine_world(routes, 3, True, False, variant=fx["lane_columns"])
+    assert out[0].tolist() == fx["canonical"]
+    # adding the same lanes in the opposite order gives the other documented answer: the order is observable
+    cols = torch.tensor([contribution(0, 0, k, fx["lane_columns"]) for k in range(3)]).to(torch.bfloat16)
+    # (the reference reverses lanes inside each contributor rank: lane 0 | lanes 2, 1; or ranks: lanes 1, 2 | lane 0)
+    assert oracle.ordered_accumulate(cols[[0, 2, 1]].unsqueeze(0))[0].float().tolist() == fx["lane_reversed"]
+    assert oracle.ordered_accumulate(cols[[1, 2, 0]].unsqueeze(0))[0].float().tolist() == fx["rank_reversed"]
+
+
+def test_combine_weights_and_biases():
+    fx = G["combine"]["weight_bias"]
+    out, out_w = combine_world([fx["weight_route"], []], 2, False, True, weights=[fx["weights"], []])
+    assert out[0].tolist() == fx["activation_ignores_weight"]          # weights never scale activations
+    assert out_w[0].tolist() == fx["restored_weights"]                 # masked lane comes back as 0
+    out, _ = combine_world([fx["bias_route"], []], 2, False, True, biases=fx["biases"])
+    assert out[0].tolist() == fx["bias_once"]                          # each bias added exactly once
+    out, _ = combine_world([[[-1, -1]], []], 2, False, True, biases=fx["biases"])
+    assert out[0].tolist() == [5.0] * H                                # no valid expert: the bias sum
+
+
+def test_combine_partial_sums_round_to_bf16_per_rank():
+    # two lanes on one rank: their fp32 sum is rounded to bf16 before it meets the other rank's row
+    idx = torch.tensor([[0, 1, 2]])                                    # E=4, R=2: lanes 0,1 -> rank 0, lane 2 -> rank 1
+    y = torch.tensor([[[256.0], [1.0], [1.0]]]).to(torch.bfloat16)    # 257 is not a bf16 value
+    grouped = oracle.combine_from_lanes(y, idx, 4, 2, reduce_in_rank=True)
+    flat = oracle.combine_from_lanes(y, idx, 4, 2, reduce_in_rank=False)
+    assert float(grouped[0, 0]) == 256.0       # bf16(256+1) = 256, then 256+1 = 257 -> 256 (ties to even)
+    assert float(flat[0, 0]) == 258.0          # 256+1+1 = 258 exactly representable
+
+
+def test_combine_matches_reference_cpp_reduction():
+    """oracle/_ref/libcombine_ref.so is the reference's own combine_reduce_origin_records
+    (csrc/backends/ascend/elastic/combine_state.hpp:317-390).  It adds contributions in (contributor rank,
+    lane) order; with lanes sorted by expert that is plain lane order, the order of the expanded layout
+    without multiple reduction."""
+    path = os.path.join(os.path.dirname(os.path.abspath(oracle.__file__)), "_ref", "libcombine_ref.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    lib = ctypes.CDLL(path)
+    lib.ref_combine_reduce_column.restype = ctypes.c_float
+    g = torch.Generator().manual_seed(21)
+    num_experts, num_ranks, K, hidden = 16, 4, 6, 8
+    for trial in range(200):
+        route = torch.sort(torch.randperm(num_experts, generator=g)[:K]).values
+        route = torch.where(torch.rand(K, generator=g) < 0.2, torch.full_like(route, -1), route)
+        scale = 10.0 ** torch.randint(-3, 8, (K, 1), generator=g).float()
+        y = (torch.randn((K, hidden), generator=g) * scale).to(torch.bfloat16)
+        y[route < 0] = 0
+        want = oracle.combine_from_lanes(y.unsqueeze(0), route.unsqueeze(0), num_experts, num_ranks, reduce_in_rank=False)[0]
+        per = num_experts // num_ranks
+        lanes, offsets, counts, acts = [], [], [], []
+        for r in range(num_ranks):
+            offsets.append(len(lanes))
+            mine = [k for k in range(K) if int(route[k]) >= 0 and int(route[k]) // per == r]
+            counts.append(len(mine))
+            for k in mine:
+                lanes.append(k)
+                acts.extend(y[k].float().tolist())
+        arr_i = lambda v: (ctypes.c_int * max(len(v), 1))(*v)
+        acts_c = (ctypes.c_float * max(len(acts), 1))(*acts)
+        route_c = (ctypes.c_int64 * K)(*route.tolist())
+        for col in range(hidden):
+            got = lib.ref_combine_reduce_column(num_ranks, arr_i(offsets), arr_i(counts), arr_i(lanes), acts_c, hidden,
+                                                route_c, K, num_experts, col, ctypes.c_float(0.0), ctypes.c_float(0.0))
+            got_bf16 = torch.tensor([got], dtype=torch.float32).to(torch.bfloat16)
+            assert got_bf16.view(torch.int16).item() == want[col].view(torch.int16).item() or \
+                (float(got_bf16) == 0.0 and float(want[col]) == 0.0), (trial, col)
+
+
+# ---------------------------------------------------------------- low latency
+def test_low_latency_invariants():
+    Rr, T, Hh, Ee, K, Mm = 4, 20, 256, 16, 4, 24
+    x, idx, w = rc.c5_sources(seed=1, R=Rr, T=T, H=Hh, E=Ee, K=K)
+    idx[0, 3] = -1
+    for dst in range(Rr):
+        px, ps, cnt, info, rng = oracle.ll_dispatch(list(x), list(idx), Mm, Ee, Rr, dst, use_fp8=True)
+        per = Ee // Rr
+        begin, n = rng >> 32, rng & 0xFFFFFFFF
+        for le in range(per):
+            e = dst * per + le
+            assert int(cnt[le]) == int((idx == e).sum())                       # count = number of matches
+            assert int(n[le].sum()) == int(cnt[le])                            # ranges partition the rows
+            for s in range(Rr):
+                b, m = int(begin[le, s]), int(n[le, s])
+                toks = info[le, b:b + m].tolist()
+                assert toks == sorted(toks) and all(e in idx[s, t].tolist() for t in toks)
+                q, sc = oracle.per_token_cast_to_fp8(x[s][toks]) if m else (None, None)
+                if m:
+                    assert torch.equal(px[le, b:b + m].view(torch.uint8), q.view(torch.uint8)) and torch.equal(ps[le, b:b + m], sc)
+        # weighted combine of "expert output = dequantised input": out ~= x * sum of weights of lanes on dst
+        y = torch.zeros((per, Rr * Mm, Hh), dtype=torch.bfloat16)
+        for le in range(per):
+            c = int(cnt[le])
+            y[le, :c] = oracle.per_token_cast_back(px[le, :c], ps[le, :c])
+        for s in range(Rr):
+            out = oracle.ll_combine(y, idx[s], w[s], info, rng, s, Ee, Rr, dst).float()
+            on_dst = ((idx[s] >= dst * per) & (idx[s] < (dst + 1) * per)).float()
+            want = x[s].float() * (w[s] * on_dst).sum(dim=1, keepdim=True)
+            assert not torch.isnan(out).any()
+            diff = 1 - 2 * ((out + 1) * (want + 1)).double().sum() / ((out + 1) ** 2 + (want + 1) ** 2).double().sum()
+            assert float(diff) < 9e-4                                           # bound used by tests/legacy/test_low_latency.py:178-181

@@ -21,7 +21,10 @@ namespace deep_ep_hip {
 
 namespace {
 
-constexpr int kThreads = 256;
+#ifndef DEEP_EP_HIP_MOVE_THREADS
+#define DEEP_EP_HIP_MOVE_THREADS 256
+#endif
+constexpr int kThreads = DEEP_EP_HIP_MOVE_THREADS;
 constexpr int kWavesPerBlock = kThreads / kWaveSize;
 
 // Per-lane routing state of one token, lanes [0, K) meaningful.
@@ -121,8 +124,51 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
 }
 
 // Token-level metadata, written once per token (by the wave that owns column tile 0).
+//
+// Compact layout with K <= 15: a destination row's recv_topk_idx (2 dwords per lane), recv_topk_weights and
+// recv_src_metadata entries go out in ONE dword store instruction: wave lanes take the roles
+//   [0, 2K) index dwords | [2K, 3K) weights | [3K, 4K + 2) metadata columns,
+// each role reading the routing lane it needs through a shuffle done once per token.
 __device__ __forceinline__ void write_token_metadata(const MoveParams& p, const Route& r, int t, int lane) {
     uint64_t masters = __ballot(r.row_c >= 0);
+    const int K = p.K;
+    if (!p.do_expand && 4 * K + 2 <= kWaveSize) {
+        int src;           // routing lane this wave lane reports on
+        if (lane < 2 * K) src = lane >> 1;
+        else if (lane < 3 * K) src = lane - 2 * K;
+        else src = lane - 3 * K - 2;                       // metadata columns 2.. (negative for columns 0 and 1)
+        const int src_c = src < 0 ? 0 : (src >= K ? 0 : src);
+        const int e_src = __shfl(r.e, src_c, kWaveSize);
+        const int d_src = __shfl(r.d, src_c, kWaveSize);
+        const uint32_t w_src = __float_as_uint(__shfl(r.w, src_c, kWaveSize));
+        while (masters) {
+            const int j = __builtin_ctzll(masters);
+            masters &= masters - 1;
+            const int row = read_lane(r.row_c, j);
+            const int dj = read_lane(r.d, j);
+            if (row >= p.recv_capacity) {
+                if (lane == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
+                continue;
+            }
+            uint32_t* dst = nullptr;
+            uint32_t v = 0;
+            if (lane < 2 * K) {
+                const int local = (d_src == dj) ? e_src - dj * p.E_l : -1;
+                v = (lane & 1) ? (local < 0 ? 0xffffffffu : 0u) : uint32_t(local);
+                if (p.recv_topk_idx != nullptr) dst = reinterpret_cast<uint32_t*>(p.recv_topk_idx + int64_t(row) * K) + lane;
+            } else if (lane < 3 * K) {
+                v = w_src;
+                if (p.recv_topk_weights != nullptr)
+                    dst = reinterpret_cast<uint32_t*>(p.recv_topk_weights + int64_t(row) * K) + (lane - 2 * K);
+            } else if (lane < 4 * K + 2) {
+                const int col = lane - 3 * K;
+                v = col == 0 ? uint32_t(p.rank_idx * p.M + t) : col == 1 ? uint32_t(p.rank_idx * K + j) : 0xffffffffu;
+                if (!p.cached) dst = reinterpret_cast<uint32_t*>(p.recv_src_metadata + int64_t(row) * (K + 2)) + col;
+            }
+            if (dst != nullptr) *dst = v;
+        }
+        return;
+    }
     while (masters) {
         const int j = __builtin_ctzll(masters);
         masters &= masters - 1;
@@ -370,12 +416,11 @@ hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
         p.xcd_remap = v != nullptr ? atoi(v) : 0;
     }
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
-        // Column tile = kPairs * 1024 channels per wavefront.
+        // Column tile = kPairs * 1024 channels per wavefront.  Two pairs (2048 channels, 8 waves per SIMD)
+        // measured best at hidden 7168: 92.8 us per dispatch against 93.7 (4 pairs) and 96.9 (7 pairs, one
+        // wavefront per token).
         int pairs = tuning_override("DEEP_EP_HIP_CAST_PAIRS");
-        if (pairs == 0) {
-            const int segs = (p.H + 1023) / 1024;
-            pairs = segs <= 1 ? 1 : segs <= 2 ? 2 : segs <= 4 ? 4 : segs == 7 ? 7 : 4;
-        }
+        if (pairs == 0) pairs = p.H <= 1024 ? 1 : 2;
         switch (pairs) {
             case 1: return launch_cast<1>(p, stream);
             case 2: return launch_cast<2>(p, stream);

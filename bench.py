@@ -53,7 +53,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4"])
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--expanded", action="store_true", help="expert-major (expanded) receive layout")
     ap.add_argument("--bf16", action="store_true", help="BF16 dispatch instead of the fused FP8 cast")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -78,6 +78,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.workload == "C5":
+        print(json.dumps(bench_low_latency(args, torch, rc, _abi, dev)))
+        return
     case = {"C2": rc.c2, "C3": rc.c3, "C4": rc.c4}[args.workload]()
     T, H, K, E, R, M = case.T, case.H, case.K, case.E, case.R, case.M
     if args.routing == "sequential":
@@ -251,6 +254,72 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens, fp8, expanded)
     print(json.dumps(result))
+
+
+def bench_low_latency(args, torch, rc, _abi, dev):
+    """C5: low-latency decode.  Destination rank 0 of 8 receives from all 8 logical source ranks (128 tokens each,
+    hidden 7168, top-8 of 256): FP8 dispatch into [32, 1024, 7168] packed buffers, weighted BF16 combine back."""
+    R, T, H, E, K, M = 8, 128, 7168, 256, 8, 128
+    E_l, rows = E // R, R * M
+    x_cpu, idx_cpu, w_cpu = rc.c5_sources(seed=0, R=R, T=T, H=H, E=E, K=K)
+    x, idx, w = x_cpu.to(dev), idx_cpu.to(dev), w_cpu.to(dev)
+    n_e = int(((idx_cpu >= 0) & (idx_cpu < E_l)).sum())            # (token, lane) pairs that land on rank 0
+    px = torch.empty((E_l, rows, H), dtype=torch.float8_e4m3fn, device=dev)
+    ps = torch.empty((E_l, H // 128, rows), dtype=torch.float32, device=dev)
+    cnt = torch.empty(E_l, dtype=torch.int32, device=dev)
+    info = torch.empty((E_l, rows), dtype=torch.int32, device=dev)
+    rng = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
+    y = torch.randn((E_l, rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)
+    out = torch.empty((R, T, H), dtype=torch.bfloat16, device=dev)
+    ws = torch.zeros(max(_abi.lib.deep_ep_hip_ll_workspace_bytes(R, T, K, E_l), 4096), dtype=torch.uint8, device=dev)
+    d = _abi.LLDispatchArgs()
+    d.use_fp8, d.num_src_ranks, d.src_rank_begin, d.src_token_stride = 1, R, 0, T
+    d.hidden, d.num_topk, d.num_experts, d.expert_begin, d.num_local_experts = H, K, E, 0, E_l
+    d.num_ranks, d.num_max_dispatch_tokens_per_rank = R, M
+    d.x, d.topk_idx = x.data_ptr(), idx.data_ptr()
+    d.packed_recv_x, d.packed_recv_x_scales, d.packed_recv_count = px.data_ptr(), ps.data_ptr(), cnt.data_ptr()
+    d.packed_recv_src_info, d.packed_recv_layout_range = info.data_ptr(), rng.data_ptr()
+    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    c = _abi.LLCombineArgs()
+    c.num_src_ranks, c.src_rank_begin, c.src_token_stride = R, 0, T
+    c.hidden, c.num_topk, c.num_experts, c.expert_begin, c.num_local_experts, c.num_ranks = H, K, E, 0, E_l, R
+    c.num_max_dispatch_tokens_per_rank = M
+    c.x, c.topk_idx, c.topk_weights = y.data_ptr(), idx.data_ptr(), w.data_ptr()
+    c.packed_recv_src_info, c.packed_recv_layout_range, c.combined_x = info.data_ptr(), rng.data_ptr(), out.data_ptr()
+    c.workspace, c.workspace_bytes = ws.data_ptr(), ws.numel()
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+
+    def dispatch():
+        _abi.check(_abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(d), sp), "ll dispatch")
+
+    def combine():
+        _abi.check(_abi.lib.deep_ep_hip_launch_ll_combine(ctypes.byref(c), sp), "ll combine")
+
+    def timed(fn, iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(iters):
+            fn()
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters
+
+    for _ in range(args.warmup):
+        dispatch(); combine()
+    torch.cuda.synchronize()
+    step_us = timed(lambda: (dispatch(), combine()), args.steps)
+    d_us, c_us = timed(dispatch, max(args.steps, 20)), timed(combine, max(args.steps, 20))
+    d_bytes = R * T * H * 2 + R * T * K * 8 + n_e * (H + (H // 128) * 4 + 4) + E_l * (4 + R * 8)
+    c_bytes = n_e * H * 2 + R * T * K * 12 + R * T * H * 2
+    return {"metric": "low-latency dispatch+combine us/call, 8 sources x 128 tokens x 7168, top-8 of 256, destination rank 0",
+            "value": round(step_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(step_us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "fp8_e4m3 dispatch / bf16 weighted combine", "data": "synthetic",
+            "config": {"workload": f"C5: R={R} T={T} H={H} E={E} K={K} M={M}, rows on rank 0: {n_e}"},
+            "us_per_call": {"ll_dispatch": round(d_us, 2), "ll_combine": round(c_us, 2)},
+            "achieved_gbs": {"ll_dispatch": round(d_bytes / d_us * 1e-3, 1), "ll_combine": round(c_bytes / c_us * 1e-3, 1)},
+            "algorithmic_bytes": {"ll_dispatch": d_bytes, "ll_combine": c_bytes}}
 
 
 def cpu_baseline(case, sample_tokens, fp8, expanded):

@@ -74,10 +74,10 @@ __device__ __forceinline__ void accumulate_rows(float (&acc)[kVecs][8], uint64_t
 template <int kVecs>
 __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p) {
     const int lane = threadIdx.x & 63;
-    const int64_t work = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-    if (work >= int64_t(p.T) * p.tiles) return;
-    const int t = int(work / p.tiles);
-    const int tile = int(work - int64_t(t) * p.tiles);
+    const unsigned work = wave_work_index(blockIdx.x, kWavesPerBlock);
+    if (work >= unsigned(p.T) * unsigned(p.tiles)) return;
+    const int t = int(work / unsigned(p.tiles));
+    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
     const int row_bytes = p.H * 2;
 
     // Biases first: their loads do not depend on the routing metadata.
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
         if (raw >= 0 && raw < p.E) e = int(raw);
         const int v = p.slot[int64_t(t) * p.K + lane];
         if (e >= 0) {
-            d = e / p.E_l;
+            d = small_div(e, 1.0f / float(p.E_l));
             if (v >= 0) {
                 row_c = (d > 0 ? p.psum_rank[d - 1] : 0) + (v - p.rank_idx * p.M);
                 if (!p.do_expand && row_c >= p.num_x_rows) {

@@ -130,6 +130,18 @@ __device__ __forceinline__ unsigned xcd_contiguous_block(unsigned block, unsigne
     return (block % kXcds) * per + block / kXcds;
 }
 
+// Index of this wavefront's work item, as a wave-uniform 32-bit value (kept in scalar registers, so the
+// divisions that split it into (token, tile) are short 32-bit sequences instead of per-lane 64-bit ones).
+__device__ __forceinline__ unsigned wave_work_index(unsigned block, unsigned waves_per_block) {
+    return block * waves_per_block + unsigned(__builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)));
+}
+
+// x / d for 0 <= x < 2^20 and 1 <= d <= 2^16 through a float reciprocal: (x + 0.5) / d is at least 0.5 / d
+// away from an integer while the float error stays below 2^-23 * x / d, so truncation is exact.
+__device__ __forceinline__ int small_div(int x, float rcp_d) {
+    return int((float(x) + 0.5f) * rcp_d);
+}
+
 // Agent-scope relaxed load/store that bypass the per-CU vector cache, for values another
 // workgroup of the same launch has just produced.
 __device__ __forceinline__ int load_agent(const int* p) {

@@ -55,7 +55,7 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
             epos = int(packed >> 16);
         }
     }
-    if (r.e >= 0) r.d = r.e / p.E_l;
+    if (r.e >= 0) r.d = small_div(r.e, 1.0f / float(p.E_l));
     else slot = -1;
     if (p.light) {
         // Exclusive prefix of the per-rank chunk counts in (rank, chunk) order: lane L scans entries
@@ -234,10 +234,10 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
     if (p.light && blockIdx.x == 0) publish_from_chunk_counts(p);
     const int lane = threadIdx.x & 63;
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
-    const int64_t work = int64_t(block) * kWavesPerBlock + (threadIdx.x >> 6);
-    if (work >= int64_t(p.T) * p.tiles) return;
-    const int t = int(work / p.tiles);
-    const int tile = int(work - int64_t(t) * p.tiles);
+    const unsigned work = wave_work_index(block, kWavesPerBlock);
+    if (work >= unsigned(p.T) * unsigned(p.tiles)) return;
+    const int t = int(work / unsigned(p.tiles));
+    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
 
     vec16 v[kVecs];
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
@@ -277,10 +277,10 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
     if (p.light && blockIdx.x == 0) publish_from_chunk_counts(p);
     const int lane = threadIdx.x & 63;
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
-    const int64_t work = int64_t(block) * kWavesPerBlock + (threadIdx.x >> 6);
-    if (work >= int64_t(p.T) * p.tiles) return;
-    const int t = int(work / p.tiles);
-    const int tile = int(work - int64_t(t) * p.tiles);
+    const unsigned work = wave_work_index(block, kWavesPerBlock);
+    if (work >= unsigned(p.T) * unsigned(p.tiles)) return;
+    const int t = int(work / unsigned(p.tiles));
+    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
 
     vec16 in[kPairs][2];
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;

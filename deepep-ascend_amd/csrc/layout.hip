@@ -64,6 +64,7 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
 
     int e[KMAX], d[KMAX];
     int flags = 0;
+    const float rcp_experts_per_rank = 1.0f / float(p.E_l);
     const uint64_t my_bit = 1ull << lane;
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
         if (raw[k] >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
         else if (raw[k] >= 0) ev = int(raw[k]);
         e[k] = ev;
-        d[k] = ev >= 0 ? ev / p.E_l : -1;
+        d[k] = ev >= 0 ? small_div(ev, rcp_experts_per_rank) : -1;
         if (ev >= 0) {
             atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[(p.R + ev) * kWaves + wave]), my_bit);
             atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[d[k] * kWaves + wave]), my_bit);

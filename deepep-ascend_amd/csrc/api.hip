@@ -302,6 +302,191 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
     return DEEP_EP_HIP_OK;
 }
 
+int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_args* a, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    REQUIRE(a != nullptr, "args is NULL");
+    const bool with_topk = a->topk_idx != nullptr;
+    const int T = a->num_tokens, H = a->hidden, R = a->num_ranks;
+    REQUIRE(R >= 1 && R <= 64, "num_ranks must be in [1, 64] (got %d)", R);
+    REQUIRE(!a->cached || !with_topk, "a cached dispatch takes no topk_idx");
+    REQUIRE(with_topk == (a->topk_weights != nullptr), "topk_idx and topk_weights go together");
+    // Routing lanes: the top-k lanes, or one lane per rank.
+    const int K = with_topk ? a->num_topk : R;
+    const int E = with_topk ? a->num_experts : R;
+    REQUIRE(with_topk || R <= DEEP_EP_HIP_MAX_TOPK, "routing by is_token_in_rank alone supports up to %d ranks", DEEP_EP_HIP_MAX_TOPK);
+    if (int rc = check_routing_shape(T, K, E, R)) return rc;
+    const bool do_layout = (a->phases & DEEP_EP_HIP_PHASE_LAYOUT) != 0;
+    const bool do_move = (a->phases & DEEP_EP_HIP_PHASE_MOVE) != 0;
+    REQUIRE(do_layout || do_move, "phases selects nothing");
+    REQUIRE(!(a->cached && do_layout), "a cached dispatch has no layout phase");
+    REQUIRE(a->rank_idx >= 0 && a->rank_idx < R, "rank_idx %d outside [0, %d)", a->rank_idx, R);
+    REQUIRE(a->expert_alignment >= 1, "expert_alignment must be >= 1");
+    REQUIRE(a->num_channels >= 0, "num_channels must be >= 0");
+    REQUIRE(a->cached || T == 0 || with_topk || a->is_token_in_rank != nullptr, "is_token_in_rank is NULL");
+    REQUIRE(a->workspace != nullptr, "workspace is NULL");
+    REQUIRE(a->cached || a->psum_num_recv_tokens_per_rank != nullptr, "psum_num_recv_tokens_per_rank is NULL");
+    const WorkspaceLayout w = make_workspace_layout(T, K, E, R);
+    if (a->workspace_bytes < w.total_bytes)
+        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
+                    (unsigned long long)a->workspace_bytes, w.total_bytes);
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    int32_t* status = reinterpret_cast<int32_t*>(ws + w.status);
+
+    int elem_in = 2;
+    switch (a->payload) {
+        case DEEP_EP_HIP_PAYLOAD_BF16: break;
+        case DEEP_EP_HIP_PAYLOAD_FP8: elem_in = 1; break;
+        case DEEP_EP_HIP_PAYLOAD_CAST_FP8: break;
+        default: return fail(DEEP_EP_HIP_ERR_INVALID_ARGUMENT, "unknown payload kind %d", a->payload);
+    }
+    if (do_move) {
+        REQUIRE(H >= 1 && (int64_t(H) * elem_in) % 16 == 0 && int64_t(H) * elem_in < (int64_t(1) << 30),
+                "a row of x must be a multiple of 16 bytes (hidden %d, %d-byte elements)", H, elem_in);
+        REQUIRE(T == 0 || a->x != nullptr, "x is NULL");
+        REQUIRE(a->recv_capacity >= 0 && a->recv_capacity < (int64_t(1) << 31), "recv_capacity out of range");
+        REQUIRE(a->recv_x != nullptr || a->recv_capacity == 0, "recv_x is NULL");
+        REQUIRE(a->send_head != nullptr || T == 0, "send_head is NULL");
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8)
+            REQUIRE(a->num_scales >= 0 && (a->num_scales == 0 || T == 0 || (a->x_scales != nullptr && a->recv_x_scales != nullptr)),
+                    "x_scales / recv_x_scales is NULL");
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8)
+            REQUIRE(H % 128 == 0 && a->num_scales == H / 128 && (a->recv_x_scales != nullptr || T == 0),
+                    "the fused FP8 cast needs hidden %% 128 == 0, num_scales == hidden / 128 and recv_x_scales");
+        REQUIRE(!with_topk || a->recv_capacity == 0 || (a->recv_topk_idx != nullptr && a->recv_topk_weights != nullptr),
+                "recv_topk_idx / recv_topk_weights is NULL");
+    }
+
+    PublishParams pub{};
+    pub.R = R; pub.E = E; pub.A = a->expert_alignment; pub.do_expand = 0;
+    pub.psum_rank = a->psum_num_recv_tokens_per_rank;
+    pub.num_unaligned = with_topk ? a->num_recv_tokens_per_expert : nullptr;
+    pub.host_counts = a->host_counts;
+    pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
+    pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
+
+    const int chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
+    const int chunks_padded = (chunks + 3) / 4 * 4;
+    const int flat = R * chunks_padded;
+    const int flat_per = flat <= 256 ? 4 : flat <= 512 ? 8 : 16;
+    const bool light = do_layout && do_move && T > 0 && flat <= 1024 && (R + E) <= 512 &&
+                       getenv("DEEP_EP_HIP_NO_LIGHT_LAYOUT") == nullptr;
+
+    if (do_layout) {
+        LayoutParams p{};
+        p.topk_idx = a->topk_idx;
+        p.route_mask = with_topk ? nullptr : a->is_token_in_rank;
+        p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
+        p.light = light ? 1 : 0;
+        p.chunks_padded = chunks_padded;
+        p.pub = pub;
+        p.status = status;
+        p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
+        p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
+        p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
+        p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
+        hipError_t err = launch_layout_kernel(p, stream);
+        if (err != hipSuccess) return hip_fail(err, "intranode dispatch layout launch");
+
+        if (a->is_token_in_rank != nullptr && (a->rank_prefix_matrix != nullptr || a->channel_prefix_matrix != nullptr ||
+                                               a->recv_channel_prefix_matrix != nullptr)) {
+            IntranodePrefixParams q{};
+            q.mask = a->is_token_in_rank;
+            q.T = T; q.R = R; q.C = a->num_channels; q.rank_idx = a->rank_idx;
+            q.rank_prefix_matrix = a->rank_prefix_matrix;
+            q.channel_prefix_matrix = a->channel_prefix_matrix;
+            q.recv_channel_prefix_matrix = a->recv_channel_prefix_matrix;
+            REQUIRE(q.C >= 1 && q.C <= 8192, "num_channels must be in [1, 8192] when the channel matrices are requested");
+            err = launch_intranode_prefix(q, stream);
+            if (err != hipSuccess) return hip_fail(err, "intranode prefix launch");
+        }
+    }
+
+    if (do_move) {
+        MoveParams m{};
+        m.x = static_cast<const uint8_t*>(a->x);
+        m.sf = static_cast<const uint32_t*>(a->x_scales);
+        m.sf_ts = a->scale_token_stride; m.sf_hs = a->scale_hidden_stride;
+        m.num_sf_packs = a->num_scales;
+        m.topk_idx = a->topk_idx;
+        m.route_mask = (with_topk || a->cached) ? nullptr : a->is_token_in_rank;
+        m.topk_weights = a->topk_weights;
+        m.pos = reinterpret_cast<const uint32_t*>(ws + w.pos);
+        m.chunk_base = reinterpret_cast<const int32_t*>(ws + w.chunk_base);
+        m.expert_start = reinterpret_cast<const int32_t*>(ws + w.expert_start);
+        m.cached_slot = a->send_head;
+        m.dst_buffer_slot_idx = nullptr;
+        m.psum_rank = a->psum_num_recv_tokens_per_rank;
+        m.recv_src_metadata = nullptr;
+        m.recv_x = static_cast<uint8_t*>(a->recv_x);
+        m.recv_sf = static_cast<uint32_t*>(a->recv_x_scales);
+        m.rsf_ts = a->recv_scale_token_stride; m.rsf_hs = a->recv_scale_hidden_stride;
+        m.recv_topk_idx = with_topk ? a->recv_topk_idx : nullptr;
+        m.recv_topk_weights = with_topk ? a->recv_topk_weights : nullptr;
+        m.recv_capacity = a->recv_capacity;
+        m.expanded_capacity = 0;
+        m.T = T; m.H = H; m.K = K; m.E = E; m.R = R; m.E_l = E / R;
+        m.rank_idx = a->rank_idx; m.M = T > 0 ? T : 1;
+        m.cached = a->cached ? 1 : 0;
+        m.do_expand = 0;
+        m.payload = a->payload;
+        m.row_bytes = H * elem_in;
+        m.light = light ? 1 : 0;
+        m.chunks_padded = chunks_padded;
+        m.flat_per = flat_per;
+        m.chunk_counts_t = reinterpret_cast<const int32_t*>(ws + w.chunk_counts);
+        m.pub = pub;
+        m.status = status;
+        m.rank_lanes = with_topk ? 0 : 1;
+        m.slot_is_row = a->cached ? 1 : 0;
+        m.zero_nonlocal_w = 1;
+        m.send_head = a->cached ? nullptr : a->send_head;
+        m.recv_src_idx = a->cached ? nullptr : a->recv_src_idx;
+        hipError_t err = launch_dispatch_move(m, stream);
+        if (err != hipSuccess) return hip_fail(err, "intranode dispatch move launch");
+
+        if (a->fill_unused_topk_idx && with_topk && !a->cached) {
+            FillTailParams f{};
+            f.recv_topk_idx = a->recv_topk_idx;
+            f.total_rows = reinterpret_cast<const int32_t*>(ws + w.totals);
+            f.capacity = a->recv_capacity;
+            f.K = K;
+            err = launch_fill_tail(f, stream);
+            if (err != hipSuccess) return hip_fail(err, "intranode fill launch");
+        }
+    }
+    return DEEP_EP_HIP_OK;
+}
+
+int deep_ep_hip_launch_intranode_combine(const deep_ep_hip_intranode_combine_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    REQUIRE(a->num_tokens >= 0, "num_tokens must be >= 0");
+    REQUIRE(a->num_ranks >= 1 && a->num_ranks <= 64, "num_ranks must be in [1, 64] (got %d)", a->num_ranks);
+    REQUIRE(a->num_topk >= 0 && a->num_topk <= DEEP_EP_HIP_MAX_TOPK, "num_topk must be in [0, %d]", DEEP_EP_HIP_MAX_TOPK);
+    REQUIRE(a->hidden >= 1 && (int64_t(a->hidden) * 2) % 16 == 0, "hidden (%d) must give rows that are multiples of 16 bytes", a->hidden);
+    REQUIRE(a->num_x_rows >= 0 && a->num_x_rows < (int64_t(1) << 31), "num_x_rows out of range");
+    const bool any = a->num_tokens > 0;
+    REQUIRE(!any || (a->send_head != nullptr && a->combined_x != nullptr), "send_head / combined_x is NULL");
+    REQUIRE(!any || a->x != nullptr || a->num_x_rows == 0, "x is NULL");
+    REQUIRE(a->num_topk == 0 || a->topk_weights == nullptr || a->combined_topk_weights != nullptr, "combined_topk_weights is NULL");
+    REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
+    CombineParams p{};
+    p.x = static_cast<const uint8_t*>(a->x);
+    p.num_x_rows = a->num_x_rows;
+    p.topk_weights = a->topk_weights;
+    p.bias0 = static_cast<const uint8_t*>(a->bias_0);
+    p.bias1 = static_cast<const uint8_t*>(a->bias_1);
+    p.slot = a->send_head;
+    p.out = static_cast<uint8_t*>(a->combined_x);
+    p.out_w = a->num_topk > 0 ? a->combined_topk_weights : nullptr;
+    p.T = a->num_tokens; p.H = a->hidden; p.K = a->num_ranks; p.E = a->num_ranks; p.R = a->num_ranks; p.E_l = 1;
+    p.rank_mode = 1;
+    p.Kw = a->num_topk;
+    p.status = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a->workspace));
+    hipError_t err = launch_combine_kernel(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "intranode combine launch");
+    return DEEP_EP_HIP_OK;
+}
+
 size_t deep_ep_hip_ll_workspace_bytes(int num_src_ranks, int src_token_stride, int num_topk, int num_local_experts) {
     if (num_src_ranks < 1 || src_token_stride < 1 || num_topk < 1 || num_local_experts < 1) return 0;
     const size_t chunks = size_t(num_src_ranks) * ((size_t(src_token_stride) + kLayoutChunk - 1) / kLayoutChunk);

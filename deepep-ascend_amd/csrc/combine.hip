@@ -99,7 +99,29 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
 
     // Routing of this token: lanes [0, K).
     int e = -1, d = -1, row_c = -1, my_row = -1, erow = -1;
-    if (lane < p.K) {
+    if (p.rank_mode) {
+        // V1 handle: lane q < R reads the receive row of this token on rank q; rows are added in ascending
+        // rank order and the weights of all rows are summed (csrc/kernels/legacy/intranode.cu:940-1033).
+        if (lane < p.K) {
+            const int v = p.slot[int64_t(t) * p.K + lane];
+            if (v >= 0) {
+                if (v < p.num_x_rows) row_c = v;
+                else atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
+            }
+        }
+        const uint64_t rows_of_token = __ballot(row_c >= 0);      // taken with every lane active
+        if (tile == 0 && p.out_w != nullptr && lane < p.Kw) {
+            float w = 0.f;
+            uint64_t rows = rows_of_token;
+            while (rows) {
+                const int j = __builtin_ctzll(rows);
+                rows &= rows - 1;
+                const int row = read_lane(row_c, j);
+                if (p.topk_weights != nullptr) w += p.topk_weights[int64_t(row) * p.Kw + lane];
+            }
+            p.out_w[int64_t(t) * p.Kw + lane] = w;
+        }
+    } else if (lane < p.K) {
         const int64_t raw = p.topk_idx[int64_t(t) * p.K + lane];
         if (raw >= 0 && raw < p.E) e = int(raw);
         const int v = p.slot[int64_t(t) * p.K + lane];
@@ -114,7 +136,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
             }
         }
     }
-    for (int j = 0; j < p.K; ++j) {
+    for (int j = 0; j < p.K && !p.rank_mode; ++j) {
         const int dj = read_lane(d, j);
         const int rj = read_lane(row_c, j);
         if (d >= 0 && dj == d && rj >= 0) my_row = rj;
@@ -128,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
     }
 
     // Weights travel back to the lane that owns them.
-    if (tile == 0 && p.out_w != nullptr && lane < p.K) {
+    if (tile == 0 && p.out_w != nullptr && lane < p.K && !p.rank_mode) {
         float w = 0.f;
         if (p.topk_weights != nullptr) {
             if (p.do_expand) {

@@ -43,16 +43,25 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
     const int chunk = t / kLayoutChunk;
     int slot = -1, epos = -1;
     if (lane < p.K) {
-        const int64_t raw = p.topk_idx[int64_t(t) * p.K + lane];
-        if (raw >= 0 && raw < p.E) r.e = int(raw);
-        if (p.topk_weights != nullptr) r.w = p.topk_weights[int64_t(t) * p.K + lane];
-        if (p.cached) {
+        if (p.cached && p.rank_lanes) {
+            // V1 cached dispatch: send_head names the receive row of every (token, rank) pair
             const int v = p.cached_slot[int64_t(t) * p.K + lane];
-            slot = v >= 0 ? v - p.rank_idx * p.M : -1;
+            if (v >= 0) r.e = lane;
+            slot = v;
         } else {
-            const uint32_t packed = p.pos[int64_t(t) * p.K + lane];
-            slot = (packed & 0xffffu) == 0xffffu ? -1 : int(packed & 0xffffu);
-            epos = int(packed >> 16);
+            const int64_t raw = p.route_mask != nullptr
+                                    ? (p.route_mask[int64_t(t) * p.K + lane] != 0 ? int64_t(lane) : int64_t(-1))
+                                    : p.topk_idx[int64_t(t) * p.K + lane];
+            if (raw >= 0 && raw < p.E) r.e = int(raw);
+            if (p.topk_weights != nullptr) r.w = p.topk_weights[int64_t(t) * p.K + lane];
+            if (p.cached) {
+                const int v = p.cached_slot[int64_t(t) * p.K + lane];
+                slot = v >= 0 ? v - p.rank_idx * p.M : -1;
+            } else {
+                const uint32_t packed = p.pos[int64_t(t) * p.K + lane];
+                slot = (packed & 0xffffu) == 0xffffu ? -1 : int(packed & 0xffffu);
+                epos = int(packed >> 16);
+            }
         }
     }
     if (r.e >= 0) r.d = small_div(r.e, 1.0f / float(p.E_l));
@@ -100,11 +109,25 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
             slot = r.row_c - bucket_start;      // slot inside the destination bucket
         }
     } else if (r.e >= 0 && slot >= 0) {
-        if (!p.cached) slot += p.chunk_base[int64_t(chunk) * n + r.d];
-        r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
+        if (p.slot_is_row) {
+            r.row_c = slot;
+        } else {
+            if (!p.cached) slot += p.chunk_base[int64_t(chunk) * n + r.d];
+            r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
+        }
     }
     if (first_tile && !p.cached && lane < p.K && p.dst_buffer_slot_idx != nullptr)
         p.dst_buffer_slot_idx[int64_t(t) * p.K + lane] = (r.e >= 0 && slot >= 0) ? p.rank_idx * p.M + slot : -1;
+    if (first_tile && !p.cached && p.send_head != nullptr) {
+        // V1 handle: wave lane q < R reports the receive row of this token on rank q (-1: not sent there)
+        int row_on_rank = -1;
+        for (int j = 0; j < p.K; ++j) {
+            const int dj = read_lane(r.d, j);
+            const int rj = read_lane(r.row_c, j);
+            if (dj == lane && rj >= 0) row_on_rank = rj;
+        }
+        if (lane < p.R) p.send_head[int64_t(t) * p.R + lane] = row_on_rank;
+    }
 
     // Every valid lane learns the compact row of its destination rank from that rank's master lane.
     for (int j = 0; j < p.K; ++j) {
@@ -157,13 +180,15 @@ __device__ __forceinline__ void write_token_metadata(const MoveParams& p, const 
                 v = (lane & 1) ? (local < 0 ? 0xffffffffu : 0u) : uint32_t(local);
                 if (p.recv_topk_idx != nullptr) dst = reinterpret_cast<uint32_t*>(p.recv_topk_idx + int64_t(row) * K) + lane;
             } else if (lane < 3 * K) {
-                v = w_src;
+                v = (p.zero_nonlocal_w && d_src != dj) ? 0u : w_src;
                 if (p.recv_topk_weights != nullptr)
                     dst = reinterpret_cast<uint32_t*>(p.recv_topk_weights + int64_t(row) * K) + (lane - 2 * K);
             } else if (lane < 4 * K + 2) {
                 const int col = lane - 3 * K;
                 v = col == 0 ? uint32_t(p.rank_idx * p.M + t) : col == 1 ? uint32_t(p.rank_idx * K + j) : 0xffffffffu;
-                if (!p.cached) dst = reinterpret_cast<uint32_t*>(p.recv_src_metadata + int64_t(row) * (K + 2)) + col;
+                if (!p.cached && p.recv_src_metadata != nullptr)
+                    dst = reinterpret_cast<uint32_t*>(p.recv_src_metadata + int64_t(row) * (K + 2)) + col;
+                if (col == 0 && p.recv_src_idx != nullptr) p.recv_src_idx[row] = t;
             }
             if (dst != nullptr) *dst = v;
         }
@@ -181,9 +206,11 @@ __device__ __forceinline__ void write_token_metadata(const MoveParams& p, const 
         if (!p.do_expand && lane < p.K) {
             if (p.recv_topk_idx != nullptr)
                 p.recv_topk_idx[int64_t(row) * p.K + lane] = (r.d == dj) ? int64_t(r.e - dj * p.E_l) : int64_t(-1);
-            if (p.recv_topk_weights != nullptr) p.recv_topk_weights[int64_t(row) * p.K + lane] = r.w;
+            if (p.recv_topk_weights != nullptr)
+                p.recv_topk_weights[int64_t(row) * p.K + lane] = (p.zero_nonlocal_w && r.d != dj) ? 0.f : r.w;
         }
-        if (!p.cached && lane < p.K + 2) {
+        if (lane == 0 && p.recv_src_idx != nullptr) p.recv_src_idx[row] = t;
+        if (!p.cached && p.recv_src_metadata != nullptr && lane < p.K + 2) {
             int v;
             if (lane < p.K) v = (p.do_expand && r.d == dj) ? r.erow : -1;
             else if (lane == p.K) v = p.rank_idx * p.M + t;
@@ -380,6 +407,45 @@ __global__ __launch_bounds__(kThreads) void cast_kernel(const CastParams p) {
     if ((lane & 7) == 0 && group < groups && elem < p.H) p.scales[int64_t(t) * groups + group] = scale_inv;
 }
 
+// ---- V1 handle bookkeeping (csrc/kernels/legacy/intranode.cu:94-125): one workgroup per destination rank
+// counts the tokens of each channel (contiguous token range) that go there, then prefix-sums over channels ----
+__global__ __launch_bounds__(kThreads) void intranode_prefix_kernel(const IntranodePrefixParams p) {
+    extern __shared__ int channel_counts[];     // [C]
+    const int d = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int per_channel = (p.T + p.C - 1) / p.C;
+    for (int c = wave; c < p.C; c += kWavesPerBlock) {
+        const int begin = min(per_channel * c, p.T), end = min(begin + per_channel, p.T);
+        int count = 0;
+        for (int t = begin + lane; t < end; t += kWaveSize) count += p.mask[int64_t(t) * p.R + d] != 0 ? 1 : 0;
+        count = wave_inclusive_sum(count);
+        if (lane == kWaveSize - 1) channel_counts[c] = count;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int c = 0; c < p.C; ++c) {
+            if (p.recv_channel_prefix_matrix != nullptr) p.recv_channel_prefix_matrix[d * p.C + c] = run;
+            run += channel_counts[c];
+            if (p.channel_prefix_matrix != nullptr) p.channel_prefix_matrix[d * p.C + c] = run;
+            channel_counts[c] = run;
+        }
+    }
+    __syncthreads();
+    // Only this source rank sends in a one-GPU call: the prefix over source ranks steps once, at rank_idx.
+    const int total = p.C > 0 ? channel_counts[p.C - 1] : 0;
+    if (p.rank_prefix_matrix != nullptr)
+        for (int i = threadIdx.x; i < p.R; i += kThreads) p.rank_prefix_matrix[i * p.R + d] = i >= p.rank_idx ? total : 0;
+}
+
+// ---- rows of recv_topk_idx beyond the received ones read -1 (csrc/kernels/legacy/intranode.cu:535-545) ----
+__global__ __launch_bounds__(kThreads) void fill_tail_kernel(const FillTailParams p) {
+    const int64_t first = int64_t(*p.total_rows) * p.K;
+    const int64_t end = p.capacity * p.K;
+    for (int64_t i = first + int64_t(blockIdx.x) * kThreads + threadIdx.x; i < end; i += int64_t(gridDim.x) * kThreads)
+        p.recv_topk_idx[i] = -1;
+}
+
 size_t publish_lds_bytes(const MoveParams& p) {
     return p.light ? size_t(p.R + 3 * p.E + kWavesPerBlock) * sizeof(int) : 0;
 }
@@ -448,6 +514,20 @@ hipError_t launch_zero_padding(const PadParams& p, hipStream_t stream) {
     const int64_t waves = int64_t(p.E) * (p.A - 1);
     const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     hipLaunchKernelGGL(zero_padding_kernel, dim3(blocks), dim3(kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_intranode_prefix(const IntranodePrefixParams& p, hipStream_t stream) {
+    if (p.R == 0 || p.C == 0) return hipSuccess;
+    hipLaunchKernelGGL(intranode_prefix_kernel, dim3(p.R), dim3(kThreads), size_t(p.C) * sizeof(int), stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_tail(const FillTailParams& p, hipStream_t stream) {
+    if (p.capacity == 0 || p.K == 0) return hipSuccess;
+    const int64_t elems = p.capacity * p.K;
+    const unsigned blocks = unsigned(elems / kThreads < 1 ? 1 : (elems / kThreads > 1024 ? 1024 : elems / kThreads));
+    hipLaunchKernelGGL(fill_tail_kernel, dim3(blocks), dim3(kThreads), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -40,6 +40,7 @@ struct PublishParams {
 
 struct LayoutParams {
     const int64_t* topk_idx;
+    const uint8_t* route_mask;       // [T, R] bool: when set, lane r of token t is "rank r, if the mask says so" (K = E = R)
     int T, K, E, R, E_l;
     int light;            // 1: only count (transposed chunk counts); the move kernel finishes the job
     int chunks_padded;    // row length of the transposed chunk counts (light mode)
@@ -63,6 +64,7 @@ struct MoveParams {
     int64_t sf_ts, sf_hs;
     int num_sf_packs;
     const int64_t* topk_idx;
+    const uint8_t* route_mask;       // see LayoutParams
     const float* topk_weights;
     const uint32_t* pos;
     const int32_t* chunk_base;
@@ -90,6 +92,12 @@ struct MoveParams {
     const int32_t* chunk_counts_t;   // [R + E][chunks_padded]
     PublishParams pub;   // written by workgroup 0
     int32_t* status;
+    // V1 (intranode) conventions
+    int rank_lanes;          // routing lanes are ranks (mask routing or a cached send_head), K == R
+    int slot_is_row;         // cached_slot holds rows of the receive buffer, not rank * M + slot
+    int zero_nonlocal_w;     // weights of lanes routed to another rank are delivered as 0
+    int32_t* send_head;      // [T, R] out: receive row of token t on rank r, or -1
+    int32_t* recv_src_idx;   // [recv_capacity] out: source token of each receive row
 };
 
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream);
@@ -108,6 +116,26 @@ struct PadParams {
 
 hipError_t launch_zero_padding(const PadParams& p, hipStream_t stream);
 
+// V1 (intranode) handle bookkeeping computed from is_token_in_rank, and the -1 fill of unused recv_topk_idx rows.
+struct IntranodePrefixParams {
+    const uint8_t* mask;             // [T, R]
+    int T, R, C, rank_idx;
+    int32_t* rank_prefix_matrix;         // [R, R]
+    int32_t* channel_prefix_matrix;      // [R, C] inclusive over channels
+    int32_t* recv_channel_prefix_matrix; // [R, C] exclusive starts
+};
+
+hipError_t launch_intranode_prefix(const IntranodePrefixParams& p, hipStream_t stream);
+
+struct FillTailParams {
+    int64_t* recv_topk_idx;          // [capacity, K]
+    const int32_t* total_rows;       // device: rows in use
+    int64_t capacity;
+    int K;
+};
+
+hipError_t launch_fill_tail(const FillTailParams& p, hipStream_t stream);
+
 struct CombineParams {
     const uint8_t* x;
     int64_t num_x_rows;
@@ -125,6 +153,10 @@ struct CombineParams {
     int do_expand, multi_red;
     int tiles;
     int32_t* status;
+    // V1 (intranode) conventions: slot is send_head [T, R] holding receive rows; terms are added in ascending
+    // rank order; weights [rows, Kw] are summed over the token's rows.
+    int rank_mode;
+    int Kw;
 };
 
 hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream);

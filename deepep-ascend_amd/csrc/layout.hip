@@ -42,7 +42,11 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
 
     // All index loads are issued before anything that could alias them is stored.
     int64_t raw[KMAX];
-    if (KMAX == 8 && p.K == 8 && p.vec_idx) {
+    if (p.route_mask != nullptr) {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+            raw[k] = (active && k < p.K && p.route_mask[int64_t(t) * p.K + k] != 0) ? int64_t(k) : int64_t(-1);
+    } else if (KMAX == 8 && p.K == 8 && p.vec_idx) {
         if (active) {
             const vec16* src = reinterpret_cast<const vec16*>(p.topk_idx + int64_t(t) * 8);
             vec16 q[4];

@@ -173,13 +173,17 @@ class ElasticBuffer:
                 reasons.append("a received row did not fit the output tensors")
             raise RuntimeError(f"DeepEP HIP backend: {what}: " + "; ".join(reasons))
 
-    def _prologue(self, previous_event, allocate_on_comm_stream: bool, async_with_compute_stream: bool):
+    def _prologue(self, previous_event, allocate_on_comm_stream: bool, async_with_compute_stream: bool,
+                  v1_rules: bool = False):
         """Returns (compute_stream, run_stream).  The reference always runs on its comm stream
         (csrc/elastic/buffer.hpp:528-551); when nothing asks for overlap the same ordering is had,
         without two cross-stream waits, by running on the caller's stream."""
         compute_stream = torch.cuda.current_stream()
-        if previous_event is not None:
+        if previous_event is not None and not v1_rules:
             _host_assert(allocate_on_comm_stream, "allocate_on_comm_stream")
+        if v1_rules and allocate_on_comm_stream:
+            # csrc/legacy/buffer.hpp:507-510
+            _host_assert(previous_event is not None and async_with_compute_stream, "previous_event.has_value() and async")
         overlap = previous_event is not None or allocate_on_comm_stream or async_with_compute_stream
         if not overlap:
             return compute_stream, compute_stream
@@ -516,3 +520,235 @@ class ElasticBuffer:
         event = self._epilogue([topk_idx, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, workspace],
                                compute_stream, run_stream, allocate_on_comm_stream, async_finish)
         return num_tokens_per_rank, None, num_tokens_per_expert, is_token_in_rank, event
+
+    def intranode_dispatch(self, x: torch.Tensor, x_scales: Optional[torch.Tensor],
+                           topk_idx: Optional[torch.Tensor], topk_weights: Optional[torch.Tensor],
+                           num_tokens_per_rank: Optional[torch.Tensor], is_token_in_rank: torch.Tensor,
+                           num_tokens_per_expert: Optional[torch.Tensor], cached_num_recv_tokens: int,
+                           cached_rank_prefix_matrix: Optional[torch.Tensor],
+                           cached_channel_prefix_matrix: Optional[torch.Tensor],
+                           expert_alignment: int, num_worst_tokens: int, config,
+                           previous_event: Optional[EventHandle], async_finish: bool, allocate_on_comm_stream: bool,
+                           cached_send_head: Optional[torch.Tensor] = None):
+        """Argument order and the 11-tuple returned follow csrc/legacy/buffer.hpp:417-717.
+        `cached_send_head` (the handle's token -> receive-row map) is the one addition: on one GPU a
+        cached dispatch scatters through it instead of replaying per-channel queues."""
+        _host_assert(not self._destroyed, "buffer is destroyed")
+        cached_mode = cached_rank_prefix_matrix is not None
+        R = self.num_ranks
+        _host_assert(R <= 64, "num_ranks <= 64 for the V1 dispatch")
+        _host_assert(config.num_sms % 2 == 0, "config.num_sms % 2 == 0")
+        num_channels = config.num_sms // 2
+        _host_assert(x.dim() == 2 and x.is_cuda and x.is_contiguous(), "x.dim() == 2 and x.is_contiguous()")
+        num_tokens, hidden = x.shape
+        _host_assert((hidden * x.element_size()) % 16 == 0, "(x.size(1) * x.element_size()) % sizeof(int4) == 0")
+        _host_assert(is_token_in_rank.dtype == torch.bool and is_token_in_rank.dim() == 2 and
+                     is_token_in_rank.is_contiguous() and tuple(is_token_in_rank.shape) == (num_tokens, R),
+                     "is_token_in_rank is a contiguous bool [num_tokens, num_ranks]")
+        i32 = dict(dtype=torch.int32, device=self.device)
+        if cached_mode:
+            _host_assert(cached_channel_prefix_matrix is not None and cached_send_head is not None, "cached handle tensors")
+            _host_assert(tuple(cached_rank_prefix_matrix.shape) == (R, R) and cached_rank_prefix_matrix.dtype == torch.int32,
+                         "cached_rank_prefix_matrix is int32 [num_ranks, num_ranks]")
+            _host_assert(tuple(cached_channel_prefix_matrix.shape) == (R, num_channels) and
+                         cached_channel_prefix_matrix.dtype == torch.int32,
+                         "cached_channel_prefix_matrix is int32 [num_ranks, num_channels]")
+            _host_assert(tuple(cached_send_head.shape) == (num_tokens, R) and cached_send_head.dtype == torch.int32 and
+                         cached_send_head.is_contiguous(), "cached send_head is int32 [num_tokens, num_ranks]")
+            _host_assert(topk_idx is None and topk_weights is None, "a cached dispatch takes no top-k tensors")
+            num_experts = 0
+        else:
+            _host_assert(num_tokens_per_rank is not None and num_tokens_per_expert is not None,
+                         "num_tokens_per_rank and num_tokens_per_expert")
+            _host_assert(num_tokens_per_rank.dtype == torch.int32 and tuple(num_tokens_per_rank.shape) == (R,) and
+                         num_tokens_per_rank.is_contiguous(), "num_tokens_per_rank is int32 [num_ranks]")
+            _host_assert(num_tokens_per_expert.dtype == torch.int32 and num_tokens_per_expert.dim() == 1 and
+                         num_tokens_per_expert.is_contiguous(), "num_tokens_per_expert is int32 [num_experts]")
+            num_experts = num_tokens_per_expert.shape[0]
+            _host_assert(num_experts % R == 0, "num_tokens_per_expert.size(0) % num_ranks == 0")
+        _host_assert((topk_idx is None) == (topk_weights is None), "topk_idx.has_value() == topk_weights.has_value()")
+        num_topk = 0
+        if topk_idx is not None:
+            num_topk = topk_idx.shape[1]
+            _host_assert(num_experts > 0, "num_experts > 0")
+            _host_assert(topk_idx.dim() == 2 and topk_idx.is_contiguous() and topk_idx.dtype == topk_idx_t and
+                         topk_idx.shape[0] == num_tokens, "topk_idx is a contiguous [num_tokens, num_topk] tensor")
+            _host_assert(tuple(topk_weights.shape) == (num_tokens, num_topk) and topk_weights.is_contiguous() and
+                         topk_weights.dtype == torch.float32, "topk_weights is contiguous FP32 [num_tokens, num_topk]")
+            _host_assert(1 <= num_topk <= _abi.MAX_TOPK, f"1 <= num_topk <= {_abi.MAX_TOPK}")
+            _host_assert(num_experts <= _abi.MAX_EXPERTS, f"num_experts <= {_abi.MAX_EXPERTS}")
+        else:
+            _host_assert(R <= _abi.MAX_TOPK, f"num_ranks <= {_abi.MAX_TOPK} without top-k tensors")
+        num_scales, scale_ts, scale_hs = 0, 0, 0
+        if x_scales is not None:
+            _host_assert(x.element_size() == 1, "x.element_size() == 1")
+            _host_assert(x_scales.dtype in (torch.float32, torch.int32), "x_scales is FP32 or int32")
+            _host_assert(x_scales.dim() == 2 and x_scales.shape[0] == num_tokens and x_scales.is_cuda, "x_scales is [num_tokens, num_scales]")
+            num_scales, scale_ts, scale_hs = x_scales.shape[1], x_scales.stride(0), x_scales.stride(1)
+            payload = _abi.PAYLOAD_FP8
+        else:
+            _host_assert(x.dtype == torch.bfloat16, "x without scales must be BF16")
+            payload = _abi.PAYLOAD_BF16
+        if num_worst_tokens > 0:
+            _host_assert(cached_mode or topk_idx is not None, "num_worst_tokens needs the top-k tensors")
+
+        compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_finish, v1_rules=True)
+        route_lanes = num_topk if topk_idx is not None else R
+        route_experts = num_experts if topk_idx is not None else R
+        workspace = self._get_workspace(num_tokens, route_lanes, route_experts)
+        per_expert_list: List[int] = []
+        with torch.cuda.stream(run_stream):
+            args = _abi.IntranodeDispatchArgs()
+            args.payload, args.cached = payload, int(cached_mode)
+            args.num_tokens, args.hidden = num_tokens, hidden
+            args.num_topk, args.num_experts = num_topk, (num_experts if topk_idx is not None else 0)
+            args.num_ranks, args.rank_idx = R, self.rank_idx
+            args.num_channels, args.expert_alignment = num_channels, expert_alignment
+            args.x, args.x_scales = _abi.ptr(x), _abi.ptr(x_scales)
+            args.scale_token_stride, args.scale_hidden_stride, args.num_scales = scale_ts, scale_hs, num_scales
+            args.topk_idx, args.topk_weights = _abi.ptr(topk_idx), _abi.ptr(topk_weights)
+            args.is_token_in_rank = _abi.ptr(is_token_in_rank)
+            args.workspace, args.workspace_bytes = _abi.ptr(workspace), workspace.numel()
+            stream_ptr = run_stream.cuda_stream
+
+            if cached_mode:
+                num_recv_tokens = cached_num_recv_tokens
+                rank_prefix_matrix, channel_prefix_matrix = cached_rank_prefix_matrix, cached_channel_prefix_matrix
+                recv_channel_prefix_matrix = torch.empty((R, num_channels), **i32)
+                send_head = cached_send_head
+                recv_src_idx = torch.empty((num_recv_tokens,), **i32)
+                args.phases = _abi.PHASE_MOVE
+            else:
+                rank_prefix_matrix = torch.empty((R, R), **i32)
+                channel_prefix_matrix = torch.empty((R, num_channels), **i32)
+                recv_channel_prefix_matrix = torch.empty((R, num_channels), **i32)
+                send_head = torch.empty((num_tokens, R), **i32)
+                counts = torch.empty(R + max(num_experts, 1), **i32)
+                args.rank_prefix_matrix = _abi.ptr(rank_prefix_matrix)
+                args.channel_prefix_matrix = _abi.ptr(channel_prefix_matrix)
+                args.recv_channel_prefix_matrix = _abi.ptr(recv_channel_prefix_matrix)
+                args.psum_num_recv_tokens_per_rank = _abi.ptr(counts)
+                args.num_recv_tokens_per_expert = _abi.ptr(counts[R:]) if topk_idx is not None else 0
+                if num_worst_tokens > 0:
+                    num_recv_tokens = num_worst_tokens
+                    args.phases = _abi.PHASE_LAYOUT | _abi.PHASE_MOVE
+                    args.fill_unused_topk_idx = 1
+                else:
+                    # The reference spins on host-mapped counters here (csrc/legacy/buffer.hpp:580-600)
+                    args.phases = _abi.PHASE_LAYOUT
+                    _abi.check(_abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(args), stream_ptr),
+                               "intranode dispatch layout")
+                    if topk_idx is None:
+                        host = torch.cat([counts[:R], num_tokens_per_expert]).cpu()
+                    else:
+                        host = counts.cpu()
+                        self._read_and_clear_status("dispatch")
+                    num_recv_tokens = int(host[R - 1])
+                    per_expert = host[R:R + num_experts]
+                    per_expert_list = ((per_expert + (expert_alignment - 1)) // expert_alignment * expert_alignment).tolist()
+                    args.phases = _abi.PHASE_MOVE
+                recv_src_idx = torch.empty((num_recv_tokens,), **i32)
+
+            recv_x = torch.empty((num_recv_tokens, hidden), dtype=x.dtype, device=self.device)
+            recv_x_scales = recv_topk_idx = recv_topk_weights = None
+            if topk_idx is not None:
+                recv_topk_idx = torch.empty((num_recv_tokens, num_topk), dtype=topk_idx.dtype, device=self.device)
+                recv_topk_weights = torch.empty((num_recv_tokens, num_topk), dtype=torch.float32, device=self.device)
+            if x_scales is not None:
+                recv_x_scales = torch.empty((num_recv_tokens, num_scales), dtype=x_scales.dtype, device=self.device)
+                args.recv_scale_token_stride, args.recv_scale_hidden_stride = num_scales, 1
+            args.send_head = _abi.ptr(send_head)
+            args.recv_src_idx = _abi.ptr(recv_src_idx)
+            args.recv_x, args.recv_x_scales = _abi.ptr(recv_x), _abi.ptr(recv_x_scales)
+            args.recv_topk_idx, args.recv_topk_weights = _abi.ptr(recv_topk_idx), _abi.ptr(recv_topk_weights)
+            args.recv_capacity = num_recv_tokens
+            _abi.check(_abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(args), stream_ptr), "intranode dispatch")
+
+        event = self._epilogue(
+            [x, x_scales, topk_idx, topk_weights, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
+             rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_x, recv_x_scales, recv_src_idx,
+             recv_topk_idx, recv_topk_weights, send_head, workspace],
+            compute_stream, run_stream, allocate_on_comm_stream, async_finish)
+        return (recv_x, recv_x_scales, recv_topk_idx, recv_topk_weights, per_expert_list, rank_prefix_matrix,
+                channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, send_head, event)
+
+    def intranode_combine(self, x: torch.Tensor, topk_weights: Optional[torch.Tensor],
+                          bias_0: Optional[torch.Tensor], bias_1: Optional[torch.Tensor],
+                          src_idx: torch.Tensor, rank_prefix_matrix: torch.Tensor,
+                          channel_prefix_matrix: torch.Tensor, send_head: torch.Tensor, config,
+                          previous_event: Optional[EventHandle], async_finish: bool, allocate_on_comm_stream: bool):
+        """Argument order and the 3-tuple returned follow csrc/legacy/buffer.hpp:719-860."""
+        _host_assert(not self._destroyed, "buffer is destroyed")
+        R = self.num_ranks
+        _host_assert(x.dim() == 2 and x.is_cuda and x.is_contiguous() and x.dtype == torch.bfloat16,
+                     "x is a contiguous BF16 [num_tokens, hidden] device tensor")
+        num_x_rows, hidden = x.shape
+        _host_assert((hidden * 2) % 16 == 0, "(hidden * sizeof(bf16)) % sizeof(int4) == 0")
+        _host_assert(src_idx.dim() == 1 and src_idx.shape[0] == num_x_rows and src_idx.dtype == torch.int32,
+                     "src_idx is int32 [num_tokens]")
+        _host_assert(send_head.dim() == 2 and send_head.shape[1] == R and send_head.dtype == torch.int32 and
+                     send_head.is_contiguous(), "send_head is int32 [num_recv_tokens, num_ranks]")
+        _host_assert(tuple(rank_prefix_matrix.shape) == (R, R) and rank_prefix_matrix.dtype == torch.int32,
+                     "rank_prefix_matrix is int32 [num_ranks, num_ranks]")
+        num_tokens = send_head.shape[0]
+        num_topk = 0
+        if topk_weights is not None:
+            _host_assert(topk_weights.dim() == 2 and topk_weights.shape[0] == num_x_rows and topk_weights.is_contiguous() and
+                         topk_weights.dtype == torch.float32 and topk_weights.is_cuda, "topk_weights is FP32 [num_tokens, num_topk]")
+            num_topk = topk_weights.shape[1]
+            _host_assert(num_topk <= _abi.MAX_TOPK, f"num_topk <= {_abi.MAX_TOPK}")
+        for b in (bias_0, bias_1):
+            if b is not None:
+                _host_assert(b.dtype == x.dtype and tuple(b.shape) == (num_tokens, hidden) and b.is_cuda and
+                             b.is_contiguous(), "bias is BF16 [num_recv_tokens, hidden]")
+        _host_assert(bias_0 is not None or bias_1 is None, "bias_1 needs bias_0")
+
+        compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_finish, v1_rules=True)
+        workspace = self._get_workspace(1, 1, R)
+        with torch.cuda.stream(run_stream):
+            recv_x = torch.empty((num_tokens, hidden), dtype=x.dtype, device=self.device)
+            recv_topk_weights = None
+            if topk_weights is not None:
+                recv_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
+            args = _abi.IntranodeCombineArgs()
+            args.num_tokens, args.hidden, args.num_ranks, args.num_topk = num_tokens, hidden, R, num_topk
+            args.x, args.num_x_rows = _abi.ptr(x), num_x_rows
+            args.topk_weights = _abi.ptr(topk_weights)
+            args.bias_0, args.bias_1 = _abi.ptr(bias_0), _abi.ptr(bias_1)
+            args.send_head = _abi.ptr(send_head)
+            args.combined_x, args.combined_topk_weights = _abi.ptr(recv_x), _abi.ptr(recv_topk_weights)
+            args.workspace, args.workspace_bytes = _abi.ptr(workspace), workspace.numel()
+            _abi.check(_abi.lib.deep_ep_hip_launch_intranode_combine(ctypes.byref(args), run_stream.cuda_stream),
+                       "intranode combine")
+        event = self._epilogue([x, topk_weights, bias_0, bias_1, src_idx, send_head, rank_prefix_matrix,
+                                channel_prefix_matrix, recv_x, recv_topk_weights, workspace],
+                               compute_stream, run_stream, allocate_on_comm_stream, async_finish)
+        return recv_x, recv_topk_weights, event
+
+
+class Config:
+    """Tuning knobs of the V1 kernels (csrc/legacy/config.hpp:24-60).  Only `num_sms` has a meaning here: it
+    fixes the number of channels (num_sms / 2) the handle's channel matrices are laid out for."""
+
+    def __init__(self, num_sms: int = 20, num_max_nvl_chunked_send_tokens: int = 6,
+                 num_max_nvl_chunked_recv_tokens: int = 256, num_max_rdma_chunked_send_tokens: int = 6,
+                 num_max_rdma_chunked_recv_tokens: int = 256):
+        _host_assert(num_sms >= 0, "num_sms >= 0")
+        _host_assert(0 < num_max_nvl_chunked_send_tokens < num_max_nvl_chunked_recv_tokens,
+                     "0 < num_max_nvl_chunked_send_tokens < num_max_nvl_chunked_recv_tokens")
+        _host_assert(0 < num_max_rdma_chunked_send_tokens < num_max_rdma_chunked_recv_tokens,
+                     "0 < num_max_rdma_chunked_send_tokens < num_max_rdma_chunked_recv_tokens")
+        self.num_sms = num_sms
+        self.num_max_nvl_chunked_send_tokens = num_max_nvl_chunked_send_tokens
+        self.num_max_nvl_chunked_recv_tokens = num_max_nvl_chunked_recv_tokens
+        self.num_max_rdma_chunked_send_tokens = num_max_rdma_chunked_send_tokens
+        self.num_max_rdma_chunked_recv_tokens = num_max_rdma_chunked_recv_tokens
+
+    def get_nvl_buffer_size_hint(self, hidden_bytes: int, num_ranks: int) -> int:
+        """Bytes the reference would stage per rank (csrc/legacy/config.hpp:53-73); nothing is staged here."""
+        nvl_ranks, rdma_ranks = min(num_ranks, 8), max(num_ranks // 8, 1)
+        slots = (self.num_sms // 2) * nvl_ranks * self.num_max_nvl_chunked_recv_tokens
+        # per queue slot: payload, 8-byte source record, 128 top-k ids and weights, 128 scales (the assumed maxima)
+        per_slot = hidden_bytes + 8 + 128 * 8 + 128 * 4 + 128 * 4
+        total = (self.num_sms // 2) * nvl_ranks * (2 * rdma_ranks + 3) * 4 + slots * per_slot
+        return (total + 127) // 128 * 128

@@ -8,7 +8,7 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
 LIB_NAME = "libdeep_ep_hip.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 PHASE_LAYOUT = 1
 PHASE_MOVE = 2
@@ -93,6 +93,59 @@ class CombineArgs(Structure):
     ]
 
 
+class IntranodeDispatchArgs(Structure):
+    _fields_ = [
+        ("phases", c_int32), ("payload", c_int32), ("cached", c_int32),
+        ("num_tokens", c_int32), ("hidden", c_int32),
+        ("num_topk", c_int32),
+        ("num_experts", c_int32),
+        ("num_ranks", c_int32), ("rank_idx", c_int32),
+        ("num_channels", c_int32),
+        ("expert_alignment", c_int32),
+        ("fill_unused_topk_idx", c_int32),
+        ("x", c_void_p),
+        ("x_scales", c_void_p),
+        ("scale_token_stride", c_int64), ("scale_hidden_stride", c_int64),
+        ("num_scales", c_int32),
+        ("topk_idx", c_void_p),
+        ("topk_weights", c_void_p),
+        ("is_token_in_rank", c_void_p),
+        ("rank_prefix_matrix", c_void_p),
+        ("channel_prefix_matrix", c_void_p),
+        ("recv_channel_prefix_matrix", c_void_p),
+        ("psum_num_recv_tokens_per_rank", c_void_p),
+        ("num_recv_tokens_per_expert", c_void_p),
+        ("host_counts", c_void_p),
+        ("send_head", c_void_p),
+        ("recv_src_idx", c_void_p),
+        ("recv_x", c_void_p),
+        ("recv_x_scales", c_void_p),
+        ("recv_scale_token_stride", c_int64), ("recv_scale_hidden_stride", c_int64),
+        ("recv_topk_idx", c_void_p),
+        ("recv_topk_weights", c_void_p),
+        ("recv_capacity", c_int64),
+        ("workspace", c_void_p),
+        ("workspace_bytes", c_uint64),
+    ]
+
+
+class IntranodeCombineArgs(Structure):
+    _fields_ = [
+        ("num_tokens", c_int32), ("hidden", c_int32), ("num_ranks", c_int32),
+        ("num_topk", c_int32),
+        ("x", c_void_p),
+        ("num_x_rows", c_int64),
+        ("topk_weights", c_void_p),
+        ("bias_0", c_void_p),
+        ("bias_1", c_void_p),
+        ("send_head", c_void_p),
+        ("combined_x", c_void_p),
+        ("combined_topk_weights", c_void_p),
+        ("workspace", c_void_p),
+        ("workspace_bytes", c_uint64),
+    ]
+
+
 class LLDispatchArgs(Structure):
     _fields_ = [
         ("use_fp8", c_int32),
@@ -153,6 +206,8 @@ EXPORTS = {
     "deep_ep_hip_launch_layout": (c_int, [POINTER(LayoutArgs), c_void_p]),
     "deep_ep_hip_launch_dispatch": (c_int, [POINTER(DispatchArgs), c_void_p]),
     "deep_ep_hip_launch_combine": (c_int, [POINTER(CombineArgs), c_void_p]),
+    "deep_ep_hip_launch_intranode_dispatch": (c_int, [POINTER(IntranodeDispatchArgs), c_void_p]),
+    "deep_ep_hip_launch_intranode_combine": (c_int, [POINTER(IntranodeCombineArgs), c_void_p]),
     "deep_ep_hip_ll_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "deep_ep_hip_launch_ll_dispatch": (c_int, [POINTER(LLDispatchArgs), c_void_p]),
     "deep_ep_hip_launch_ll_combine": (c_int, [POINTER(LLCombineArgs), c_void_p]),

@@ -1,6 +1,12 @@
 """`Buffer`: the part of the V1 Python surface that sits on the routing hot path —
-`get_dispatch_layout` and the low-latency packed dispatch / combine (reference
-deep_ep/buffers/legacy.py:293-319, 553-670; host side csrc/legacy/buffer.hpp:337-404, 1463-1715).
+`get_dispatch_layout`, `dispatch` / `combine` inside one scale-up domain, and the low-latency packed
+dispatch / combine (reference deep_ep/buffers/legacy.py:293-455, 553-670; host side
+csrc/legacy/buffer.hpp:337-860, 1463-1715).
+
+`dispatch` moves the tokens of logical source rank `group.rank()`; the received rows are the concatenation
+over destination ranks d of what d gets from this source, in token order (rows of destination d start at
+`rank_prefix_matrix[-1][:d].sum()`).  The handle is the reference's 6-tuple; its `send_head` holds receive
+rows instead of queue positions (opaque to callers either way).
 
 Logical ranks on one GPU.  `group.size()` = R logical ranks, `group.rank()` = this process's logical
 rank.  The packed buffers returned by `low_latency_dispatch` are those of destination rank
@@ -12,7 +18,7 @@ rank.  The packed buffers returned by `low_latency_dispatch` are those of destin
 Rows of one expert are filled by source rank ascending, then token ascending.
 """
 import ctypes
-from typing import Callable, Optional, Tuple
+from typing import Callable, List, Optional, Tuple, Union
 
 import torch
 
@@ -76,6 +82,87 @@ class Buffer:
         a, b, c, d, event = self.runtime.get_dispatch_layout(topk_idx, num_experts, unwrap_event(previous_event),
                                                              async_finish, allocate_on_comm_stream)
         return a, b, c, d, EventOverlap(event)
+
+    @staticmethod
+    def set_num_sms(new_num_sms: int) -> None:
+        assert new_num_sms % 2 == 0, 'The SM count must be even'
+        Buffer.num_sms = new_num_sms
+
+    @staticmethod
+    def get_dispatch_config(num_ranks: int) -> '_C.Config':
+        """Default tuning config (deep_ep/buffers/legacy.py:243-266).  Only `num_sms` matters here: it fixes the
+        channel count of the handle's channel matrices."""
+        return _C.Config(Buffer.num_sms, 6, 256, 6, 128)
+
+    @staticmethod
+    def get_combine_config(num_ranks: int) -> '_C.Config':
+        return _C.Config(Buffer.num_sms, 6, 256, 6, 128)
+
+    @staticmethod
+    def _unpack_bias(bias):
+        bias_0, bias_1 = None, None
+        if isinstance(bias, torch.Tensor):
+            bias_0 = bias
+        elif isinstance(bias, tuple):
+            assert len(bias) == 2
+            bias_0, bias_1 = bias
+        return bias_0, bias_1
+
+    def dispatch(self, x: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]],
+                 handle: Optional[Tuple] = None,
+                 num_tokens_per_rank: Optional[torch.Tensor] = None,
+                 num_tokens_per_rdma_rank: Optional[torch.Tensor] = None,
+                 is_token_in_rank: Optional[torch.Tensor] = None,
+                 num_tokens_per_expert: Optional[torch.Tensor] = None,
+                 topk_idx: Optional[torch.Tensor] = None, topk_weights: Optional[torch.Tensor] = None,
+                 expert_alignment: int = 1, num_worst_tokens: int = 0, config=None,
+                 previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
+                 allocate_on_comm_stream: bool = False):
+        """Dispatch tokens to the ranks that own their experts (signature and returns of
+        deep_ep/buffers/legacy.py:322-404).
+
+        Returns (recv_x or (recv_x, recv_x_scales), recv_topk_idx, recv_topk_weights,
+        num_recv_tokens_per_expert_list, handle, event).  `recv_topk_idx` holds ids local to the receiving
+        rank or -1; `recv_topk_weights` is 0 where `recv_topk_idx` is -1.  The list has one aligned count per
+        expert of every destination rank (empty with `num_worst_tokens`).  With `handle=` the layout is reused
+        and only `recv_x` is returned.
+        """
+        config = self.get_dispatch_config(self.group_size) if config is None else config
+        x, x_scales = x if isinstance(x, tuple) else (x, None)
+        if handle is not None:
+            assert topk_idx is None and topk_weights is None
+            rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, is_token_in_rank, send_head = handle
+            num_recv_tokens = recv_src_idx.size(0)
+            recv_x, recv_x_scales, _, _, _, _, _, _, _, _, event = self.runtime.intranode_dispatch(
+                x, x_scales, None, None, None, is_token_in_rank, None, num_recv_tokens, rank_prefix_matrix,
+                channel_prefix_matrix, expert_alignment, num_worst_tokens, config, unwrap_event(previous_event),
+                async_finish, allocate_on_comm_stream, cached_send_head=send_head)
+            return (recv_x, recv_x_scales) if x_scales is not None else recv_x, None, None, None, None, EventOverlap(event)
+        assert num_tokens_per_rank is not None and is_token_in_rank is not None and num_tokens_per_expert is not None
+        (recv_x, recv_x_scales, recv_topk_idx, recv_topk_weights, num_recv_tokens_per_expert_list, rank_prefix_matrix,
+         channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, send_head, event) = \
+            self.runtime.intranode_dispatch(x, x_scales, topk_idx, topk_weights, num_tokens_per_rank, is_token_in_rank,
+                                            num_tokens_per_expert, 0, None, None, expert_alignment, num_worst_tokens,
+                                            config, unwrap_event(previous_event), async_finish, allocate_on_comm_stream)
+        handle = (rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, is_token_in_rank, send_head)
+        return ((recv_x, recv_x_scales) if x_scales is not None else recv_x, recv_topk_idx, recv_topk_weights,
+                num_recv_tokens_per_expert_list, handle, EventOverlap(event))
+
+    def combine(self, x: torch.Tensor, handle: Tuple, topk_weights: Optional[torch.Tensor] = None,
+                bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor], None] = None, config=None,
+                previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
+                allocate_on_comm_stream: bool = False):
+        """Reduce (add, **without** weights) the rows of every token back to its origin
+        (deep_ep/buffers/legacy.py:407-455): fp32 sum of the biases and of the token's rows in ascending rank
+        order, one rounding to BF16; `topk_weights` rows are summed the same way.
+        Returns (combined_x, combined_topk_weights, event)."""
+        config = self.get_combine_config(self.group_size) if config is None else config
+        rank_prefix_matrix, _, channel_prefix_matrix, src_idx, is_recv_token_in_rank, send_head = handle
+        bias_0, bias_1 = Buffer._unpack_bias(bias)
+        recv_x, recv_topk_weights, event = self.runtime.intranode_combine(
+            x, topk_weights, bias_0, bias_1, src_idx, rank_prefix_matrix, channel_prefix_matrix, send_head, config,
+            unwrap_event(previous_event), async_finish, allocate_on_comm_stream)
+        return recv_x, recv_topk_weights, EventOverlap(event)
 
     def _workspace(self, num_bytes: int) -> torch.Tensor:
         if self._ll_workspace is None or self._ll_workspace.numel() < num_bytes:

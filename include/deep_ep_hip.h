@@ -24,6 +24,10 @@
  *                                   csrc/backends/ascend/elastic/kernels.hpp:274-288
  *   deep_ep_hip_launch_combine      csrc/kernels/elastic/combine.hpp:114,248 (launch_combine +
  *                                   launch_combine_reduce_epilogue)
+ *   deep_ep_hip_launch_intranode_dispatch  csrc/kernels/legacy/intranode.cu:20-175 (notify_dispatch),
+ *                                   :205-612 (dispatch), called from csrc/legacy/buffer.hpp:417-717
+ *   deep_ep_hip_launch_intranode_combine   csrc/kernels/legacy/intranode.cu:700-1095 (combine), called from
+ *                                   csrc/legacy/buffer.hpp:719-860
  *   deep_ep_hip_launch_ll_dispatch  csrc/kernels/legacy/internode_ll.cu:464-554
  *   deep_ep_hip_launch_ll_combine   csrc/kernels/legacy/internode_ll.cu:1140-1238
  *   deep_ep_hip_launch_cast_fp8     deep_ep/utils/math.py:30-39 (per_token_cast_to_fp8)
@@ -38,7 +42,7 @@
 extern "C" {
 #endif
 
-#define DEEP_EP_HIP_ABI_VERSION 1
+#define DEEP_EP_HIP_ABI_VERSION 2
 
 #define DEEP_EP_HIP_OK 0
 #define DEEP_EP_HIP_ERR_INVALID_ARGUMENT (-1)
@@ -167,6 +171,85 @@ typedef struct {
 } deep_ep_hip_combine_args;
 
 int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * V1 `Buffer.dispatch` / `Buffer.combine` inside one scale-up domain (the reference's "intranode" pair),
+ * one logical source rank per call.
+ *
+ * Routing comes from topk_idx when it is given (then recv_topk_idx / recv_topk_weights are produced:
+ * local expert ids or -1, weights of lanes owned by another rank delivered as 0), otherwise from
+ * is_token_in_rank alone.  Receive rows are the concatenation over destination ranks d of the rows d gets
+ * from this source, in token order.  Handle tensors with the reference's meaning: rank_prefix_matrix[i][d] =
+ * rows rank d holds from source ranks <= i (only rank_idx sends here), channel_prefix_matrix[d][c] =
+ * tokens of channels <= c sent to d (channel c = tokens [c*ceil(T/C), (c+1)*ceil(T/C))),
+ * recv_channel_prefix_matrix[d][c] = the same, exclusive.  send_head[t][d] is the receive row of token t on
+ * rank d, or -1 (the reference stores a queue position there; the field is opaque to callers and is what
+ * cached dispatch and combine consume).
+ * Limits: num_ranks <= 64; everything else as for deep_ep_hip_launch_dispatch.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    int32_t phases;                 /* DEEP_EP_HIP_PHASE_*; cached: MOVE only */
+    int32_t payload;                /* DEEP_EP_HIP_PAYLOAD_* */
+    int32_t cached;                 /* send_head is an input; topk_idx / is_token_in_rank are not read */
+    int32_t num_tokens, hidden;
+    int32_t num_topk;               /* 0 when topk_idx is NULL */
+    int32_t num_experts;            /* 0 when topk_idx is NULL */
+    int32_t num_ranks, rank_idx;
+    int32_t num_channels;           /* columns of the channel matrices (reference: config.num_sms / 2) */
+    int32_t expert_alignment;
+    int32_t fill_unused_topk_idx;   /* 1: rows of recv_topk_idx at and beyond the received count are set to -1
+                                       (`num_worst_tokens` mode) */
+
+    const void* x;                  /* [num_tokens, hidden] bf16 or e4m3 */
+    const void* x_scales;           /* payload FP8: [num_tokens, num_scales] 4-byte elements */
+    int64_t scale_token_stride, scale_hidden_stride;
+    int32_t num_scales;
+    const int64_t* topk_idx;        /* [num_tokens, num_topk] or NULL */
+    const float* topk_weights;      /* [num_tokens, num_topk] or NULL (given iff topk_idx is) */
+    const uint8_t* is_token_in_rank; /* [num_tokens, num_ranks] bool */
+
+    /* handle and counts */
+    int32_t* rank_prefix_matrix;            /* [num_ranks, num_ranks] out (phase 1), may be NULL */
+    int32_t* channel_prefix_matrix;         /* [num_ranks, num_channels] out (phase 1), may be NULL */
+    int32_t* recv_channel_prefix_matrix;    /* [num_ranks, num_channels] out (phase 1), may be NULL */
+    int32_t* psum_num_recv_tokens_per_rank; /* [num_ranks] inclusive, out of phase 1, read by phase 2 */
+    int32_t* num_recv_tokens_per_expert;    /* [num_experts] counts before alignment, out of phase 1, or NULL */
+    int32_t* host_counts;                   /* host-mapped [num_ranks + num_experts] or NULL (see dispatch) */
+    int32_t* send_head;                     /* [num_tokens, num_ranks]: out of phase 2 (input when cached) */
+    int32_t* recv_src_idx;                  /* [recv_capacity] out of phase 2, or NULL */
+
+    void* recv_x;                   /* [recv_capacity, hidden] */
+    void* recv_x_scales;            /* [recv_capacity, num_scales], strides below */
+    int64_t recv_scale_token_stride, recv_scale_hidden_stride;
+    int64_t* recv_topk_idx;         /* [recv_capacity, num_topk] or NULL */
+    float* recv_topk_weights;       /* [recv_capacity, num_topk] or NULL */
+    int64_t recv_capacity;
+
+    void* workspace;                /* deep_ep_hip_workspace_bytes(num_tokens, max(num_topk, num_ranks),
+                                       max(num_experts, num_ranks), num_ranks) bytes */
+    uint64_t workspace_bytes;
+} deep_ep_hip_intranode_dispatch_args;
+
+int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_args* args, void* stream);
+
+/* combined_x[t] = bf16( bias_0[t] + bias_1[t] + sum over ranks d ascending with send_head[t][d] >= 0 of
+ * x[send_head[t][d]] ) in fp32; combined_topk_weights[t] = sum of the same rows of topk_weights. */
+typedef struct {
+    int32_t num_tokens, hidden, num_ranks;
+    int32_t num_topk;               /* columns of topk_weights, 0 if none */
+    const void* x;                  /* bf16 [num_x_rows, hidden] */
+    int64_t num_x_rows;
+    const float* topk_weights;      /* [num_x_rows, num_topk] or NULL */
+    const void* bias_0;             /* bf16 [num_tokens, hidden] or NULL */
+    const void* bias_1;
+    const int32_t* send_head;       /* handle: [num_tokens, num_ranks] */
+    void* combined_x;               /* bf16 [num_tokens, hidden] out */
+    float* combined_topk_weights;   /* [num_tokens, num_topk] out or NULL */
+    void* workspace;                /* >= 256 bytes (status word) */
+    uint64_t workspace_bytes;
+} deep_ep_hip_intranode_combine_args;
+
+int deep_ep_hip_launch_intranode_combine(const deep_ep_hip_intranode_combine_args* args, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Low-latency packed layout (V1 `Buffer.low_latency_dispatch/combine`) for one logical

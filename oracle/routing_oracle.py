@@ -25,6 +25,13 @@ Each function names the reference source it restates (paths relative to the refe
   combine()                 the same reduction driven from received rows + handle
                             (deep_ep/include/deep_ep/impls/combine.cuh:86-237,
                              combine_reduce_epilogue.cuh:62-142, combine_utils.cuh:111-168)
+  intranode_world_dispatch() csrc/kernels/legacy/intranode.cu:20-175 (counts, prefix matrices), :320-400 (send
+                            side: row order, local ids, weights zeroed off-rank), :420-545 (receive side:
+                            rank offset + channel offset, recv_src_idx, -1 fill), as driven by
+                            csrc/legacy/buffer.hpp:417-717; checked by tests/legacy/test_intranode.py:90-186
+  intranode_dispatch()      one source rank's share of the above, destinations concatenated
+  intranode_combine()       csrc/kernels/legacy/intranode.cu:940-1033 (bias_0 + bias_1, then rows in ascending
+                            rank order, fp32, one rounding; top-k weights summed over the same rows)
   ll_dispatch()             csrc/legacy/buffer.hpp:1515-1541 + csrc/kernels/legacy/internode_ll.cu:361-461
   ll_combine()              csrc/kernels/legacy/internode_ll.cu:1072-1135 (BF16 branch :704-711)
 
@@ -32,7 +39,8 @@ Pinning status (which independent evidence fixes each function) is listed in tes
 layout -> brute force + literal cases; FP8 cast -> C software e4m3 encoder (oracle/fp8_ref.c) +
 closed-form identities; dispatch -> world composition vs. the literal two-rank cases and
 permutation invariants; combine -> the reference's literal known answers; low latency -> the
-invariants the reference's own test asserts.
+invariants the reference's own test asserts; V1 intranode pair -> the assertions of the reference's
+tests/legacy/test_intranode.py replayed on a whole logical world + composition of per-source shares.
 """
 from __future__ import annotations
 
@@ -478,3 +486,145 @@ def ll_combine(x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tens
             r = row_of[(le, t)]
             out[t] = out[t] + x[le, r].to(torch.float32) * topk_weights[t, k]
     return out.to(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------------------------
+# V1 dispatch / combine inside one scale-up domain ("intranode")
+# ---------------------------------------------------------------------------------------------
+def channel_range(num_tokens: int, num_channels: int, channel: int) -> Tuple[int, int]:
+    """csrc/kernels/legacy/utils.cuh:444-448."""
+    per = ceil_div(num_tokens, num_channels)
+    start = min(per * channel, num_tokens)
+    return start, min(start + per, num_tokens)
+
+
+@dataclass
+class IntranodeRecv:
+    """What one destination rank holds after a V1 dispatch of a whole logical world."""
+    recv_x: torch.Tensor
+    recv_x_scales: Optional[torch.Tensor]
+    recv_topk_idx: Optional[torch.Tensor]
+    recv_topk_weights: Optional[torch.Tensor]
+    recv_src_idx: torch.Tensor
+    num_recv_tokens_per_expert_list: List[int]
+    rank_prefix_matrix: torch.Tensor           # [R, R], identical on every rank
+    recv_channel_prefix_matrix: torch.Tensor   # [R, C]: start of (source, channel) inside the source's rows
+
+
+def _channel_prefix(mask: torch.Tensor, num_channels: int) -> torch.Tensor:
+    T, R = mask.shape
+    out = torch.zeros((R, num_channels), dtype=torch.int32)
+    for c in range(num_channels):
+        lo, hi = channel_range(T, num_channels, c)
+        out[:, c] = mask[lo:hi].sum(dim=0).to(torch.int32)
+    return out.cumsum(dim=1).to(torch.int32)
+
+
+def intranode_world_dispatch(xs: Sequence[TensorOrPair], masks: Sequence[torch.Tensor],
+                             topk_idxs: Optional[Sequence[torch.Tensor]], topk_weights: Optional[Sequence[torch.Tensor]],
+                             num_experts: int, expert_alignment: int = 1, num_channels: int = 10):
+    """Returns (per-destination IntranodeRecv list, per-source channel_prefix_matrix list)."""
+    R = len(xs)
+    E_l = num_experts // R if num_experts else 0
+    with_topk = topk_idxs is not None
+    counts = torch.stack([m.sum(dim=0).to(torch.int32) for m in masks])           # [source, destination]
+    rank_prefix = counts.cumsum(dim=0).to(torch.int32)
+    channel_prefix = [_channel_prefix(m, num_channels) for m in masks]
+    out = []
+    for j in range(R):
+        rows_x, rows_s, rows_idx, rows_w, rows_src = [], [], [], [], []
+        for i in range(R):
+            x, sf = _unpack(xs[i])
+            sel = masks[i][:, j].nonzero().flatten()                               # token order
+            rows_x.append(x[sel])
+            if sf is not None:
+                rows_s.append(sf[sel])
+            rows_src.append(sel.to(torch.int32))
+            if with_topk:
+                idx = topk_idxs[i][sel]
+                local = (idx >= j * E_l) & (idx < (j + 1) * E_l)
+                rows_idx.append(torch.where(local, idx - j * E_l, torch.full_like(idx, -1)))
+                rows_w.append(torch.where(local, topk_weights[i][sel], torch.zeros_like(topk_weights[i][sel])))
+        per_expert = []
+        if with_topk:
+            stacked = torch.cat([t.flatten() for t in topk_idxs])
+            for e in range(j * E_l, (j + 1) * E_l):
+                per_expert.append(align(int((stacked == e).sum()), expert_alignment))
+        recv_channel = torch.zeros((R, num_channels), dtype=torch.int32)
+        for i in range(R):
+            recv_channel[i, 1:] = channel_prefix[i][j, :-1]
+        out.append(IntranodeRecv(
+            recv_x=torch.cat(rows_x), recv_x_scales=torch.cat(rows_s) if rows_s else None,
+            recv_topk_idx=torch.cat(rows_idx) if with_topk else None,
+            recv_topk_weights=torch.cat(rows_w) if with_topk else None,
+            recv_src_idx=torch.cat(rows_src), num_recv_tokens_per_expert_list=per_expert,
+            rank_prefix_matrix=rank_prefix, recv_channel_prefix_matrix=recv_channel))
+    return out, channel_prefix
+
+
+@dataclass
+class IntranodeShare:
+    """One source rank's contribution, destinations concatenated in rank order (what a one-GPU call returns)."""
+    recv_x: torch.Tensor
+    recv_x_scales: Optional[torch.Tensor]
+    recv_topk_idx: Optional[torch.Tensor]
+    recv_topk_weights: Optional[torch.Tensor]
+    recv_src_idx: torch.Tensor
+    num_recv_tokens_per_expert_list: List[int]
+    rank_prefix_matrix: torch.Tensor
+    channel_prefix_matrix: torch.Tensor
+    recv_channel_prefix_matrix: torch.Tensor
+    send_head: torch.Tensor                    # [T, R]: row of the concatenated receive buffer, or -1
+
+
+def intranode_dispatch(x: TensorOrPair, mask: torch.Tensor, topk_idx: Optional[torch.Tensor],
+                       topk_weights: Optional[torch.Tensor], num_experts: int, num_ranks: int, rank: int,
+                       expert_alignment: int = 1, num_channels: int = 10) -> IntranodeShare:
+    R = num_ranks
+    T = mask.shape[0]
+    data, sf = _unpack(x)
+    # A world in which only `rank` holds tokens
+    empty_mask = torch.zeros((0, R), dtype=torch.bool)
+    xs = [(data[:0], sf[:0]) if sf is not None else data[:0] for _ in range(R)]
+    masks = [empty_mask for _ in range(R)]
+    idxs = [topk_idx[:0] for _ in range(R)] if topk_idx is not None else None
+    ws = [topk_weights[:0] for _ in range(R)] if topk_idx is not None else None
+    xs[rank], masks[rank] = x, mask
+    if topk_idx is not None:
+        idxs[rank], ws[rank] = topk_idx, topk_weights
+    world, channel_prefix = intranode_world_dispatch(xs, masks, idxs, ws, num_experts, expert_alignment, num_channels)
+    send_head = torch.full((T, R), -1, dtype=torch.int32)
+    base = 0
+    for j in range(R):
+        sel = mask[:, j].nonzero().flatten()
+        send_head[sel, j] = base + torch.arange(sel.numel(), dtype=torch.int32)
+        base += sel.numel()
+    cat = lambda parts: torch.cat(parts) if parts[0] is not None else None
+    return IntranodeShare(
+        recv_x=torch.cat([w.recv_x for w in world]),
+        recv_x_scales=cat([w.recv_x_scales for w in world]),
+        recv_topk_idx=cat([w.recv_topk_idx for w in world]),
+        recv_topk_weights=cat([w.recv_topk_weights for w in world]),
+        recv_src_idx=torch.cat([w.recv_src_idx for w in world]),
+        num_recv_tokens_per_expert_list=[c for w in world for c in w.num_recv_tokens_per_expert_list],
+        rank_prefix_matrix=world[0].rank_prefix_matrix,
+        channel_prefix_matrix=channel_prefix[rank],
+        recv_channel_prefix_matrix=torch.stack([w.recv_channel_prefix_matrix[rank] for w in world]),
+        send_head=send_head)
+
+
+def intranode_combine(x: torch.Tensor, send_head: torch.Tensor, topk_weights: Optional[torch.Tensor] = None,
+                      bias=None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """x: [rows, H] bf16 laid out like the dispatched rows; returns (combined_x [T, H], combined weights)."""
+    T, R = send_head.shape
+    H = x.shape[1]
+    acc = _bias_sum(bias)
+    acc = torch.zeros((T, H), dtype=torch.float32) if acc is None else acc.clone()
+    w_out = None if topk_weights is None else torch.zeros((T, topk_weights.shape[1]), dtype=torch.float32)
+    for j in range(R):
+        rows = send_head[:, j].long()
+        has = rows >= 0
+        acc[has] = acc[has] + x[rows[has]].to(torch.float32)
+        if w_out is not None:
+            w_out[has] = w_out[has] + topk_weights[rows[has]]
+    return acc.to(torch.bfloat16), w_out

@@ -31,12 +31,14 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(_abi.lib, name), f"{name} is declared in the header but not exported"
     assert sorted(_abi.EXPORTS) == names, "ctypes binding table and header disagree"
-    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 1
+    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 2
 
 
 def test_ctypes_structs_match_the_header_layout():
     structs = {"deep_ep_hip_layout_args": _abi.LayoutArgs, "deep_ep_hip_dispatch_args": _abi.DispatchArgs,
-               "deep_ep_hip_combine_args": _abi.CombineArgs, "deep_ep_hip_ll_dispatch_args": _abi.LLDispatchArgs,
+               "deep_ep_hip_combine_args": _abi.CombineArgs,
+               "deep_ep_hip_intranode_dispatch_args": _abi.IntranodeDispatchArgs,
+               "deep_ep_hip_intranode_combine_args": _abi.IntranodeCombineArgs, "deep_ep_hip_ll_dispatch_args": _abi.LLDispatchArgs,
                "deep_ep_hip_ll_combine_args": _abi.LLCombineArgs, "deep_ep_hip_cast_args": _abi.CastArgs}
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {"]
     for cname, cls in structs.items():

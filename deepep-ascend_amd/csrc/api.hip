@@ -512,6 +512,8 @@ int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* a, void* 
     REQUIRE(a->hidden >= 16 && a->hidden % 16 == 0, "hidden must be a multiple of 16");
     REQUIRE(!a->use_fp8 || a->hidden % 128 == 0, "FP8 needs hidden %% 128 == 0");
     REQUIRE(!a->use_fp8 || a->packed_recv_x_scales != nullptr, "packed_recv_x_scales is NULL");
+    REQUIRE(!a->round_scale || a->use_fp8, "round_scale needs use_fp8");
+    REQUIRE(!a->use_ue8m0 || (a->round_scale && a->hidden % 512 == 0), "use_ue8m0 needs round_scale and hidden %% 512 == 0");
     REQUIRE(a->x != nullptr && a->topk_idx != nullptr && a->packed_recv_x != nullptr && a->packed_recv_count != nullptr &&
             a->packed_recv_src_info != nullptr && a->packed_recv_layout_range != nullptr, "NULL tensor");
     const size_t need = deep_ep_hip_ll_workspace_bytes(a->num_src_ranks, a->src_token_stride, a->num_topk, a->num_local_experts);
@@ -523,6 +525,8 @@ int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* a, void* 
     const size_t chunks = size_t(a->num_src_ranks) * ((size_t(a->src_token_stride) + kLayoutChunk - 1) / kLayoutChunk);
     LLDispatchParams p{};
     p.use_fp8 = a->use_fp8 ? 1 : 0;
+    p.round_scale = a->round_scale ? 1 : 0;
+    p.use_ue8m0 = a->use_ue8m0 ? 1 : 0;
     p.S = a->num_src_ranks; p.src_rank_begin = a->src_rank_begin; p.src_token_stride = a->src_token_stride;
     p.num_tokens_per_src = a->num_tokens_per_src;
     p.H = a->hidden; p.K = a->num_topk; p.E = a->num_experts; p.expert_begin = a->expert_begin;

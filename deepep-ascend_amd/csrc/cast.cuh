@@ -13,6 +13,11 @@ namespace deep_ep_hip {
 
 // Each lane holds 16 consecutive BF16 channels in (a, b); 8 consecutive lanes form one group of
 // 128 channels.  Writes the 16 e4m3 bytes to `out` and returns the group's stored scale.
+//
+// pow2_scale: the scale is rounded up to a power of two (csrc/kernels/legacy/utils.cuh:481-503, `round_scale`):
+// exponent = ceil(log2(amax * (1/448))) read off the fp32 bit pattern, payload = e4m3(x * 2^-exponent), stored
+// scale = 2^exponent.
+template <bool kPow2Scale = false>
 __device__ __forceinline__ float cast_16_channels(const vec16& a, const vec16& b, vec16& out) {
     const uint32_t wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     float f[16];
@@ -24,8 +29,16 @@ __device__ __forceinline__ float cast_16_channels(const vec16& a, const vec16& b
         amax = fmaxf(amax, fmaxf(fabsf(f[2 * i]), fabsf(f[2 * i + 1])));
     }
     amax = fmaxf(group8_max(amax), 1e-4f);
-    const float scale = 448.0f / amax;
-    const float scale_inv = amax / 448.0f;
+    float scale, scale_inv;
+    if constexpr (kPow2Scale) {
+        const uint32_t bits = __float_as_uint(amax * (1.0f / 448.0f));
+        const int exponent = int((bits >> 23) & 0xffu) - 127 + ((bits & 0x7fffffu) != 0u ? 1 : 0);
+        scale = __uint_as_float(uint32_t(127 - exponent) << 23);
+        scale_inv = __uint_as_float(uint32_t(127 + exponent) << 23);
+    } else {
+        scale = 448.0f / amax;
+        scale_inv = amax / 448.0f;
+    }
 #pragma unroll
     for (int i = 0; i < 16; ++i) f[i] = f[i] * scale;
     out.x = pack_e4m3x4(f[0], f[1], f[2], f[3]);

@@ -172,6 +172,7 @@ hipError_t launch_cast_kernel(const CastParams& p, hipStream_t stream);
 
 struct LLDispatchParams {
     int use_fp8;
+    int round_scale, use_ue8m0;
     int S, src_rank_begin, src_token_stride;
     const int32_t* num_tokens_per_src;
     int H, K, E, expert_begin, E_l, R, M;

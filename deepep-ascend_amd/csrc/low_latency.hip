@@ -157,7 +157,8 @@ __device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int til
     if constexpr (kFp8) {
 #pragma unroll
         for (int q = 0; q < kPairs; ++q) {
-            const float scale_inv = cast_16_channels(in[q][0], in[q][1], out[q]);
+            const float scale_inv = p.round_scale ? cast_16_channels<true>(in[q][0], in[q][1], out[q])
+                                                  : cast_16_channels<false>(in[q][0], in[q][1], out[q]);
             const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
             if ((lane >> 3) == q) my_scale = gathered;
         }
@@ -180,8 +181,17 @@ __device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int til
                 const int elem = (tile * kPairs + q) * 1024 + lane * 16;
                 if (elem < p.H) store16_stream(dst + elem, out[q]);
             }
-            if (owns_scale)
-                p.packed_scales[(int64_t(dle) * num_groups + group) * rows_per_expert + dslot] = my_scale;
+            if (owns_scale) {
+                if (p.use_ue8m0) {
+                    // exponent bytes, four groups to an int32 pack; packs column-major like the fp32 scales
+                    // (csrc/kernels/legacy/internode_ll.cu:440-457)
+                    uint8_t* bytes = reinterpret_cast<uint8_t*>(p.packed_scales);
+                    const int64_t pack = (int64_t(dle) * (num_groups / 4) + (group >> 2)) * rows_per_expert + dslot;
+                    bytes[pack * 4 + (group & 3)] = uint8_t(__float_as_uint(my_scale) >> 23);
+                } else {
+                    p.packed_scales[(int64_t(dle) * num_groups + group) * rows_per_expert + dslot] = my_scale;
+                }
+            }
         } else {
             uint8_t* dst = p.packed_x + row * row_bytes;
 #pragma unroll

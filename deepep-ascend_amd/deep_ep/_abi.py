@@ -149,6 +149,8 @@ class IntranodeCombineArgs(Structure):
 class LLDispatchArgs(Structure):
     _fields_ = [
         ("use_fp8", c_int32),
+        ("round_scale", c_int32),
+        ("use_ue8m0", c_int32),
         ("num_src_ranks", c_int32), ("src_rank_begin", c_int32),
         ("src_token_stride", c_int32),
         ("num_tokens_per_src", c_void_p),

@@ -44,6 +44,7 @@ class Buffer:
         self.runtime = _C.ElasticBuffer(self.rank, self.group_size, 0, [], _C.get_elastic_buffer_alignment(), 0,
                                         False, True, True, 0, 0, 300, 100, explicitly_destroy)
         self._ll_workspace: Optional[torch.Tensor] = None
+        self._ll_combine_buffer: Optional[torch.Tensor] = None
 
     def destroy(self) -> None:
         assert self.explicitly_destroy, '`explicitly_destroy` flag must be set'
@@ -184,11 +185,15 @@ class Buffer:
             recv_count: `[E/R]` int32;
             handle: `(src_info [E/R, R*M] int32, layout_range [E/R, R] int64 = (begin << 32) | count,
                       num_max_dispatch_tokens_per_rank, hidden, num_experts)`;
-            hook: None (there is no separate receive phase on one GPU).
-        FP8 scales follow the torch recipe (amax / 448 by IEEE division).
+            hook: with `return_recv_hook`, a callable to invoke before reading the outputs (the reference splits
+                send and receive around it; on one GPU everything is already enqueued and it does nothing).
+        FP8 scales follow the torch recipe (amax / 448 by IEEE division); with `round_scale` they are rounded up
+        to powers of two (csrc/kernels/legacy/utils.cuh:481-503) and with `use_ue8m0` returned as exponent bytes
+        packed four to an int32: `[E/R, R*M, hidden // 512]`, column-major in the last two dimensions.
         """
-        assert not (round_scale or use_ue8m0), 'power-of-two / UE8M0 scales are not implemented in the HIP backend'
-        assert not return_recv_hook, 'there is no separate receive phase on one GPU'
+        assert not round_scale or use_fp8, '`round_scale` needs `use_fp8`'
+        assert not use_ue8m0 or round_scale, '`use_ue8m0` needs `round_scale`'
+        assert not (return_recv_hook and async_finish), 'a receive hook and `async_finish` exclude each other'
         R, M = self.group_size, num_max_dispatch_tokens_per_rank
         assert x.dtype == torch.bfloat16 and x.is_contiguous() and x.is_cuda
         assert topk_idx.is_contiguous() and topk_idx.dtype == _C.topk_idx_t
@@ -215,12 +220,15 @@ class Buffer:
             packed_recv_layout_range = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
             packed_recv_count = torch.empty((E_l,), dtype=torch.int32, device=dev)
             packed_recv_x_scales = None
-            if use_fp8:
+            if use_fp8 and use_ue8m0:
+                assert H % 512 == 0
+                packed_recv_x_scales = torch.empty((E_l, H // 512, rows), dtype=torch.int32, device=dev).transpose(1, 2)
+            elif use_fp8:
                 packed_recv_x_scales = torch.empty((E_l, H // 128, rows), dtype=torch.float32, device=dev).transpose(1, 2)
             if T > 0:
                 ws = self._workspace(_abi.lib.deep_ep_hip_ll_workspace_bytes(S, T, K, E_l))
                 args = _abi.LLDispatchArgs()
-                args.use_fp8 = int(use_fp8)
+                args.use_fp8, args.round_scale, args.use_ue8m0 = int(use_fp8), int(round_scale), int(use_ue8m0)
                 args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
                 args.num_tokens_per_src = 0
                 args.hidden, args.num_topk, args.num_experts = H, K, num_experts
@@ -243,7 +251,17 @@ class Buffer:
         event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
         handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H, num_experts)
         recv = (packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x
-        return recv, packed_recv_count, handle, EventOverlap(event, tensors if async_finish else None), None
+        hook = (lambda: None) if return_recv_hook else None
+        return recv, packed_recv_count, handle, EventOverlap(event, tensors if async_finish else None), hook
+
+    def get_next_low_latency_combine_buffer(self, handle: tuple) -> torch.Tensor:
+        """`[E/R, R*M, hidden]` BF16 buffer a caller may fill instead of passing `x` to `low_latency_combine`
+        (`zero_copy=True`), deep_ep/buffers/legacy.py:673-689."""
+        src_info, layout_range, M, H, num_experts = handle
+        shape = (num_experts // self.group_size, self.group_size * M, H)
+        if self._ll_combine_buffer is None or tuple(self._ll_combine_buffer.shape) != shape:
+            self._ll_combine_buffer = torch.empty(shape, dtype=torch.bfloat16, device=self.runtime.device)
+        return self._ll_combine_buffer
 
     def low_latency_combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
                             handle: tuple, use_logfmt: bool = False, zero_copy: bool = False,
@@ -255,11 +273,19 @@ class Buffer:
         `x` is `[E/R, R*M, hidden]` BF16 laid out like the dispatched buffers; `topk_idx` / `topk_weights` are
         those of the dispatched tokens (`[T, K]`, or `[R, T, K]` for the stacked form).  Each token sums, in lane
         order and in fp32, `weight * row` over its lanes whose expert lives on this rank, then rounds once to
-        BF16.  Returns (combined_x, event, hook=None).
+        BF16.  Returns (combined_x, event, hook); `hook` is a no-op callable with `return_recv_hook`, else None.
+        With `zero_copy` the rows are read from `get_next_low_latency_combine_buffer(handle)` instead of `x`.
+        `use_logfmt` is refused: LogFMT-10 is a wire format for rows in flight between GPUs
+        (csrc/kernels/legacy/internode_ll.cu:556-712); nothing is in flight here, and its encode/decode is built on
+        the approximate log2/exp2 instructions of another vendor's hardware, so its rounding cannot be reproduced.
         """
-        assert not use_logfmt, 'LogFMT is not implemented in the HIP backend'
-        assert not return_recv_hook, 'there is no separate receive phase on one GPU'
+        if use_logfmt:
+            raise NotImplementedError('LogFMT combine is a transport codec; the one-GPU HIP backend has no transport')
+        assert not (return_recv_hook and async_finish), 'a receive hook and `async_finish` exclude each other'
         src_info, layout_range, M, H, num_experts = handle
+        if zero_copy:
+            assert self._ll_combine_buffer is not None, 'call get_next_low_latency_combine_buffer() first'
+            x = self._ll_combine_buffer
         R = self.group_size
         E_l = num_experts // R
         assert x.dtype == torch.bfloat16 and x.is_contiguous() and tuple(x.shape) == (E_l, R * M, H)
@@ -297,4 +323,5 @@ class Buffer:
                            "low_latency_combine")
         tensors = (x, topk_idx, topk_weights, src_info, layout_range, combined_x)
         event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
-        return combined_x, EventOverlap(event, tensors if async_finish else None), None
+        hook = (lambda: None) if return_recv_hook else None
+        return combined_x, EventOverlap(event, tensors if async_finish else None), hook

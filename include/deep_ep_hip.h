@@ -259,7 +259,10 @@ int deep_ep_hip_launch_intranode_combine(const deep_ep_hip_intranode_combine_arg
  * Fill order inside an expert buffer: source rank ascending, then token ascending.
  * ---------------------------------------------------------------------------------------- */
 typedef struct {
-    int32_t use_fp8;                    /* 1: e4m3 payload + fp32 scales; 0: bf16 payload */
+    int32_t use_fp8;                    /* 1: e4m3 payload + scales; 0: bf16 payload */
+    int32_t round_scale;                /* fp8: scales rounded up to powers of two */
+    int32_t use_ue8m0;                  /* fp8 + round_scale: scales stored as exponent bytes, 4 per int32 pack;
+                                           needs hidden % 512 == 0 */
     int32_t num_src_ranks, src_rank_begin;
     int32_t src_token_stride;           /* rows of x reserved per source rank */
     const int32_t* num_tokens_per_src;  /* [num_src_ranks] device, or NULL = src_token_stride each */
@@ -271,7 +274,8 @@ typedef struct {
     const void* x;                      /* bf16 [num_src_ranks * src_token_stride, hidden] */
     const int64_t* topk_idx;            /* [num_src_ranks * src_token_stride, num_topk] */
     void* packed_recv_x;                /* [num_local_experts, rows, hidden] */
-    float* packed_recv_x_scales;        /* fp8: element (e, row, g) at e*rows*G + g*rows + row */
+    float* packed_recv_x_scales;        /* fp8: element (e, row, g) at e*rows*G + g*rows + row (G = hidden/128);
+                                           use_ue8m0: byte (e, row, g) at ((e*G/4 + g/4)*rows + row)*4 + g%4 */
     int32_t* packed_recv_count;         /* [num_local_experts] out */
     int32_t* packed_recv_src_info;      /* [num_local_experts, rows] out */
     int64_t* packed_recv_layout_range;  /* [num_local_experts, num_ranks] out: (begin<<32)|count */

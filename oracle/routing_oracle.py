@@ -106,6 +106,32 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q.view(T, Hp)[:, :H].contiguous(), scales.view(T, Hp // 128)
 
 
+def per_token_cast_to_fp8_pow2(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The `round_scale` variant of the low-latency kernels (csrc/kernels/legacy/utils.cuh:477-503 as used by
+    internode_ll.cu:223-243): exponent = ceil(log2(amax * fp32(1/448))) with amax clamped below at 1e-4,
+    payload = e4m3fn(x * 2^-exponent), scale = 2^exponent (fp32).  Scaling by a power of two is exact, so the
+    only rounding is the e4m3 conversion."""
+    assert x.dim() == 2
+    T, H = x.shape
+    assert H % 128 == 0
+    g = x.to(torch.float32).view(T, H // 128, 128)
+    amax = g.abs().amax(dim=2).clamp(min=1e-4)
+    ratio = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+    mantissa, exponent = torch.frexp(ratio)                         # ratio = mantissa * 2^exponent, 0.5 <= mantissa < 1
+    exponent = torch.where(mantissa == 0.5, exponent - 1, exponent)  # ceil(log2(ratio))
+    scale_inv = torch.ldexp(torch.ones_like(ratio), exponent)
+    q = torch.ldexp(g, (-exponent).unsqueeze(2)).to(torch.float8_e4m3fn)
+    return q.view(T, H).contiguous(), scale_inv.view(T, H // 128)
+
+
+def pack_ue8m0(scales: torch.Tensor) -> torch.Tensor:
+    """fp32 power-of-two scales [..., G] -> int32 [..., G / 4]: byte k of pack p is the biased exponent of scale
+    4p + k (csrc/kernels/legacy/utils.cuh:505-512, internode_ll.cu:440-457; decode deep_ep/utils/math.py:51-53)."""
+    exps = (scales.contiguous().view(torch.int32) >> 23) & 0xff
+    exps = exps.view(*scales.shape[:-1], scales.shape[-1] // 4, 4)
+    return (exps[..., 0] | (exps[..., 1] << 8) | (exps[..., 2] << 16) | (exps[..., 3] << 24)).to(torch.int32)
+
+
 def per_token_cast_back(x_fp8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
     """Inverse of per_token_cast_to_fp8 up to quantisation: bf16(fp32(q) * scale)."""
     T, H = x_fp8.shape
@@ -414,7 +440,7 @@ def combine(x: torch.Tensor, handle_topk_idx: torch.Tensor, recv_src_metadata: t
 
 def ll_dispatch(xs: Sequence[torch.Tensor], topk_idxs: Sequence[torch.Tensor],
                 num_max_dispatch_tokens_per_rank: int, num_experts: int, num_ranks: int,
-                dst_rank: int, use_fp8: bool = True):
+                dst_rank: int, use_fp8: bool = True, round_scale: bool = False):
     """What logical destination rank `dst_rank` holds after every source rank in `xs` has sent.
 
     xs[s] is source rank s's bf16 [T_s, H]; entries may be None (that source sends nothing).
@@ -439,7 +465,7 @@ def ll_dispatch(xs: Sequence[torch.Tensor], topk_idxs: Sequence[torch.Tensor],
         x = xs[s]
         idx = topk_idxs[s].to(torch.int64)
         if use_fp8:
-            q, sc = per_token_cast_to_fp8(x)
+            q, sc = per_token_cast_to_fp8_pow2(x) if round_scale else per_token_cast_to_fp8(x)
         for le in range(E_l):
             e = dst_rank * E_l + le
             toks = (idx == e).any(dim=1).nonzero(as_tuple=True)[0]

@@ -70,3 +70,58 @@ def test_ll_stacked_sources(R, T, H, E, K, M, use_fp8):
             assert_equal(handle1[1], r1[4], "single-source layout_range")
             out1, _, _ = buf.low_latency_combine(y.cuda() * 0 + 1, idx[s].cuda(), w[s].cuda(), handle1)
             assert out1.shape == (T, H)
+
+
+@pytest.mark.parametrize("R,T,H,E,K,M", [(8, 128, 7168, 256, 8, 128), (2, 40, 1024, 8, 2, 64), (2, 1500, 512, 16, 9, 1500)])
+@pytest.mark.parametrize("use_ue8m0", [False, True])
+def test_ll_power_of_two_scales_hooks_and_zero_copy(R, T, H, E, K, M, use_ue8m0):
+    """`round_scale` / `use_ue8m0` scale formats, `return_recv_hook` and the zero-copy combine buffer
+    (the mode loop of the reference's tests/legacy/test_low_latency.py:89-104,160-173)."""
+    import deep_ep
+    x, idx, w = rc.c5_sources(seed=6, R=R, T=T, H=H, E=E, K=K)
+    x = (x.float() * torch.logspace(-3, 3, T).view(1, T, 1)).to(torch.bfloat16)      # spread the exponents
+    dst_rank = R - 1
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(dst_rank, R), low_latency_mode=True)
+    recv, count, handle, event, hook = buf.low_latency_dispatch(x.cuda(), idx.cuda(), M, E, use_fp8=True, round_scale=True,
+                                                                use_ue8m0=use_ue8m0, return_recv_hook=True)
+    assert callable(hook)
+    hook()
+    ref_x, ref_s, ref_cnt, ref_info, ref_range = oracle.ll_dispatch(list(x), list(idx), M, E, R, dst_rank, True, round_scale=True)
+    assert_equal(count, ref_cnt, "packed_recv_count")
+    assert_equal(handle[1], ref_range, "packed_recv_layout_range")
+    E_l, rows = E // R, R * M
+    if use_ue8m0:
+        assert recv[1].dtype == torch.int32 and recv[1].shape == (E_l, rows, H // 512)
+        assert recv[1].stride(1) == 1 and recv[1].stride(2) == rows
+    else:
+        assert recv[1].dtype == torch.float32 and recv[1].shape == (E_l, rows, H // 128)
+    for e in range(E_l):
+        n = int(ref_cnt[e])
+        assert_equal(recv[0][e, :n].view(torch.uint8), ref_x[e, :n].view(torch.uint8), f"packed_recv_x[{e}]")
+        expect = oracle.pack_ue8m0(ref_s[e, :n]) if use_ue8m0 else ref_s[e, :n]
+        assert_equal(recv[1][e, :n], expect, f"scales[{e}]")
+    # the reference's decode rule recovers the dispatched values to FP8 accuracy
+    if use_ue8m0:
+        packs = torch.empty(recv[1].shape, dtype=torch.int32)
+        packs.copy_(recv[1])
+        sc = (packs.view(torch.uint8).to(torch.int32) << 23).view(torch.float32)
+    else:
+        sc = recv[1].cpu()
+    for e in range(E_l):
+        n = int(ref_cnt[e])
+        if n:
+            back = oracle.per_token_cast_back(recv[0][e, :n].cpu(), sc[e, :n].contiguous())
+            src = torch.cat([x[s][ref_info[e, (ref_range[e, s] >> 32):(ref_range[e, s] >> 32) + (ref_range[e, s] & 0xffffffff)].long()]
+                             for s in range(R)])
+            assert float((back.float() - src.float()).abs().max() / src.float().abs().max()) < 0.07
+
+    # zero-copy combine: same result as passing the tensor
+    y = torch.randn((E_l, rows, H), generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
+    out_a, _, hook_a = buf.low_latency_combine(y, idx.cuda(), w.cuda(), handle, return_recv_hook=True)
+    hook_a()
+    buf.get_next_low_latency_combine_buffer(handle)[:, :, :] = y
+    out_b, _, hook_b = buf.low_latency_combine(torch.empty_like(y), idx.cuda(), w.cuda(), handle, zero_copy=True)
+    assert hook_b is None
+    assert_equal(out_a, out_b, "zero-copy combine")
+    with pytest.raises(NotImplementedError):
+        buf.low_latency_combine(y, idx.cuda(), w.cuda(), handle, use_logfmt=True)

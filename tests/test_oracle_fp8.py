@@ -145,3 +145,43 @@ def test_ordered_sum_matches_c_restatement(cref):
     # the reference's bf16 known answer: contributions are bf16 first (301 -> 300, 302 -> 302), sum 602 -> bf16 600
     data = torch.tensor([[301.0], [302.0]]).to(torch.bfloat16)
     assert float(oracle.ordered_accumulate(data.unsqueeze(0))[0, 0]) == 600.0
+
+
+# ---- power-of-two scales (`round_scale`) and UE8M0 packing ----
+def test_pow2_scales_against_exact_arithmetic_and_the_c_encoder(cref):
+    """Independent restatement with Python's exact rationals: the scale is the smallest power of two that is
+    >= fp32(amax * fp32(1/448)); the payload is the nearest e4m3 code of x / scale (C nearest-code search)."""
+    import math
+    from fractions import Fraction
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn((64, 256), generator=g) * torch.logspace(-6, 4, 64).unsqueeze(1)).to(torch.bfloat16)
+    x[0] = 0                                     # all-zero groups: amax clamps to 1e-4
+    x[1, :128] = 448.0                           # ratio exactly 1 -> exponent 0
+    x[2, :128] = 449.0                           # bf16(449) = 448 as well
+    x[3, :128] = 452.0                           # just above: exponent 1
+    q, s = oracle.per_token_cast_to_fp8_pow2(x)
+    inv448 = np.float32(1.0) / np.float32(448.0)
+    for t in range(x.shape[0]):
+        for grp in range(2):
+            vals = x[t, grp * 128:(grp + 1) * 128].float()
+            amax = max(float(vals.abs().max()), float(np.float32(1e-4)))
+            ratio = Fraction(float(np.float32(amax) * inv448))
+            e = math.ceil(math.log2(ratio)) if ratio != 2 ** round(math.log2(ratio)) else round(math.log2(ratio))
+            assert Fraction(2) ** (e - 1) < ratio <= Fraction(2) ** e
+            assert float(s[t, grp]) == 2.0 ** e
+            for c in range(0, 128, 17):
+                exact = float(vals[c]) / 2.0 ** e
+                code = cref.oracle_e4m3_from_f32(exact)
+                assert int(q[t, grp * 128 + c].view(torch.uint8)) == code
+    assert float(s[1, 0]) == 1.0 and float(s[2, 0]) == 1.0 and float(s[3, 0]) == 2.0
+    assert float(s[0, 0]) == 2.0 ** -22            # 1e-4 / 448 = 2.23e-7 -> 2^-22 = 2.38e-7
+
+
+def test_ue8m0_packing_round_trips_through_the_reference_decode_rule():
+    s = torch.tensor([[1.0, 2.0, 0.5, 2.0 ** -22, 2.0 ** 10, 2.0 ** -3, 1.0, 4.0]])
+    packed = oracle.pack_ue8m0(s)
+    assert packed.shape == (1, 2) and packed.dtype == torch.int32
+    assert packed[0, 0].item() == (127 | (128 << 8) | (126 << 16) | (105 << 24))
+    # decode as deep_ep/utils/math.py:51-53 does
+    back = (packed.view(torch.uint8).to(torch.int32) << 23).view(torch.float32)
+    assert torch.equal(back.view(1, 8), s)

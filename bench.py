@@ -269,6 +269,7 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     cnt = torch.empty(E_l, dtype=torch.int32, device=dev)
     info = torch.empty((E_l, rows), dtype=torch.int32, device=dev)
     rng = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
+    lane_rows = torch.empty((R * T, K), dtype=torch.int32, device=dev)    # what Buffer keeps beside the handle
     y = torch.randn((E_l, rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)
     out = torch.empty((R, T, H), dtype=torch.bfloat16, device=dev)
     ws = torch.zeros(max(_abi.lib.deep_ep_hip_ll_workspace_bytes(R, T, K, E_l), 4096), dtype=torch.uint8, device=dev)
@@ -279,6 +280,7 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     d.x, d.topk_idx = x.data_ptr(), idx.data_ptr()
     d.packed_recv_x, d.packed_recv_x_scales, d.packed_recv_count = px.data_ptr(), ps.data_ptr(), cnt.data_ptr()
     d.packed_recv_src_info, d.packed_recv_layout_range = info.data_ptr(), rng.data_ptr()
+    d.lane_rows = lane_rows.data_ptr()
     d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
     c = _abi.LLCombineArgs()
     c.num_src_ranks, c.src_rank_begin, c.src_token_stride = R, 0, T
@@ -286,6 +288,7 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     c.num_max_dispatch_tokens_per_rank = M
     c.x, c.topk_idx, c.topk_weights = y.data_ptr(), idx.data_ptr(), w.data_ptr()
     c.packed_recv_src_info, c.packed_recv_layout_range, c.combined_x = info.data_ptr(), rng.data_ptr(), out.data_ptr()
+    c.lane_rows = 0 if os.environ.get("BENCH_LL_SEARCH") else lane_rows.data_ptr()
     c.workspace, c.workspace_bytes = ws.data_ptr(), ws.numel()
     stream = torch.cuda.current_stream()
     sp = stream.cuda_stream

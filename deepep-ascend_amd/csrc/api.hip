@@ -539,6 +539,7 @@ int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* a, void* 
     p.packed_src_info = a->packed_recv_src_info;
     p.packed_layout_range = a->packed_recv_layout_range;
     p.cumulative_stats = a->cumulative_local_expert_recv_stats;
+    p.lane_slot = a->lane_rows;
     size_t off = 256;
     p.status = reinterpret_cast<int32_t*>(ws);
     p.done_counter = reinterpret_cast<uint32_t*>(ws + 4);
@@ -574,6 +575,7 @@ int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* a, void* st
     p.topk_weights = a->topk_weights;
     p.src_info = a->packed_recv_src_info;
     p.layout_range = a->packed_recv_layout_range;
+    p.lane_slot = a->lane_rows;
     p.out = static_cast<uint8_t*>(a->combined_x);
     p.status = reinterpret_cast<int32_t*>(a->workspace);
     hipError_t err = launch_ll_combine(p, static_cast<hipStream_t>(stream));

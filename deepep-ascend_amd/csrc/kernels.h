@@ -184,6 +184,7 @@ struct LLDispatchParams {
     int32_t* packed_src_info;
     int64_t* packed_layout_range;
     int32_t* cumulative_stats;
+    int32_t* lane_slot;      // optional [S*stride, K]: packed row (le * rows + slot) of every (token, lane), -1 none
     // workspace
     int32_t* status;
     uint32_t* done_counter;
@@ -203,6 +204,7 @@ struct LLCombineParams {
     const float* topk_weights;
     const int32_t* src_info;
     const int64_t* layout_range;
+    const int32_t* lane_slot;    // optional: what the dispatch recorded; replaces the search through src_info
     uint8_t* out;
     int32_t* status;
 };

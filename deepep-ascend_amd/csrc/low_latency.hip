@@ -142,7 +142,7 @@ __device__ __forceinline__ void ll_load_tile(const LLDispatchParams& p, int64_t 
 
 // Casts (FP8) and stores the tile to every (local expert, slot) named by lanes [0, K); t = token id within its source.
 template <int kPairs, bool kFp8>
-__device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int tile, int lane, int t, int le, int slot,
+__device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int64_t g, int tile, int lane, int t, int le, int slot,
                                               const vec16 (&in)[kPairs][2]) {
     const int rows_per_expert = p.R * p.M;
     const int row_bytes = p.H * 2;
@@ -151,6 +151,8 @@ __device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int til
         slot = -1;
     }
     if (tile == 0 && slot >= 0) p.packed_src_info[int64_t(le) * rows_per_expert + slot] = t;
+    // optional shortcut for combine: the packed row of every (token, lane)
+    if (tile == 0 && p.lane_slot != nullptr && lane < p.K) p.lane_slot[g * p.K + lane] = slot >= 0 ? le * rows_per_expert + slot : -1;
 
     vec16 out[kPairs];
     float my_scale = 0.f;
@@ -233,26 +235,24 @@ __global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchP
             slot = p.chunk_base[chunk * p.E_l + le] + p.pos_expert[g * p.K + lane];
         }
     }
-    ll_store_tile<kPairs, kFp8>(p, tile, lane, t, le, slot, in);
+    ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
 }
 
-// Single-kernel path for decode-sized calls.  Every workgroup (16 wavefronts) first rebuilds the complete
-// routing picture in LDS - one bit per (local expert, token), set from its own pass over all topk_idx rows
-// (tens of KB, L2 resident after the first workgroup) - so slots are prefix popcounts and no workgroup
-// waits for another: no second launch, no ticket, no global scan.  Workgroup 0 also publishes counts and
-// per-source ranges.  Each wavefront then moves one (token, column tile).
-constexpr int kFusedThreads = 256;
-constexpr int kFusedWaves = kFusedThreads / kWaveSize;
-
-template <int kPairs, bool kFp8>
+// Single-kernel path for decode-sized calls.  Every workgroup first rebuilds the complete routing picture in
+// LDS - one bit per (local expert, token), set from its own pass over all topk_idx rows (tens of KB, L2
+// resident) - so slots are prefix popcounts and no workgroup waits for another: no second launch, no ticket,
+// no global scan.  Workgroup 0 only publishes counts and per-source ranges; the wavefronts of the other
+// workgroups each move one (token, column tile).
+template <int kPairs, bool kFp8, int kFusedThreads>
 __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatchParams p, const int tiles) {
+    constexpr int kFusedWaves = kFusedThreads / kWaveSize;
     extern __shared__ uint64_t bits[];          // [E_l][words], bit g of row le: token g selects local expert le
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int total_tokens = p.S * p.src_token_stride;
     const int words = (total_tokens + 63) / 64;
 
     // This wavefront's work item; its payload loads go out before the routing pass.
-    const unsigned work = wave_work_index(blockIdx.x, kFusedWaves);
+    const unsigned work = blockIdx.x == 0 ? ~0u : wave_work_index(blockIdx.x - 1, kFusedWaves);
     const bool has_work = work < unsigned(total_tokens) * unsigned(tiles);
     const unsigned gu = has_work ? work / unsigned(tiles) : 0u;
     const int64_t g = gu;
@@ -266,61 +266,44 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     for (int i = tid; i < p.E_l * words; i += kFusedThreads) bits[i] = 0ull;
     __syncthreads();
     // Pass over the whole index table: 16-byte loads (two entries), fully coalesced, all of a thread's loads
-    // in flight at once; token and source of an entry come from float reciprocals (integer division by a
-    // run-time value is about 40 instructions, too slow with one wavefront per SIMD).
-    int flags = 0;
+    // in flight at once (addresses are clamped instead of predicated, so no load waits for another).  With
+    // random routing some lane of the wavefront holds a local expert in almost every step, so the "taken" side
+    // below runs every time: it is kept to a dozen instructions (no division, no returning atomic; range and
+    // duplicate checks are left to the wavefront that later moves the token).
     const int total_entries = total_tokens * p.K;
     const float rcp_k = 1.0f / float(p.K), rcp_stride = 1.0f / float(p.src_token_stride);
-    // Most entries name experts of other ranks: they are dismissed with three instructions on the raw words.
+    const bool ragged = p.num_tokens_per_src != nullptr;
     auto note = [&](int f, uint32_t lo, uint32_t hi) {
-        if (hi != 0u) return;                                    // negative: no selection
-        if (lo >= uint32_t(p.E)) {
-            flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
-            return;
-        }
         const uint32_t le = lo - uint32_t(p.expert_begin);
-        if (le >= uint32_t(p.E_l)) return;                       // another rank's expert
+        if (hi != 0u || le >= uint32_t(p.E_l) || lo >= uint32_t(p.E)) return;   // no selection / another rank's expert
         const int gg = small_div(f, rcp_k);
-        const int ss = small_div(gg, rcp_stride);
-        if (gg - ss * p.src_token_stride >= tokens_of_source(p, ss)) return;
-        const unsigned long long bit = 1ull << (gg & 63);
-        const unsigned long long old =
-            atomicOr(reinterpret_cast<unsigned long long*>(&bits[int(le) * words + (gg >> 6)]), bit);
-        if (old & bit) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+        if (ragged) {
+            const int ss = small_div(gg, rcp_stride);
+            if (gg - ss * p.src_token_stride >= tokens_of_source(p, ss)) return;
+        }
+        atomicOr(reinterpret_cast<unsigned long long*>(&bits[int(le) * words + (gg >> 6)]), 1ull << (gg & 63));
     };
     const bool aligned16 = (reinterpret_cast<uintptr_t>(p.topk_idx) & 15) == 0;
     const int pairs_total = aligned16 ? total_entries / 2 : 0;
     const vec16* idx2 = reinterpret_cast<const vec16*>(p.topk_idx);
-    for (int q0 = tid; q0 < pairs_total; q0 += kFusedThreads * 16) {
-        vec16 v[16];
+    constexpr int kBatch = 8;
+    for (int q0 = tid; q0 < pairs_total; q0 += kFusedThreads * kBatch) {
+        vec16 v[kBatch];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            const int q = q0 + u * kFusedThreads;
-            v[u] = q < pairs_total ? idx2[q] : vec16{0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-        }
+        for (int u = 0; u < kBatch; ++u) v[u] = idx2[min(q0 + u * kFusedThreads, pairs_total - 1)];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
+        for (int u = 0; u < kBatch; ++u) {
             const int q = q0 + u * kFusedThreads;
-            if (q >= pairs_total) continue;
-            note(2 * q, v[u].x, v[u].y);
-            note(2 * q + 1, v[u].z, v[u].w);
+            const uint32_t dead = q < pairs_total ? 0u : 0xffffffffu;      // entries past the end read as "none"
+            note(2 * q, v[u].x, v[u].y | dead);
+            note(2 * q + 1, v[u].z, v[u].w | dead);
         }
     }
     for (int f = 2 * pairs_total + tid; f < total_entries; f += kFusedThreads) {
         const uint64_t raw = uint64_t(p.topk_idx[f]);
         note(f, uint32_t(raw), uint32_t(raw >> 32));
     }
-    if (flags != 0 && blockIdx.x == 0) atomicOr(p.status, flags);
     __syncthreads();
-
-    // rows of expert le that come from tokens [0, g): prefix popcount
-    auto rows_before = [&](int le, int gpos) {
-        const uint64_t* row = bits + le * words;
-        int n = 0;
-        for (int wd = 0; wd < (gpos >> 6); ++wd) n += __popcll(row[wd]);
-        if (gpos & 63) n += __popcll(row[gpos >> 6] & ((1ull << (gpos & 63)) - 1ull));
-        return n;
-    };
 
     if (blockIdx.x == 0) {
         // counts and per-source ranges: one walk over each expert's words, cut at the source boundaries
@@ -343,18 +326,35 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
             p.packed_count[le] = running;
             if (p.cumulative_stats != nullptr) p.cumulative_stats[le] += running;
         }
+        return;
     }
     if (!live) return;
 
-    int le = -1, slot = -1;
+    // rows of expert le that come from tokens [0, g): prefix popcount
+    auto rows_before = [&](int le, int gpos) {
+        const uint64_t* row = bits + le * words;
+        int n = 0;
+        for (int wd = 0; wd < (gpos >> 6); ++wd) n += __popcll(row[wd]);
+        if (gpos & 63) n += __popcll(row[gpos >> 6] & ((1ull << (gpos & 63)) - 1ull));
+        return n;
+    };
+    int le = -1, slot = -1, flags = 0;
     if (lane < p.K) {
         const int64_t raw = p.topk_idx[g * p.K + lane];
+        if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
         if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) {
             le = int(raw) - p.expert_begin;
             slot = rows_before(le, int(g));
         }
     }
-    ll_store_tile<kPairs, kFp8>(p, tile, lane, t, le, slot, in);
+    if (tile == 0) {
+        for (int j = 0; j < p.K; ++j) {
+            const int other = read_lane(le, j);
+            if (lane != j && le >= 0 && le == other) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+        }
+        if (flags != 0) atomicOr(p.status, flags);
+    }
+    ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
 }
 
 // Weighted reduce: one wavefront per (token, column tile of kVecs * 512 channels).
@@ -374,58 +374,65 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
     const int rows_per_expert = p.R * p.M;
     const int row_bytes = p.H * 2;
 
-    int le = -1;
+    int le = -1, recorded = -1;
     float w = 0.f;
     if (lane < p.K) {
         const int64_t raw = p.topk_idx[g * p.K + lane];
-        if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) le = int(raw) - p.expert_begin;
+        if (p.lane_slot != nullptr) recorded = p.lane_slot[g * p.K + lane];    // issued together with the index load
         w = p.topk_weights[g * p.K + lane];
+        if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) le = int(raw) - p.expert_begin;
     }
 
-    // Find the packed row of every lane: the rows this source rank put into the lane's expert are
-    // [begin, begin + count); the wavefront scans their source-token ids for this token.  Ranges are loaded by
-    // the lanes in parallel and, for the first 8 lanes and up to 128 rows each, all id loads are issued before
-    // the first comparison: two memory round trips instead of two per lane.
-    int my_begin = 0, my_count = 0;
-    if (le >= 0) {
-        const int64_t range = p.layout_range[int64_t(le) * p.R + src_rank];
-        my_begin = int(range >> 32);
-        my_count = min(int(range & 0xffffffff), rows_per_expert - my_begin);
-    }
     int row_of_lane = -1;
-    constexpr int kFast = 8;
-    int ids0[kFast], ids1[kFast];
-#pragma unroll
-    for (int k = 0; k < kFast; ++k) {
-        const int kle = read_lane(le, k), kb = read_lane(my_begin, k), kc = read_lane(my_count, k);
-        const int32_t* ids = p.src_info + int64_t(kle < 0 ? 0 : kle) * rows_per_expert + kb;
-        ids0[k] = (k < p.K && kle >= 0 && lane < kc) ? ids[lane] : -1;
-        ids1[k] = (k < p.K && kle >= 0 && lane + kWaveSize < kc) ? ids[lane + kWaveSize] : -1;
-    }
-#pragma unroll
-    for (int k = 0; k < kFast; ++k) {
-        const int kb = read_lane(my_begin, k);
-        const uint64_t m0 = __ballot(ids0[k] == t), m1 = __ballot(ids1[k] == t);
-        const int found = m0 ? kb + __builtin_ctzll(m0) : m1 ? kb + kWaveSize + __builtin_ctzll(m1) : -1;
-        if (lane == k) row_of_lane = found;
-    }
-    // Lanes past the eighth, and ranges longer than 128 rows.
-    for (int k = 0; k < p.K; ++k) {
-        const int kle = read_lane(le, k), kb = read_lane(my_begin, k), kc = read_lane(my_count, k);
-        const int have = read_lane(row_of_lane, k);
-        if (kle < 0 || have >= 0) continue;
-        const int first = k < kFast ? 2 * kWaveSize : 0;
-        int found = -1;
-        for (int base = first; base < kc; base += kWaveSize) {
-            const int i = base + lane;
-            const bool hit = i < kc && p.src_info[int64_t(kle) * rows_per_expert + kb + i] == t;
-            const uint64_t m = __ballot(hit);
-            if (m) {
-                found = kb + base + __builtin_ctzll(m);
-                break;
-            }
+    if (p.lane_slot != nullptr) {
+        // the dispatch that produced the handle also recorded the packed row of every (token, lane)
+        if (le >= 0 && recorded >= le * rows_per_expert && recorded < (le + 1) * rows_per_expert)
+            row_of_lane = recorded - le * rows_per_expert;
+    } else {
+        // Find the packed row of every lane: the rows this source rank put into the lane's expert are
+        // [begin, begin + count); the wavefront scans their source-token ids for this token.  Ranges are loaded by
+        // the lanes in parallel and, for the first 8 lanes and up to 128 rows each, all id loads are issued before
+        // the first comparison: two memory round trips instead of two per lane.
+        int my_begin = 0, my_count = 0;
+        if (le >= 0) {
+            const int64_t range = p.layout_range[int64_t(le) * p.R + src_rank];
+            my_begin = int(range >> 32);
+            my_count = min(int(range & 0xffffffff), rows_per_expert - my_begin);
         }
-        if (lane == k) row_of_lane = found;
+        constexpr int kFast = 8;
+        int ids0[kFast], ids1[kFast];
+    #pragma unroll
+        for (int k = 0; k < kFast; ++k) {
+            const int kle = read_lane(le, k), kb = read_lane(my_begin, k), kc = read_lane(my_count, k);
+            const int32_t* ids = p.src_info + int64_t(kle < 0 ? 0 : kle) * rows_per_expert + kb;
+            ids0[k] = (k < p.K && kle >= 0 && lane < kc) ? ids[lane] : -1;
+            ids1[k] = (k < p.K && kle >= 0 && lane + kWaveSize < kc) ? ids[lane + kWaveSize] : -1;
+        }
+    #pragma unroll
+        for (int k = 0; k < kFast; ++k) {
+            const int kb = read_lane(my_begin, k);
+            const uint64_t m0 = __ballot(ids0[k] == t), m1 = __ballot(ids1[k] == t);
+            const int found = m0 ? kb + __builtin_ctzll(m0) : m1 ? kb + kWaveSize + __builtin_ctzll(m1) : -1;
+            if (lane == k) row_of_lane = found;
+        }
+        // Lanes past the eighth, and ranges longer than 128 rows.
+        for (int k = 0; k < p.K; ++k) {
+            const int kle = read_lane(le, k), kb = read_lane(my_begin, k), kc = read_lane(my_count, k);
+            const int have = read_lane(row_of_lane, k);
+            if (kle < 0 || have >= 0) continue;
+            const int first = k < kFast ? 2 * kWaveSize : 0;
+            int found = -1;
+            for (int base = first; base < kc; base += kWaveSize) {
+                const int i = base + lane;
+                const bool hit = i < kc && p.src_info[int64_t(kle) * rows_per_expert + kb + i] == t;
+                const uint64_t m = __ballot(hit);
+                if (m) {
+                    found = kb + base + __builtin_ctzll(m);
+                    break;
+                }
+            }
+            if (lane == k) row_of_lane = found;
+        }
     }
 
     float acc[kVecs][8];
@@ -481,14 +488,31 @@ hipError_t launch_move(const LLDispatchParams& p, hipStream_t stream) {
 
 }  // namespace
 
-template <int kPairs>
+template <int kPairs, int kFusedThreads>
 hipError_t launch_fused(const LLDispatchParams& p, hipStream_t stream, size_t lds) {
+    constexpr int kFusedWaves = kFusedThreads / kWaveSize;
     const int tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
     const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
-    const unsigned blocks = unsigned((waves + kFusedWaves - 1) / kFusedWaves);
-    if (p.use_fp8) hipLaunchKernelGGL((ll_fused_kernel<kPairs, true>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
-    else hipLaunchKernelGGL((ll_fused_kernel<kPairs, false>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+    const unsigned blocks = unsigned((waves + kFusedWaves - 1) / kFusedWaves) + 1;   // workgroup 0 publishes only
+    if (p.use_fp8)
+        hipLaunchKernelGGL((ll_fused_kernel<kPairs, true, kFusedThreads>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+    else
+        hipLaunchKernelGGL((ll_fused_kernel<kPairs, false, kFusedThreads>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
     return hipGetLastError();
+}
+
+template <int kFusedThreads>
+hipError_t launch_fused_by_width(const LLDispatchParams& p, hipStream_t stream, size_t lds) {
+    // Up to 4 x 1024 channels per wavefront: fatter wavefronts spend longer in the (serial) cast than the
+    // extra wavefronts cost to launch.
+    const int segs = (p.H + 1023) / 1024;
+    const char* env = getenv("DEEP_EP_HIP_LL_PAIRS");
+    const int forced = env != nullptr ? atoi(env) : 0;
+    switch (forced == 1 || forced == 2 || forced == 4 ? forced : segs <= 1 ? 1 : segs <= 2 ? 2 : 4) {
+        case 1: return launch_fused<1, kFusedThreads>(p, stream, lds);
+        case 2: return launch_fused<2, kFusedThreads>(p, stream, lds);
+        default: return launch_fused<4, kFusedThreads>(p, stream, lds);
+    }
 }
 
 hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
@@ -498,14 +522,11 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
     const size_t fused_lds = size_t(p.E_l) * ((total_tokens + 63) / 64) * sizeof(uint64_t);
     if (total_tokens <= 2048 && fused_lds <= 32 * 1024 && getenv("DEEP_EP_HIP_LL_TWO_KERNELS") == nullptr)
     {
-        // Up to 4 x 1024 channels per wavefront: fatter wavefronts spend longer in the (serial) cast than the
-        // extra wavefronts cost to launch.
-        const int segs = (p.H + 1023) / 1024;
-        switch (segs <= 1 ? 1 : segs <= 2 ? 2 : 4) {
-            case 1: return launch_fused<1>(p, stream, fused_lds);
-            case 2: return launch_fused<2>(p, stream, fused_lds);
-            default: return launch_fused<4>(p, stream, fused_lds);
-        }
+        const char* env = getenv("DEEP_EP_HIP_LL_THREADS");
+        const int threads = env != nullptr ? atoi(env) : 512;
+        if (threads == 256) return launch_fused_by_width<256>(p, stream, fused_lds);
+        if (threads == 1024) return launch_fused_by_width<1024>(p, stream, fused_lds);
+        return launch_fused_by_width<512>(p, stream, fused_lds);
     }
 
     const int chunks_per_src = (p.src_token_stride + kThreads - 1) / kThreads;
@@ -522,13 +543,16 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
 
 hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream) {
     if (p.S <= 0 || p.src_token_stride <= 0) return hipSuccess;
-    const int vecs = (p.H * 2 <= 1024) ? 1 : 4;
+    const char* env = getenv("DEEP_EP_HIP_LL_COMBINE_VECS");
+    int vecs = env != nullptr ? atoi(env) : 0;
+    if (vecs != 1 && vecs != 2 && vecs != 4)
+        vecs = (p.H * 2 <= 1024 || int64_t(p.S) * p.src_token_stride <= 4096) ? 1 : 4;   // decode sizes: many small wavefronts
     const int tiles = (p.H * 2 + vecs * 1024 - 1) / (vecs * 1024);
     const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
     const unsigned blocks = unsigned((waves + kMoveWaves - 1) / kMoveWaves);
     if (vecs == 1) hipLaunchKernelGGL(ll_combine_kernel<1>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
-    else if (vecs == 4) hipLaunchKernelGGL(ll_combine_kernel<4>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
-    else hipLaunchKernelGGL(ll_combine_kernel<7>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    else if (vecs == 2) hipLaunchKernelGGL(ll_combine_kernel<2>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    else hipLaunchKernelGGL(ll_combine_kernel<4>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
     return hipGetLastError();
 }
 

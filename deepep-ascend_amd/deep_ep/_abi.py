@@ -166,6 +166,7 @@ class LLDispatchArgs(Structure):
         ("packed_recv_src_info", c_void_p),
         ("packed_recv_layout_range", c_void_p),
         ("cumulative_local_expert_recv_stats", c_void_p),
+        ("lane_rows", c_void_p),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
     ]
@@ -184,6 +185,7 @@ class LLCombineArgs(Structure):
         ("topk_weights", c_void_p),
         ("packed_recv_src_info", c_void_p),
         ("packed_recv_layout_range", c_void_p),
+        ("lane_rows", c_void_p),
         ("combined_x", c_void_p),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),

@@ -45,6 +45,7 @@ class Buffer:
                                         False, True, True, 0, 0, 300, 100, explicitly_destroy)
         self._ll_workspace: Optional[torch.Tensor] = None
         self._ll_combine_buffer: Optional[torch.Tensor] = None
+        self._ll_lane_rows = None
 
     def destroy(self) -> None:
         assert self.explicitly_destroy, '`explicitly_destroy` flag must be set'
@@ -219,6 +220,7 @@ class Buffer:
             # ranges of source ranks that do not send in this call stay (begin 0, count 0)
             packed_recv_layout_range = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
             packed_recv_count = torch.empty((E_l,), dtype=torch.int32, device=dev)
+            lane_rows = torch.empty((S * T, K), dtype=torch.int32, device=dev)
             packed_recv_x_scales = None
             if use_fp8 and use_ue8m0:
                 assert H % 512 == 0
@@ -241,6 +243,7 @@ class Buffer:
                 args.packed_recv_src_info = _abi.ptr(packed_recv_src_info)
                 args.packed_recv_layout_range = _abi.ptr(packed_recv_layout_range)
                 args.cumulative_local_expert_recv_stats = _abi.ptr(cumulative_local_expert_recv_stats)
+                args.lane_rows = _abi.ptr(lane_rows)
                 args.workspace, args.workspace_bytes = _abi.ptr(ws), ws.numel()
                 _abi.check(_abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(args), run_stream.cuda_stream),
                            "low_latency_dispatch")
@@ -250,6 +253,9 @@ class Buffer:
                    packed_recv_layout_range, cumulative_local_expert_recv_stats)
         event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
         handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H, num_experts)
+        # The handle keeps the reference's five fields; the packed row of every (token, lane) rides beside it and
+        # lets the combine of this very handle skip its search through src_info.
+        self._ll_lane_rows = (packed_recv_src_info, lane_rows, tuple(topk_idx.shape)) if T > 0 else None
         recv = (packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x
         hook = (lambda: None) if return_recv_hook else None
         return recv, packed_recv_count, handle, EventOverlap(event, tensors if async_finish else None), hook
@@ -317,6 +323,9 @@ class Buffer:
                 args.x, args.topk_idx, args.topk_weights = _abi.ptr(x), _abi.ptr(topk_idx), _abi.ptr(topk_weights)
                 args.packed_recv_src_info = _abi.ptr(src_info)
                 args.packed_recv_layout_range = _abi.ptr(layout_range)
+                cached = self._ll_lane_rows
+                if cached is not None and cached[0] is src_info and cached[2] == tuple(topk_idx.shape):
+                    args.lane_rows = _abi.ptr(cached[1])
                 args.combined_x = _abi.ptr(combined_x)
                 args.workspace, args.workspace_bytes = _abi.ptr(ws), ws.numel()
                 _abi.check(_abi.lib.deep_ep_hip_launch_ll_combine(ctypes.byref(args), run_stream.cuda_stream),

@@ -280,6 +280,10 @@ typedef struct {
     int32_t* packed_recv_src_info;      /* [num_local_experts, rows] out */
     int64_t* packed_recv_layout_range;  /* [num_local_experts, num_ranks] out: (begin<<32)|count */
     int32_t* cumulative_local_expert_recv_stats; /* [num_local_experts] += counts, or NULL */
+    int32_t* lane_rows;                 /* optional out [num_src_ranks * src_token_stride, num_topk]: e * rows + slot of
+                                           the packed row each (token, lane) went to, -1 if none.  Not part of the
+                                           reference's handle; passing it to the combine saves the search through
+                                           packed_recv_src_info */
     void* workspace;
     uint64_t workspace_bytes;
 } deep_ep_hip_ll_dispatch_args;
@@ -300,6 +304,7 @@ typedef struct {
     const float* topk_weights;          /* [num_src_ranks * src_token_stride, num_topk] */
     const int32_t* packed_recv_src_info;
     const int64_t* packed_recv_layout_range;
+    const int32_t* lane_rows;           /* optional: lane_rows of the dispatch that made the handle */
     void* combined_x;                   /* bf16 [num_src_ranks * src_token_stride, hidden] out; rows past a
                                            source's token count are left untouched */
     void* workspace;

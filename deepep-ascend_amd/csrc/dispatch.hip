@@ -41,45 +41,62 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
     Route r{-1, -1, -1, -1, -1, 0.f};
     const int n = p.R + p.E;
     const int chunk = t / kLayoutChunk;
-    int slot = -1, epos = -1;
+
+    // ---- issue every load that does not depend on another one, then consume: one memory round trip ----
+    int64_t raw = -1;
+    uint8_t mask_byte = 0;
+    uint32_t word = 0xffffffffu;     // cached: handle slot (-1 = none); otherwise the packed positions of the layout pass
+    const bool rank_lanes_cached = p.cached && p.rank_lanes;
     if (lane < p.K) {
-        if (p.cached && p.rank_lanes) {
+        const int64_t at = int64_t(t) * p.K + lane;
+        if (p.route_mask != nullptr) mask_byte = p.route_mask[at];
+        else if (!rank_lanes_cached) raw = p.topk_idx[at];
+        if (p.topk_weights != nullptr) r.w = p.topk_weights[at];
+        const uint32_t* words = p.cached ? reinterpret_cast<const uint32_t*>(p.cached_slot) : p.pos;
+        word = words[at];
+    }
+    // Light mode: per-rank chunk counts, flattened [R][chunks_padded]; lane L holds entries [L * per, (L + 1) * per).
+    const int per = p.flat_per;
+    vec16 counts[4];
+    if (p.light) {
+        const int nflat = p.R * p.chunks_padded;
+        // addresses are clamped instead of predicated (and masked only when consumed) so that the loads do not
+        // wait for each other
+#pragma unroll
+        for (int u = 0; u < 4; ++u) counts[u] = load16(p.chunk_counts_t + min(lane * per + u * 4, nflat - 4));
+    }
+
+    int slot = -1, epos = -1;
+    const int cached_v = int(word);
+    const uint32_t packed = word;
+    if (lane < p.K) {
+        if (rank_lanes_cached) {
             // V1 cached dispatch: send_head names the receive row of every (token, rank) pair
-            const int v = p.cached_slot[int64_t(t) * p.K + lane];
-            if (v >= 0) r.e = lane;
-            slot = v;
+            if (cached_v >= 0) r.e = lane;
+            slot = cached_v;
         } else {
-            const int64_t raw = p.route_mask != nullptr
-                                    ? (p.route_mask[int64_t(t) * p.K + lane] != 0 ? int64_t(lane) : int64_t(-1))
-                                    : p.topk_idx[int64_t(t) * p.K + lane];
+            if (p.route_mask != nullptr) raw = mask_byte != 0 ? int64_t(lane) : int64_t(-1);
             if (raw >= 0 && raw < p.E) r.e = int(raw);
-            if (p.topk_weights != nullptr) r.w = p.topk_weights[int64_t(t) * p.K + lane];
             if (p.cached) {
-                const int v = p.cached_slot[int64_t(t) * p.K + lane];
-                slot = v >= 0 ? v - p.rank_idx * p.M : -1;
+                slot = cached_v >= 0 ? cached_v - p.rank_idx * p.M : -1;
             } else {
-                const uint32_t packed = p.pos[int64_t(t) * p.K + lane];
                 slot = (packed & 0xffffu) == 0xffffu ? -1 : int(packed & 0xffffu);
                 epos = int(packed >> 16);
             }
         }
     }
-    if (r.e >= 0) r.d = small_div(r.e, 1.0f / float(p.E_l));
+    if (r.e >= 0) r.d = small_div(r.e, p.rcp_E_l);
     else slot = -1;
     if (p.light) {
-        // Exclusive prefix of the per-rank chunk counts in (rank, chunk) order: lane L scans entries
-        // [L * per, (L + 1) * per) of the flattened [R][chunks_padded] table, a wave scan joins the lanes.
+        // Exclusive prefix of the per-rank chunk counts in (rank, chunk) order; a wave scan joins the lanes.
         // The prefix at (d, chunk) is at once the start of bucket d and the rows that earlier chunks put
         // into it, so no other table is needed.
-        const int per = p.flat_per;
-        const int nflat = p.R * p.chunks_padded;
         int ex[16];
         int sum = 0;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            vec16 v{0, 0, 0, 0};
-            if (u * 4 < per && lane * per + u * 4 < nflat)
-                v = load16(p.chunk_counts_t + lane * per + u * 4);
+            const bool held = u * 4 < per && lane * per + u * 4 < p.R * p.chunks_padded;
+            const vec16 v = held ? counts[u] : vec16{0, 0, 0, 0};
             ex[4 * u] = sum; sum += int(v.x);
             ex[4 * u + 1] = sum; sum += int(v.y);
             ex[4 * u + 2] = sum; sum += int(v.z);
@@ -477,6 +494,7 @@ int tuning_override(const char* name) {
 
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
+    p.rcp_E_l = 1.0f / float(p.E_l);
     {
         const char* v = getenv("DEEP_EP_HIP_XCD_REMAP");
         p.xcd_remap = v != nullptr ? atoi(v) : 0;

@@ -80,6 +80,7 @@ struct MoveParams {
     float* recv_topk_weights;
     int64_t recv_capacity, expanded_capacity;
     int T, H, K, E, R, E_l, rank_idx, M;
+    float rcp_E_l;       // 1 / E_l (set by the launcher)
     int cached, do_expand;
     int payload;         // DEEP_EP_HIP_PAYLOAD_*
     int row_bytes;       // input row bytes

@@ -60,7 +60,6 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     off = 256;
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
     w.chunk_counts = off;  off = align_up(off + chunks_padded * n * 4, 256);
-    w.chunk_base = off;    off = align_up(off + chunks * n * 4, 256);
     w.pos = off;           off = align_up(off + lanes * 4, 256);
     w.total_bytes = off;
     return w;
@@ -107,7 +106,6 @@ int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
     p.status = reinterpret_cast<int32_t*>(ws + w.status);
     p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
     p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
-    p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
     hipError_t err = launch_layout_kernel(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "layout launch");
     return DEEP_EP_HIP_OK;
@@ -180,15 +178,17 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
     pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
 
-    // Light mode: when layout and move run in one call on the compact layout, the layout kernel only
-    // counts; every wavefront of the move kernel prefix-sums the (small) per-rank part of the chunk
-    // counts itself and workgroup 0 publishes the handle tensors.  That removes the serial tail of the
-    // layout kernel (ticket, fences, scan by the last workgroup) from the critical path.
+    // The layout kernel leaves per-chunk totals [bucket][chunk]; the wavefronts of the move kernel prefix-sum
+    // what they need from them (the whole per-rank part at once while R * chunks <= 1024, single rows
+    // otherwise).  When layout and move run in one call on the compact layout ("light"), the layout kernel
+    // only counts and workgroup 0 of the move kernel publishes the handle tensors: no ticket, no fences and
+    // no serial tail on the critical path.
     const int chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
     const int chunks_padded = (chunks + 3) / 4 * 4;
     const int flat = R * chunks_padded;
     const int flat_per = flat <= 256 ? 4 : flat <= 512 ? 8 : 16;
-    const bool light = do_layout && do_move && !a->do_expand && T > 0 && flat <= 1024 && (R + E) <= 512 &&
+    const bool flat_ok = T > 0 && flat <= 1024 && !a->cached;
+    const bool light = do_layout && do_move && !a->do_expand && flat_ok && (R + E) <= 512 &&
                        getenv("DEEP_EP_HIP_NO_LIGHT_LAYOUT") == nullptr;
 
     if (do_layout) {
@@ -196,14 +196,12 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         p.topk_idx = a->topk_idx;
         p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
         p.light = light ? 1 : 0;
-        p.chunks_padded = chunks_padded;
         p.copied_topk_idx = a->copied_topk_idx;
         p.pub = pub;
         p.status = status;
         p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
         p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
-        p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
-        p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
+            p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
         hipError_t err = launch_layout_kernel(p, stream);
         if (err != hipSuccess) return hip_fail(err, "dispatch layout launch");
     }
@@ -217,7 +215,6 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         m.topk_idx = a->topk_idx;
         m.topk_weights = a->topk_weights;
         m.pos = reinterpret_cast<const uint32_t*>(ws + w.pos);
-        m.chunk_base = reinterpret_cast<const int32_t*>(ws + w.chunk_base);
         m.expert_start = reinterpret_cast<const int32_t*>(ws + w.expert_start);
         m.cached_slot = a->dst_buffer_slot_idx;
         m.dst_buffer_slot_idx = a->dst_buffer_slot_idx;
@@ -236,7 +233,8 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         m.do_expand = a->do_expand ? 1 : 0;
         m.payload = a->payload;
         m.row_bytes = H * elem_in;
-        m.light = light ? 1 : 0;
+        m.flat = flat_ok ? 1 : 0;
+        m.publish = light ? 1 : 0;
         m.chunks_padded = chunks_padded;
         m.flat_per = flat_per;
         m.chunk_counts_t = reinterpret_cast<const int32_t*>(ws + w.chunk_counts);
@@ -368,7 +366,8 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
     const int chunks_padded = (chunks + 3) / 4 * 4;
     const int flat = R * chunks_padded;
     const int flat_per = flat <= 256 ? 4 : flat <= 512 ? 8 : 16;
-    const bool light = do_layout && do_move && T > 0 && flat <= 1024 && (R + E) <= 512 &&
+    const bool flat_ok = T > 0 && flat <= 1024 && !a->cached;
+    const bool light = do_layout && do_move && flat_ok && (R + E) <= 512 &&
                        getenv("DEEP_EP_HIP_NO_LIGHT_LAYOUT") == nullptr;
 
     if (do_layout) {
@@ -377,13 +376,11 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         p.route_mask = with_topk ? nullptr : a->is_token_in_rank;
         p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
         p.light = light ? 1 : 0;
-        p.chunks_padded = chunks_padded;
         p.pub = pub;
         p.status = status;
         p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
         p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
-        p.chunk_base = reinterpret_cast<int32_t*>(ws + w.chunk_base);
-        p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
+            p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
         hipError_t err = launch_layout_kernel(p, stream);
         if (err != hipSuccess) return hip_fail(err, "intranode dispatch layout launch");
 
@@ -411,7 +408,6 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.route_mask = (with_topk || a->cached) ? nullptr : a->is_token_in_rank;
         m.topk_weights = a->topk_weights;
         m.pos = reinterpret_cast<const uint32_t*>(ws + w.pos);
-        m.chunk_base = reinterpret_cast<const int32_t*>(ws + w.chunk_base);
         m.expert_start = reinterpret_cast<const int32_t*>(ws + w.expert_start);
         m.cached_slot = a->send_head;
         m.dst_buffer_slot_idx = nullptr;
@@ -430,7 +426,8 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.do_expand = 0;
         m.payload = a->payload;
         m.row_bytes = H * elem_in;
-        m.light = light ? 1 : 0;
+        m.flat = flat_ok ? 1 : 0;
+        m.publish = light ? 1 : 0;
         m.chunks_padded = chunks_padded;
         m.flat_per = flat_per;
         m.chunk_counts_t = reinterpret_cast<const int32_t*>(ws + w.chunk_counts);

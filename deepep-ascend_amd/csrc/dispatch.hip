@@ -39,7 +39,6 @@ struct Route {
 
 __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int lane, bool first_tile) {
     Route r{-1, -1, -1, -1, -1, 0.f};
-    const int n = p.R + p.E;
     const int chunk = t / kLayoutChunk;
 
     // ---- issue every load that does not depend on another one, then consume: one memory round trip ----
@@ -55,15 +54,18 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
         const uint32_t* words = p.cached ? reinterpret_cast<const uint32_t*>(p.cached_slot) : p.pos;
         word = words[at];
     }
-    // Light mode: per-rank chunk counts, flattened [R][chunks_padded]; lane L holds entries [L * per, (L + 1) * per).
+    // Flat mode: per-rank chunk counts, flattened [R][chunks_padded]; lane L holds entries [L * per, (L + 1) * per).
     const int per = p.flat_per;
     vec16 counts[4];
-    if (p.light) {
+    if (p.flat) {
         const int nflat = p.R * p.chunks_padded;
         // addresses are clamped instead of predicated (and masked only when consumed) so that the loads do not
         // wait for each other
 #pragma unroll
-        for (int u = 0; u < 4; ++u) counts[u] = load16(p.chunk_counts_t + min(lane * per + u * 4, nflat - 4));
+        for (int u = 0; u < 4; ++u) {
+            counts[u] = vec16{0, 0, 0, 0};
+            if (u * 4 < per) counts[u] = load16(p.chunk_counts_t + min(lane * per + u * 4, nflat - 4));   // uniform branch
+        }
     }
 
     int slot = -1, epos = -1;
@@ -87,7 +89,7 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
     }
     if (r.e >= 0) r.d = small_div(r.e, p.rcp_E_l);
     else slot = -1;
-    if (p.light) {
+    if (p.flat) {
         // Exclusive prefix of the per-rank chunk counts in (rank, chunk) order; a wave scan joins the lanes.
         // The prefix at (d, chunk) is at once the start of bucket d and the rows that earlier chunks put
         // into it, so no other table is needed.
@@ -129,7 +131,8 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
         if (p.slot_is_row) {
             r.row_c = slot;
         } else {
-            if (!p.cached) slot += p.chunk_base[int64_t(chunk) * n + r.d];
+            // large R * chunks: each master lane sums its own bucket's row
+            if (!p.cached) slot += row_prefix(p.chunk_counts_t, p.chunks_padded, r.d, chunk);
             r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
         }
     }
@@ -152,12 +155,15 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
         const int rj = read_lane(r.row_c, j);
         if (r.d >= 0 && dj == r.d && rj >= 0) r.my_row = rj;
     }
+    int expert_rows_before = 0;
+    if (p.do_expand && !p.cached)    // rows that earlier chunks put into this lane's expert
+        expert_rows_before = row_prefix(p.chunk_counts_t, p.chunks_padded, p.R + (r.e >= 0 ? r.e : 0), chunk);
     if (p.do_expand && r.e >= 0) {
         if (p.cached) {
             if (r.my_row >= 0 && r.my_row < p.recv_capacity)
                 r.erow = p.recv_src_metadata[int64_t(r.my_row) * (p.K + 2) + 2 + lane];
         } else {
-            r.erow = p.expert_start[r.e] + p.chunk_base[int64_t(chunk) * n + p.R + r.e] + epos;
+            r.erow = p.expert_start[r.e] + expert_rows_before + epos;
         }
     }
     return r;
@@ -251,31 +257,17 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
     return __ballot(row_of_lane >= 0);
 }
 
-// Light mode: workgroup 0 sums the transposed chunk counts and publishes the handle tensors.  Every thread
-// of the workgroup must call this before any early exit.
+// Layout and move in one call: workgroup 0 sums the transposed chunk counts and publishes the handle tensors.
+// Every thread of the workgroup must call this before any early exit.
 __device__ __forceinline__ void publish_from_chunk_counts(const MoveParams& p) {
-    extern __shared__ int publish_lds[];          // [R + E] totals, [2 * E] scratch, then per-wave scan slots
-    const int n = p.R + p.E;
-    int* totals = publish_lds;
-    int* scratch = totals + n;
-    int* scan_tmp = scratch + 2 * p.E;
-    for (int j = threadIdx.x; j < n; j += kThreads) {
-        const int32_t* row = p.chunk_counts_t + int64_t(j) * p.chunks_padded;
-        int sum = 0;
-        for (int c = 0; c < p.chunks_padded; c += 4) {
-            const vec16 v = load16(row + c);
-            sum += int(v.x) + int(v.y) + int(v.z) + int(v.w);
-        }
-        totals[j] = sum;
-    }
-    __syncthreads();
-    publish_counts<kThreads>(p.pub, totals, scratch, scan_tmp);
+    extern __shared__ int publish_lds[];
+    publish_from_transposed_counts<kThreads>(p.pub, p.chunk_counts_t, p.chunks_padded, publish_lds);
 }
 
 // ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
 template <int kVecs>
 __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
-    if (p.light && blockIdx.x == 0) publish_from_chunk_counts(p);
+    if (p.publish && blockIdx.x == 0) publish_from_chunk_counts(p);
     const int lane = threadIdx.x & 63;
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
@@ -318,7 +310,7 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
 template <int kPairs>
 __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
-    if (p.light && blockIdx.x == 0) publish_from_chunk_counts(p);
+    if (p.publish && blockIdx.x == 0) publish_from_chunk_counts(p);
     const int lane = threadIdx.x & 63;
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
@@ -463,8 +455,8 @@ __global__ __launch_bounds__(kThreads) void fill_tail_kernel(const FillTailParam
         p.recv_topk_idx[i] = -1;
 }
 
-size_t publish_lds_bytes(const MoveParams& p) {
-    return p.light ? size_t(p.R + 3 * p.E + kWavesPerBlock) * sizeof(int) : 0;
+size_t move_lds_bytes(const MoveParams& p) {
+    return p.publish ? publish_lds_bytes(p.R, p.E, kThreads) : 0;
 }
 
 template <int kVecs>
@@ -472,7 +464,7 @@ hipError_t launch_copy(MoveParams p, hipStream_t stream) {
     p.tiles = (p.row_bytes + kVecs * 1024 - 1) / (kVecs * 1024);
     const int64_t waves = int64_t(p.T) * p.tiles;
     const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(dispatch_copy_kernel<kVecs>, dim3(blocks), dim3(kThreads), publish_lds_bytes(p), stream, p);
+    hipLaunchKernelGGL(dispatch_copy_kernel<kVecs>, dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 
@@ -481,7 +473,7 @@ hipError_t launch_cast(MoveParams p, hipStream_t stream) {
     p.tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
     const int64_t waves = int64_t(p.T) * p.tiles;
     const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(dispatch_cast_kernel<kPairs>, dim3(blocks), dim3(kThreads), publish_lds_bytes(p), stream, p);
+    hipLaunchKernelGGL(dispatch_cast_kernel<kPairs>, dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 

@@ -14,8 +14,7 @@ struct WorkspaceLayout {
     size_t done_counter;   // uint32: workgroups of the layout kernel that have finished
     size_t totals;         // int32[2]: total compact rows, total expanded rows (incl. padding)
     size_t expert_start;   // int32[E]: first expanded row of each expert
-    size_t chunk_counts;   // int32[C][R+E]
-    size_t chunk_base;     // int32[C][R+E]: exclusive prefix over chunks
+    size_t chunk_counts;   // int32[R+E][C padded to a multiple of 4]: per-chunk totals, transposed
     size_t pos;            // uint32[Tmax*K]: chunk-relative positions, rank slot | expert position << 16
     size_t total_bytes;
 };
@@ -42,17 +41,15 @@ struct LayoutParams {
     const int64_t* topk_idx;
     const uint8_t* route_mask;       // [T, R] bool: when set, lane r of token t is "rank r, if the mask says so" (K = E = R)
     int T, K, E, R, E_l;
-    int light;            // 1: only count (transposed chunk counts); the move kernel finishes the job
-    int chunks_padded;    // row length of the transposed chunk counts (light mode)
-    int slab_rows;        // chunk rows staged in LDS per pass of the final scan (set by the launcher)
+    int light;            // 1: only count; the move kernel of the same call sums the chunk totals and publishes
+    int chunks_padded;    // row length of the transposed chunk counts (set by the launcher)
     int vec_idx;          // topk_idx is 16-byte aligned (set by the launcher)
     uint8_t* is_token_in_rank;       // optional
     int64_t* copied_topk_idx;        // optional
     PublishParams pub;
     int32_t* status;
     uint32_t* done_counter;
-    int32_t* chunk_counts;
-    int32_t* chunk_base;
+    int32_t* chunk_counts;           // [R + E][chunks_padded]
     uint32_t* pos;                   // optional (layout-only calls skip the per-lane positions)
 };
 
@@ -67,7 +64,6 @@ struct MoveParams {
     const uint8_t* route_mask;       // see LayoutParams
     const float* topk_weights;
     const uint32_t* pos;
-    const int32_t* chunk_base;
     const int32_t* expert_start;
     const int32_t* cached_slot;
     int32_t* dst_buffer_slot_idx;
@@ -86,8 +82,9 @@ struct MoveParams {
     int row_bytes;       // input row bytes
     int tiles;           // column tiles per token
     int xcd_remap;       // give each XCD a contiguous token range
-    // light mode (compact layout, layout and move in one call): bases come from the transposed chunk counts
-    int light;
+    // Row bases come from the transposed chunk counts of the layout pass.
+    int flat;            // 1: R * chunks_padded <= 1024, a wavefront prefix-sums the whole rank part at once
+    int publish;         // 1: layout and move in one call (compact layout): workgroup 0 sums and publishes
     int chunks_padded;   // row length of chunk_counts_t
     int flat_per;        // rank-part entries each lane scans (4, 8 or 16)
     const int32_t* chunk_counts_t;   // [R + E][chunks_padded]

@@ -11,8 +11,8 @@
 //   count  = popcount(bitmap)                      and
 //   position of token t among chunk tokens routed to the same bucket = popcount(bitmap & lanes below t)
 // with no ordering-dependent atomics: placement is a pure function of the input.  Chunk totals go
-// to global memory; the last workgroup to finish turns them into exclusive chunk bases and into the
-// public prefix sums.
+// to global memory (transposed, so that a consumer prefix-sums along a row); the last workgroup to finish sums
+// them and publishes the public prefix sums.
 #include "common.cuh"
 #include "kernels.h"
 #include "publish.cuh"
@@ -28,7 +28,6 @@ constexpr int kWaves = kThreads / kWaveSize;
 template <int KMAX>
 __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) {
     extern __shared__ uint64_t bitmap[];   // [(R + E)][kWaves]
-    __shared__ int scan_tmp[kWaves];
     __shared__ int is_last;
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -134,22 +133,19 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     }
     if (flags != 0) atomicOr(p.status, flags);
 
+    // Chunk totals go out transposed, [bucket][chunk], so that consumers prefix-sum along rows; the padding
+    // columns up to a multiple of four are cleared by the first workgroup.
     for (int j = tid; j < n; j += kThreads) {
         int c = 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) c += __popcll(bitmap[j * kWaves + w]);
-        if (p.light) p.chunk_counts[int64_t(j) * p.chunks_padded + chunk] = c;   // [bucket][chunk]
-        else p.chunk_counts[int64_t(chunk) * n + j] = c;                         // [chunk][bucket]
+        p.chunk_counts[int64_t(j) * p.chunks_padded + chunk] = c;
     }
-    if (p.light) {
-        // The consumer (the move kernel) prefix-sums the transposed counts itself; only the padding
-        // columns still have to be cleared.
-        const int pad = p.chunks_padded - int(gridDim.x);
-        if (chunk == 0)
-            for (int i = tid; i < n * pad; i += kThreads)
-                p.chunk_counts[int64_t(i / pad) * p.chunks_padded + gridDim.x + i % pad] = 0;
-        return;
-    }
+    const int pad = p.chunks_padded - int(gridDim.x);
+    if (chunk == 0)
+        for (int i = tid; i < n * pad; i += kThreads)
+            p.chunk_counts[int64_t(i / pad) * p.chunks_padded + gridDim.x + i % pad] = 0;
+    if (p.light) return;      // the move kernel of the same call sums and publishes
 
     // Hand the chunk totals to whichever workgroup finishes last: release our stores, take a ticket.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
@@ -162,62 +158,8 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     if (!is_last) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
-    // ---- last workgroup: chunk bases and public prefix sums ----
-    // LDS is re-carved as int arrays: a staging slab of chunk rows, then totals / aligned / scanned.
-    int* stage = reinterpret_cast<int*>(bitmap);           // [slab_rows][n]
-    int* totals = stage + size_t(p.slab_rows) * n;         // [n]
-    int* aligned = totals + n;                             // [E] then scanned in place
-    const int num_chunks = gridDim.x;
-    for (int j = tid; j < n; j += kThreads) totals[j] = 0;
-    for (int c0 = 0; c0 < num_chunks; c0 += p.slab_rows) {
-        const int rows = min(p.slab_rows, num_chunks - c0);
-        const int32_t* src = p.chunk_counts + int64_t(c0) * n;
-        // 16-byte coalesced loads, all of a thread's loads in flight before its first LDS write (a plain
-        // copy loop would wait for each load in turn: one memory round trip per iteration).
-        const int total = rows * n;
-        const int total4 = (int64_t(c0) * n) % 4 == 0 ? total / 4 : 0;   // 16-byte path needs an aligned slab
-        const vec16* src4 = reinterpret_cast<const vec16*>(src);
-        vec16* stage4 = reinterpret_cast<vec16*>(stage);
-        for (int i0 = tid; i0 < total4; i0 += kThreads * 12) {
-            vec16 v[12];
-#pragma unroll
-            for (int u = 0; u < 12; ++u) {
-                const int i = i0 + u * kThreads;
-                v[u] = i < total4 ? src4[i] : vec16{0, 0, 0, 0};
-            }
-#pragma unroll
-            for (int u = 0; u < 12; ++u) {
-                const int i = i0 + u * kThreads;
-                if (i < total4) stage4[i] = v[u];
-            }
-        }
-        for (int i = total4 * 4 + tid; i < total; i += kThreads) stage[i] = src[i];
-        __syncthreads();
-        // Exclusive scan down each column, one column per thread, LDS reads batched by 8.
-        for (int j = tid; j < n; j += kThreads) {
-            int running = totals[j];
-            for (int r0 = 0; r0 < rows; r0 += 8) {
-                int v[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = (r0 + u < rows) ? stage[(r0 + u) * n + j] : 0;
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    if (r0 + u < rows) stage[(r0 + u) * n + j] = running;
-                    running += v[u];
-                }
-            }
-            totals[j] = running;
-        }
-        __syncthreads();
-        int32_t* dstb = p.chunk_base + int64_t(c0) * n;
-        vec16* dstb4 = reinterpret_cast<vec16*>(dstb);
-        for (int i = tid; i < total4; i += kThreads) dstb4[i] = stage4[i];
-        for (int i = total4 * 4 + tid; i < total; i += kThreads) dstb[i] = stage[i];
-        __syncthreads();
-    }
-
-    __syncthreads();
-    publish_counts<kThreads>(p.pub, totals, aligned, scan_tmp);
+    // ---- last workgroup: per-bucket totals and the public prefix sums (LDS is re-carved as int arrays) ----
+    publish_from_transposed_counts<kThreads>(p.pub, p.chunk_counts, p.chunks_padded, reinterpret_cast<int*>(bitmap));
     if (tid == 0) *p.done_counter = 0u;                    // ready for the next launch
 }
 
@@ -226,17 +168,13 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
 hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream) {
     const int num_chunks = p.T > 0 ? (p.T + kThreads - 1) / kThreads : 1;
     const int n = p.R + p.E;
-    // LDS holds the bitmap words [n][kWaves] first; the last workgroup re-carves it as a staging slab of
-    // chunk rows plus three int arrays of at most n entries.
+    // LDS holds the bitmap words [n][kWaves] first; the last workgroup re-carves it for the publishing step.
     const size_t bitmap_bytes = size_t(n) * kWaves * sizeof(uint64_t);
-    const size_t budget = 60 * 1024;
-    int slab_rows = int((budget - 3 * size_t(n) * 4) / (size_t(n) * 4));
-    slab_rows = slab_rows < 1 ? 1 : (slab_rows > num_chunks ? num_chunks : slab_rows);
-    const size_t scan_bytes = (size_t(slab_rows) + 3) * n * 4;
-    const size_t lds = bitmap_bytes > scan_bytes ? bitmap_bytes : scan_bytes;
+    const size_t publish_bytes = publish_lds_bytes(p.R, p.E, kThreads);
+    const size_t lds = bitmap_bytes > publish_bytes ? bitmap_bytes : publish_bytes;
     LayoutParams q = p;
     q.vec_idx = (reinterpret_cast<uintptr_t>(p.topk_idx) % 16 == 0) ? 1 : 0;
-    q.slab_rows = slab_rows;
+    q.chunks_padded = (num_chunks + 3) / 4 * 4;
     dim3 grid(num_chunks), block(kThreads);
     if (p.K <= 8) {
         hipLaunchKernelGGL(layout_kernel<8>, grid, block, lds, stream, q);

@@ -68,4 +68,55 @@ __device__ void publish_counts(const PublishParams& q, int* totals, int* scratch
     if (q.host_counts != nullptr) __threadfence_system();
 }
 
+// Sums the transposed chunk counts [R + E][chunks_padded] (padding columns are zero) into per-bucket totals and
+// publishes them.  lds: int[R + E] totals, int[2 * E] scratch, one int per wavefront.  Must be called by every
+// thread of the workgroup.
+template <int kThreads>
+__device__ void publish_from_transposed_counts(const PublishParams& q, const int32_t* counts_t, int chunks_padded,
+                                               int* lds) {
+    const int n = q.R + q.E;
+    int* totals = lds;
+    int* scratch = totals + n;
+    int* scan_tmp = scratch + 2 * q.E;
+    for (int j = threadIdx.x; j < n; j += kThreads) {
+        const int32_t* row = counts_t + int64_t(j) * chunks_padded;
+        int sum = 0;
+        for (int c0 = 0; c0 < chunks_padded; c0 += 32) {
+            vec16 v[8];                                   // all loads of a pass in flight together
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = load16(row + min(c0 + 4 * u, chunks_padded - 4));
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + 4 * u < chunks_padded) sum += int(v[u].x) + int(v[u].y) + int(v[u].z) + int(v[u].w);
+        }
+        totals[j] = sum;
+    }
+    __syncthreads();
+    publish_counts<kThreads>(q, totals, scratch, scan_tmp);
+}
+
+// Bytes of LDS publish_from_transposed_counts needs.
+inline size_t publish_lds_bytes(int R, int E, int threads) {
+    return size_t(R + 3 * E + threads / kWaveSize) * sizeof(int);
+}
+
+// Rows that chunks [0, chunk) put into `bucket`: a masked sum over the bucket's row of the transposed counts.
+// `chunk` must be uniform over the wavefront.
+__device__ __forceinline__ int row_prefix(const int32_t* counts_t, int chunks_padded, int bucket, int chunk) {
+    const int32_t* row = counts_t + int64_t(bucket) * chunks_padded;
+    int sum = 0;
+    for (int c0 = 0; c0 < chunk; c0 += 32) {
+        vec16 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = load16(row + min(c0 + 4 * u, chunks_padded - 4));
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int b = c0 + 4 * u;
+            sum += (b < chunk ? int(v[u].x) : 0) + (b + 1 < chunk ? int(v[u].y) : 0) +
+                   (b + 2 < chunk ? int(v[u].z) : 0) + (b + 3 < chunk ? int(v[u].w) : 0);
+        }
+    }
+    return sum;
+}
+
 }  // namespace deep_ep_hip

@@ -48,6 +48,10 @@ CASES = {
     "ragged_chunks": lambda: rc.small("ragged", 1000, 384, 32, 4, 5, seed=6, masked_ratio=0.1),
     "r1_world": lambda: rc.small("r1", 513, 1024, 16, 1, 3, seed=7, masked_ratio=0.05),
     "k9": lambda: rc.small("k9", 200, 2048, 64, 8, 9, seed=8, masked_ratio=0.05),
+    # 64 ranks x 20 chunks: too many (rank, chunk) pairs for one wavefront-wide prefix pass
+    "many_ranks": lambda: rc.small("many_ranks", 5000, 256, 128, 64, 8, seed=9, masked_ratio=0.05),
+    # 36 chunks: a row of chunk totals is summed in two passes
+    "many_chunks": lambda: rc.small("many_chunks", 9000, 128, 32, 8, 4, seed=10, masked_ratio=0.05),
 }
 
 

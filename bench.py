@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0
 # dispatch, each scaled by what the same counter reads for a plain copy kernel of known size: x2.000 for
 # FETCH_SIZE, x1.000 for WRITE_SIZE on this machine).  Keyed by (workload, layout, payload, kernel).
 MEASURED_TRAFFIC_BYTES = {
-    ("C3", "compact", "fp8", "dispatch"): int((58872.3 * 2.0 + 320348.6 * 1.0) * 1024),
-    ("C3", "compact", "fp8", "combine"): int((308818.4 * 2.0 + 114944.0 * 1.0) * 1024),
+    ("C3", "compact", "fp8", "dispatch"): int((60115.8 * 2.0 + 320764.5 * 1.0) * 1024),
+    ("C3", "compact", "fp8", "combine"): int((308813.4 * 2.0 + 114944.0 * 1.0) * 1024),
 }
 
 

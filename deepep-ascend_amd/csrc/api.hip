@@ -319,7 +319,10 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
     REQUIRE(!(a->cached && do_layout), "a cached dispatch has no layout phase");
     REQUIRE(a->rank_idx >= 0 && a->rank_idx < R, "rank_idx %d outside [0, %d)", a->rank_idx, R);
     REQUIRE(a->expert_alignment >= 1, "expert_alignment must be >= 1");
-    REQUIRE(a->num_channels >= 0, "num_channels must be >= 0");
+    REQUIRE(a->num_channels >= 0 && a->num_channels <= 8192, "num_channels must be in [0, 8192]");
+    REQUIRE(a->num_channels >= 1 || (a->rank_prefix_matrix == nullptr && a->channel_prefix_matrix == nullptr &&
+                                     a->recv_channel_prefix_matrix == nullptr),
+            "num_channels must be >= 1 when the prefix matrices are requested");
     REQUIRE(a->cached || T == 0 || with_topk || a->is_token_in_rank != nullptr, "is_token_in_rank is NULL");
     REQUIRE(a->workspace != nullptr, "workspace is NULL");
     REQUIRE(a->cached || a->psum_num_recv_tokens_per_rank != nullptr, "psum_num_recv_tokens_per_rank is NULL");
@@ -392,7 +395,6 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
             q.rank_prefix_matrix = a->rank_prefix_matrix;
             q.channel_prefix_matrix = a->channel_prefix_matrix;
             q.recv_channel_prefix_matrix = a->recv_channel_prefix_matrix;
-            REQUIRE(q.C >= 1 && q.C <= 8192, "num_channels must be in [1, 8192] when the channel matrices are requested");
             err = launch_intranode_prefix(q, stream);
             if (err != hipSuccess) return hip_fail(err, "intranode prefix launch");
         }

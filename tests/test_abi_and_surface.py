@@ -122,6 +122,54 @@ def test_other_entry_points_validate():
     assert _abi.lib.deep_ep_hip_launch_cast_fp8(None, None) == -1
 
 
+def _intranode_args(**kw):
+    a = _abi.IntranodeDispatchArgs()
+    a.phases = _abi.PHASE_LAYOUT
+    a.num_tokens, a.hidden, a.num_ranks, a.num_channels, a.expert_alignment = 16, 256, 2, 4, 1
+    a.is_token_in_rank = a.workspace = a.psum_num_recv_tokens_per_rank = 0x1000   # never dereferenced
+    a.workspace_bytes = 1 << 30
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    (dict(num_ranks=65), "num_ranks"), (dict(num_ranks=0), "num_ranks"),
+    (dict(topk_idx=0x1000, num_topk=2, num_experts=8), "go together"),
+    (dict(cached=1, topk_idx=0x1000, topk_weights=0x1000, num_topk=2, num_experts=8), "cached"),
+    (dict(cached=1), "layout phase"), (dict(rank_idx=2), "rank_idx"), (dict(phases=0), "phases"),
+    (dict(expert_alignment=0), "expert_alignment"), (dict(is_token_in_rank=0), "is_token_in_rank"),
+    (dict(workspace=0), "workspace"), (dict(payload=9), "payload"),
+    (dict(topk_idx=0x1000, topk_weights=0x1000, num_topk=2, num_experts=9), "divisible"),
+    (dict(num_ranks=40, num_tokens=4), "up to 32 ranks"),
+    (dict(phases=_abi.PHASE_MOVE, hidden=100, payload=_abi.PAYLOAD_FP8), "16 bytes"),
+    (dict(phases=_abi.PHASE_MOVE, x=0x1000, recv_x=0x1000, recv_capacity=8), "send_head"),
+    (dict(rank_prefix_matrix=0x1000, num_channels=0), "num_channels"),
+])
+def test_intranode_dispatch_rejects_bad_arguments_before_launch(kw, fragment):
+    rc = _abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(_intranode_args(**kw)), None)
+    assert rc == -1, kw
+    assert fragment in _abi.last_error(), _abi.last_error()
+
+
+def test_intranode_combine_and_low_latency_validate():
+    c = _abi.IntranodeCombineArgs()
+    c.num_tokens, c.hidden, c.num_ranks, c.num_topk = 4, 100, 2, 0
+    assert _abi.lib.deep_ep_hip_launch_intranode_combine(ctypes.byref(c), None) == -1 and "16 bytes" in _abi.last_error()
+    c.hidden, c.num_ranks = 128, 65
+    assert _abi.lib.deep_ep_hip_launch_intranode_combine(ctypes.byref(c), None) == -1 and "num_ranks" in _abi.last_error()
+    c.num_ranks, c.num_topk = 2, 33
+    assert _abi.lib.deep_ep_hip_launch_intranode_combine(ctypes.byref(c), None) == -1 and "num_topk" in _abi.last_error()
+    l = _abi.LLDispatchArgs()
+    l.num_src_ranks, l.src_token_stride, l.num_topk, l.num_experts, l.num_local_experts = 1, 8, 2, 8, 4
+    l.expert_begin, l.num_ranks, l.num_max_dispatch_tokens_per_rank, l.hidden = 4, 2, 8, 256
+    l.x = l.topk_idx = l.packed_recv_x = l.packed_recv_count = l.packed_recv_src_info = l.packed_recv_layout_range = 0x1000
+    l.use_fp8, l.round_scale = 0, 1
+    assert _abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(l), None) == -1 and "round_scale" in _abi.last_error()
+    l.use_fp8, l.use_ue8m0, l.packed_recv_x_scales = 1, 1, 0x1000          # 256 is not a multiple of 512
+    assert _abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(l), None) == -1 and "use_ue8m0" in _abi.last_error()
+
+
 def test_missing_library_fails_loudly():
     env = dict(os.environ, DEEP_EP_HIP_LIBRARY="/nonexistent/libdeep_ep_hip.so",
                PYTHONPATH=os.path.join(ROOT, "deepep-ascend_amd"))

@@ -23,7 +23,10 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / kWaveSize;
-constexpr int kBatch = 4;   // source rows whose loads are issued together
+#ifndef DEEP_EP_HIP_COMBINE_BATCH
+#define DEEP_EP_HIP_COMBINE_BATCH 4
+#endif
+constexpr int kBatch = DEEP_EP_HIP_COMBINE_BATCH;   // source rows whose loads are issued together
 
 template <int kVecs>
 __device__ __forceinline__ void add_row(float (&acc)[kVecs][8], const vec16 (&v)[kVecs]) {

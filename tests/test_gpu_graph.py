@@ -54,3 +54,35 @@ def test_graph_replays_match_eager(fp8):
         assert torch.equal(g_out.view(torch.int16), e_out.view(torch.int16))
         assert torch.equal(g_w, e_w)
     buf.check_device_status()
+
+
+def test_low_latency_graph_replays_match_eager():
+    """The decode loop is launch bound (two ~10 us kernels per step): captured once, replayed per step."""
+    import deep_ep
+    R, T, H, E, K, M = 8, 128, 2048, 64, 4, 128
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(3, R), low_latency_mode=True)
+    sets = [rc.c5_sources(seed=s, R=R, T=T, H=H, E=E, K=K) for s in (30, 31, 32)]
+    x_s, idx_s, w_s = (t.cuda() for t in sets[0])
+
+    def step(x, idx, w):
+        recv, count, handle, _, _ = buf.low_latency_dispatch(x, idx, M, E, use_fp8=True)
+        q, sf = recv
+        y = (q.float().view(*q.shape[:2], -1, 128) * sf.unsqueeze(3)).view(q.shape).to(torch.bfloat16)
+        out, _, _ = buf.low_latency_combine(y, idx, w, handle)
+        return count, handle[1], out
+
+    step(x_s, idx_s, w_s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_count, g_range, g_out = step(x_s, idx_s, w_s)
+    for x, idx, w in sets + sets[:1]:
+        x, idx, w = x.cuda(), idx.cuda(), w.cuda()
+        e_count, e_range, e_out = step(x, idx, w)
+        torch.cuda.synchronize()
+        x_s.copy_(x); idx_s.copy_(idx); w_s.copy_(w)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_count, e_count)
+        assert torch.equal(g_range, e_range)
+        assert torch.equal(g_out.view(torch.int16), e_out.view(torch.int16))

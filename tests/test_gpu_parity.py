@@ -50,6 +50,9 @@ CASES = {
     "k9": lambda: rc.small("k9", 200, 2048, 64, 8, 9, seed=8, masked_ratio=0.05),
     # 64 ranks x 20 chunks: too many (rank, chunk) pairs for one wavefront-wide prefix pass
     "many_ranks": lambda: rc.small("many_ranks", 5000, 256, 128, 64, 8, seed=9, masked_ratio=0.05),
+    "k20": lambda: rc.small("k20", 150, 256, 64, 4, 20, seed=11, masked_ratio=0.2),
+    # the limits of the interface: 1024 experts on 512 ranks
+    "max_buckets": lambda: rc.small("max_buckets", 600, 128, 1024, 512, 8, seed=12, masked_ratio=0.05),
     # 36 chunks: a row of chunk totals is summed in two passes
     "many_chunks": lambda: rc.small("many_chunks", 9000, 128, 32, 8, 4, seed=10, masked_ratio=0.05),
 }

@@ -60,6 +60,8 @@ def main():
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--routing", default="case", choices=["case", "sequential"],
                     help="sequential: every token goes to ranks 0..4 (dest rows of consecutive tokens are adjacent)")
+    ap.add_argument("--stream-yardsticks", action="store_true",
+                    help="also time plain torch kernels with the same read/write mixes (context for the roofline fractions)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain 1 GiB read + 1 GiB write elementwise kernel (scale for rocprof byte counters)")
     ap.add_argument("--l2-flush", action="store_true", help="zero a 256 MB buffer between per-kernel timings")
@@ -251,9 +253,45 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
+    if args.stream_yardsticks:
+        result["stream_yardsticks_gbs"] = stream_yardsticks(torch, dev)
+
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens, fp8, expanded)
     print(json.dumps(result))
+
+
+def stream_yardsticks(torch, dev, iters=10):
+    """What plain library kernels reach on this GPU for the traffic mixes of the routing kernels (GB/s of HBM
+    bytes moved): a fill (write only), an elementwise kernel (1 read : 1 write), a 1 : 3 broadcast (the dispatch
+    mix: every source row written to several destinations) and a 3 : 1 elementwise kernel (towards the combine mix)."""
+    n = 256 * 1024 * 1024                                  # fp32 elements: 1 GiB per tensor, beyond the 256 MB last-level cache
+    a = torch.ones(n, dtype=torch.float32, device=dev)
+    a2 = torch.ones(n, dtype=torch.float32, device=dev)
+    a3 = torch.ones(n, dtype=torch.float32, device=dev)
+    b = torch.empty(n, dtype=torch.float32, device=dev)
+    b3 = torch.empty((3, n), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream()
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(iters):
+            fn()
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / iters
+
+    nbytes = n * 4
+    out = {
+        "write_only_fill": round(nbytes / timed(lambda: b.fill_(1.0)) * 1e-9, 1),
+        "elementwise_1r_1w": round(2 * nbytes / timed(lambda: torch.mul(a, 1.0, out=b)) * 1e-9, 1),
+        "broadcast_1r_3w": round(4 * nbytes / timed(lambda: torch.mul(a.unsqueeze(0).expand(3, n), 1.0, out=b3)) * 1e-9, 1),
+        "elementwise_3r_1w": round(4 * nbytes / timed(lambda: torch.addcmul(a, a2, a3, out=b)) * 1e-9, 1),
+    }
+    return out
 
 
 def bench_low_latency(args, torch, rc, _abi, dev):

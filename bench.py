@@ -64,6 +64,8 @@ def main():
                     help="also time plain torch kernels with the same read/write mixes (context for the roofline fractions)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain 1 GiB read + 1 GiB write elementwise kernel (scale for rocprof byte counters)")
+    ap.add_argument("--fresh-input", action="store_true",
+                    help="per-kernel timings: rewrite x with a copy kernel right before every (untimed) call, as a producer would")
     ap.add_argument("--l2-flush", action="store_true", help="zero a 256 MB buffer between per-kernel timings")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -165,13 +167,17 @@ def main():
         combine()
 
     flush_buf = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev) if args.l2_flush else None
+    x_master = x.clone() if args.fresh_input else None
 
     def timed(fn, iters, flush=False):
         """Average duration in us of fn over iters launches, by HIP events on the launch stream."""
-        if flush:
+        if flush or args.fresh_input:
             total = 0.0
             for _ in range(iters):
-                flush_buf.zero_()
+                if flush:
+                    flush_buf.zero_()
+                if args.fresh_input:
+                    x.copy_(x_master)          # a producer kernel has just written the input (untimed)
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream); fn(); e1.record(stream)
                 e1.synchronize()
@@ -225,7 +231,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{case.name}: T={T} H={H} E={E} R={R} K={K} "
                                f"{'expanded' if expanded else 'compact'} layout, N_r={N_r}, N_e={N_e}",
-                   "l2_flush": bool(args.l2_flush)},
+                   "l2_flush": bool(args.l2_flush), "fresh_input": bool(args.fresh_input)},
         "us_per_call": {"dispatch": round(dispatch_us, 2), "dispatch_layout": round(layout_us, 2),
                         "dispatch_move": round(move_us, 2), "combine": round(combine_us, 2)},
         "achieved_gbs": {"dispatch": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us), 1),

@@ -156,8 +156,8 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
         if (r.d >= 0 && dj == r.d && rj >= 0) r.my_row = rj;
     }
     int expert_rows_before = 0;
-    if (p.do_expand && !p.cached)    // rows that earlier chunks put into this lane's expert
-        expert_rows_before = row_prefix(p.chunk_counts_t, p.chunks_padded, p.R + (r.e >= 0 ? r.e : 0), chunk);
+    if (p.do_expand && !p.cached && r.e >= 0)    // rows that earlier chunks put into this lane's expert
+        expert_rows_before = row_prefix(p.chunk_counts_t, p.chunks_padded, p.R + r.e, chunk);
     if (p.do_expand && r.e >= 0) {
         if (p.cached) {
             if (r.my_row >= 0 && r.my_row < p.recv_capacity)
@@ -326,8 +326,13 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
         in[q][0] = vec16{0, 0, 0, 0};
         in[q][1] = vec16{0, 0, 0, 0};
         if (elem < p.H) {
-            in[q][0] = load16_stream(src + int64_t(elem) * 2);
-            in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+            if (p.plain_loads) {
+                in[q][0] = load16(src + int64_t(elem) * 2);
+                in[q][1] = load16(src + int64_t(elem) * 2 + 16);
+            } else {
+                in[q][0] = load16_stream(src + int64_t(elem) * 2);
+                in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+            }
         }
     }
 
@@ -490,6 +495,8 @@ hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
     {
         const char* v = getenv("DEEP_EP_HIP_XCD_REMAP");
         p.xcd_remap = v != nullptr ? atoi(v) : 0;
+        const char* pl = getenv("DEEP_EP_HIP_PLAIN_LOADS");
+        p.plain_loads = pl != nullptr ? atoi(pl) : 0;
     }
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
         // Column tile = kPairs * 1024 channels per wavefront.  Two pairs (2048 channels, 8 waves per SIMD)

@@ -82,6 +82,7 @@ struct MoveParams {
     int row_bytes;       // input row bytes
     int tiles;           // column tiles per token
     int xcd_remap;       // give each XCD a contiguous token range
+    int plain_loads;     // payload loads without the non-temporal hint
     // Row bases come from the transposed chunk counts of the layout pass.
     int flat;            // 1: R * chunks_padded <= 1024, a wavefront prefix-sums the whole rank part at once
     int publish;         // 1: layout and move in one call (compact layout): workgroup 0 sums and publishes

@@ -155,3 +155,23 @@ def test_argument_errors():
     with pytest.raises(RuntimeError):
         buf.dispatch(x, num_tokens_per_rank=per_rank, is_token_in_rank=mask, num_tokens_per_expert=per_expert,
                      config=deep_ep.Config(7, 6, 256))                      # odd num_sms
+
+
+def test_empty_inputs():
+    """No tokens at all, and tokens that go nowhere (every top-k slot masked)."""
+    import deep_ep
+    R, E, K, H = 4, 16, 3, 256
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(1, R))
+    for T, fill in ((0, 0), (5, -1)):
+        x = torch.randn((T, H), device="cuda").to(torch.bfloat16)
+        idx = torch.full((T, K), fill, dtype=torch.int64, device="cuda")
+        w = torch.rand((T, K), device="cuda")
+        per_rank, _, per_expert, mask, _ = buf.get_dispatch_layout(idx, E)
+        assert int(per_rank.sum()) == 0 and int(per_expert.sum()) == 0 and mask.shape == (T, R) and not bool(mask.any())
+        recv_x, recv_idx, recv_w, lst, handle, _ = buf.dispatch(x, num_tokens_per_rank=per_rank, is_token_in_rank=mask,
+                                                               num_tokens_per_expert=per_expert, topk_idx=idx, topk_weights=w)
+        assert recv_x.shape == (0, H) and recv_idx.shape == (0, K) and recv_w.shape == (0, K) and lst == [0] * E
+        assert int(handle[0].abs().sum()) == 0 and handle[5].shape == (T, R) and bool((handle[5] == -1).all())
+        out, out_w, _ = buf.combine(recv_x, handle, topk_weights=recv_w)
+        assert out.shape == (T, H) and bool((out == 0).all()) and bool((out_w == 0).all())
+    buf.runtime._read_and_clear_status("intranode")

@@ -125,3 +125,21 @@ def test_ll_power_of_two_scales_hooks_and_zero_copy(R, T, H, E, K, M, use_ue8m0)
     assert_equal(out_a, out_b, "zero-copy combine")
     with pytest.raises(NotImplementedError):
         buf.low_latency_combine(y, idx.cuda(), w.cuda(), handle, use_logfmt=True)
+
+
+def test_ll_empty_and_unrouted_tokens():
+    import deep_ep
+    R, E, K, H, M = 2, 8, 2, 512, 16
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(0, R), low_latency_mode=True)
+    for T, fill in ((0, 0), (7, -1), (7, 5)):              # nothing; nothing selected; everything on the other rank
+        x = torch.randn((T, H), device="cuda").to(torch.bfloat16)
+        idx = torch.full((T, K), fill, dtype=torch.int64, device="cuda")
+        if fill == 5:
+            idx[:, 1] = 6
+        w = torch.rand((T, K), device="cuda")
+        recv, count, handle, _, _ = buf.low_latency_dispatch(x, idx, M, E, use_fp8=True)
+        assert recv[0].shape == (E // R, R * M, H) and int(count.sum()) == 0
+        assert int((handle[1] & 0xffffffff).sum()) == 0
+        y = torch.ones((E // R, R * M, H), dtype=torch.bfloat16, device="cuda")
+        out, _, _ = buf.low_latency_combine(y, idx, w, handle)
+        assert out.shape == (T, H) and bool((out == 0).all())

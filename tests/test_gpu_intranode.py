@@ -175,3 +175,42 @@ def test_empty_inputs():
         out, out_w, _ = buf.combine(recv_x, handle, topk_weights=recv_w)
         assert out.shape == (T, H) and bool((out == 0).all()) and bool((out_w == 0).all())
     buf.runtime._read_and_clear_status("intranode")
+
+
+def test_per_source_calls_compose_into_the_world():
+    """One call per logical source rank; the slices of every destination, stacked in source order, are what that
+    destination holds in a real R-rank run (rows, local ids, weights, source indices, rank_prefix_matrix)."""
+    import deep_ep
+    R, T, H, E, K = 4, 300, 256, 32, 5
+    g = torch.Generator().manual_seed(77)
+    xs, idxs, ws, masks = [], [], [], []
+    for r in range(R):
+        n = T - 17 * r
+        xs.append(torch.randn((n, H), generator=g).to(torch.bfloat16))
+        scores = torch.rand((n, E), generator=g)
+        idx = torch.topk(scores, K, dim=-1, sorted=False)[1].to(torch.int64)
+        idxs.append(idx.masked_fill(torch.rand(idx.shape, generator=g) < 0.15, -1))
+        ws.append(torch.rand((n, K), generator=g))
+        masks.append(oracle.layout(idxs[-1], E, R)[2])
+    world, _ = oracle.intranode_world_dispatch(xs, masks, idxs, ws, E, 1, num_channels=10)
+    parts = [[] for _ in range(R)]
+    prefix_sum = torch.zeros((R, R), dtype=torch.int32)
+    for r in range(R):
+        buf = deep_ep.Buffer(deep_ep.LogicalGroup(r, R))
+        idx_d = idxs[r].cuda()
+        per_rank, _, per_expert, mask_d, _ = buf.get_dispatch_layout(idx_d, E)
+        recv_x, recv_idx, recv_w, _, handle, _ = buf.dispatch(
+            xs[r].cuda(), num_tokens_per_rank=per_rank, is_token_in_rank=mask_d, num_tokens_per_expert=per_expert,
+            topk_idx=idx_d, topk_weights=ws[r].cuda())
+        counts = per_rank.cpu()
+        starts = counts.cumsum(0) - counts
+        for j in range(R):
+            lo, hi = int(starts[j]), int(starts[j] + counts[j])
+            parts[j].append((recv_x[lo:hi].cpu(), recv_idx[lo:hi].cpu(), recv_w[lo:hi].cpu(), handle[3][lo:hi].cpu()))
+        prefix_sum += handle[0].cpu()
+    for j in range(R):
+        assert_equal(torch.cat([p[0] for p in parts[j]]), world[j].recv_x, f"recv_x of rank {j}")
+        assert_equal(torch.cat([p[1] for p in parts[j]]), world[j].recv_topk_idx, f"recv_topk_idx of rank {j}")
+        assert_equal(torch.cat([p[2] for p in parts[j]]), world[j].recv_topk_weights, f"recv_topk_weights of rank {j}")
+        assert_equal(torch.cat([p[3] for p in parts[j]]), world[j].recv_src_idx, f"recv_src_idx of rank {j}")
+    assert_equal(prefix_sum, world[0].rank_prefix_matrix, "rank_prefix_matrix summed over the calls")

@@ -213,6 +213,28 @@ def main():
     dispatch_us = timed(lambda: dispatch(_abi.PHASE_LAYOUT | _abi.PHASE_MOVE), k, args.l2_flush)
     combine_us = timed(combine, k, args.l2_flush)
 
+    def distribution(fn, iters, flush):
+        """min / p50 / p95 / mean in us over single launches, each bracketed by its own pair of HIP events (the
+        events add a few us to every sample).  flush: a 256 MB buffer is zeroed before each launch."""
+        buf = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev) if flush else None
+        samples = []
+        for _ in range(iters):
+            if flush:
+                buf.zero_()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream); fn(); e1.record(stream)
+            e1.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e3)
+        samples.sort()
+        pick = lambda q: samples[min(len(samples) - 1, int(q * len(samples)))]
+        return {"min": round(samples[0], 2), "p50": round(pick(0.5), 2), "p95": round(pick(0.95), 2),
+                "mean": round(sum(samples) / len(samples), 2)}
+
+    full_dispatch = lambda: dispatch(_abi.PHASE_LAYOUT | _abi.PHASE_MOVE)
+    dist = {"dispatch": distribution(full_dispatch, k, False), "combine": distribution(combine, k, False),
+            "dispatch_after_cache_flush": distribution(full_dispatch, k, True),
+            "combine_after_cache_flush": distribution(combine, k, True)}
+
     def gbs(nbytes, us):
         return nbytes / us * 1e-3
 
@@ -232,6 +254,7 @@ def main():
         "config": {"workload": f"{case.name}: T={T} H={H} E={E} R={R} K={K} "
                                f"{'expanded' if expanded else 'compact'} layout, N_r={N_r}, N_e={N_e}",
                    "l2_flush": bool(args.l2_flush), "fresh_input": bool(args.fresh_input)},
+        "us_per_single_launch": dist,
         "us_per_call": {"dispatch": round(dispatch_us, 2), "dispatch_layout": round(layout_us, 2),
                         "dispatch_move": round(move_us, 2), "combine": round(combine_us, 2)},
         "achieved_gbs": {"dispatch": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us), 1),

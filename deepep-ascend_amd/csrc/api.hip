@@ -508,6 +508,8 @@ int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* a, void* 
     REQUIRE(a->num_max_dispatch_tokens_per_rank >= 1, "num_max_dispatch_tokens_per_rank must be positive");
     REQUIRE(int64_t(a->num_ranks) * a->num_max_dispatch_tokens_per_rank < (int64_t(1) << 31), "rows per expert overflow int32");
     REQUIRE(a->src_token_stride <= a->num_max_dispatch_tokens_per_rank, "src_token_stride exceeds num_max_dispatch_tokens_per_rank");
+    REQUIRE(a->lane_rows == nullptr || int64_t(a->num_local_experts) * a->num_ranks * a->num_max_dispatch_tokens_per_rank < (int64_t(1) << 31),
+            "lane_rows needs num_local_experts * rows per expert below 2^31");
     REQUIRE(a->hidden >= 16 && a->hidden % 16 == 0, "hidden must be a multiple of 16");
     REQUIRE(!a->use_fp8 || a->hidden % 128 == 0, "FP8 needs hidden %% 128 == 0");
     REQUIRE(!a->use_fp8 || a->packed_recv_x_scales != nullptr, "packed_recv_x_scales is NULL");

@@ -117,3 +117,31 @@ def test_bf16_round_trip(name, do_expand):
     assert torch.equal((out + 0.0).view(torch.int16), (acc.to(torch.bfloat16) + 0.0).view(torch.int16))
     assert torch.equal(out_w, torch.where(idx >= 0, w, torch.zeros_like(w)))
     buf.check_device_status()
+
+
+@pytest.mark.parametrize("name", ["C3", "C4"])
+def test_combine_against_fp32_reference_within_one_bf16_ulp(name):
+    """Random expert outputs at full size: the combined rows against an fp32 scatter-add done by the library
+    (different accumulation order), tolerance = 1 BF16 ulp of the fp32 result (the tolerance stated for the path) plus fp32 reordering slack."""
+    case = rc.c3() if name == "C3" else rc.c4()
+    buf = _buffer(case)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    recv_x, recv_idx, recv_w, handle, _ = buf.dispatch(x, idx, w, num_experts=case.E)
+    n = handle.num_recv_tokens
+    g = torch.Generator(device="cuda").manual_seed(5)
+    y = torch.randn((n, case.H), generator=g, device="cuda").to(torch.bfloat16)
+    bias = torch.randn((case.T, case.H), generator=g, device="cuda").to(torch.bfloat16)
+    out, _, _ = buf.combine(y, handle, bias=bias)
+    ref = bias.float()
+    ref.index_add_(0, handle.recv_src_metadata[:n, 0].long(), y.float())
+    ref_bf16 = ref.to(torch.bfloat16).float()
+    # 1 BF16 ulp of the result (8 significant bits: 2^(exponent - 8) with frexp's exponent), plus the slack a
+    # different fp32 summation order can cause where the terms cancel (2^-21 of the sum of magnitudes)
+    ulp = torch.ldexp(torch.ones_like(ref_bf16), torch.frexp(ref_bf16)[1] - 8)
+    magnitudes = bias.float().abs()
+    magnitudes.index_add_(0, handle.recv_src_metadata[:n, 0].long(), y.float().abs())
+    err = (out.float() - ref_bf16).abs()
+    bound = ulp + magnitudes * 2.0 ** -21
+    assert bool((err <= bound).all()), f"max error {float((err / bound).max()):.2f} of the bound"
+    # and the great majority of elements agree exactly
+    assert float((err == 0).float().mean()) > 0.98

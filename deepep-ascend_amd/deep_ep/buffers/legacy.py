@@ -57,6 +57,24 @@ class Buffer:
         return EventOverlap(_C.EventHandle())
 
     @staticmethod
+    def is_sm90_compiled() -> bool:
+        """The reference gates its FP8 paths on this (deep_ep/buffers/legacy.py:149-151); they are always built here."""
+        return True
+
+    def get_comm_stream(self) -> torch.cuda.Stream:
+        return self.runtime.get_comm_stream()
+
+    def clean_low_latency_buffer(self, num_max_dispatch_tokens_per_rank: int, hidden: int, num_experts: int) -> None:
+        """Nothing is staged between calls on one GPU, so there is nothing to clean
+        (deep_ep/buffers/legacy.py:538-551)."""
+
+    def internode_dispatch(self, *args, **kwargs):
+        raise NotImplementedError('the HIP backend has one scale-up domain: there are no RDMA ranks to dispatch to')
+
+    def internode_combine(self, *args, **kwargs):
+        raise NotImplementedError('the HIP backend has one scale-up domain: there are no RDMA ranks to combine from')
+
+    @staticmethod
     def get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
                                        num_experts: int) -> int:
         """Bytes the reference would reserve (csrc/legacy/config.hpp:131-188); nothing is staged here."""

@@ -229,6 +229,16 @@ def test_signatures_are_drop_in():
                                                             "use_fp8", "round_scale", "use_ue8m0", "async_finish", "return_recv_hook"]
     assert _params(deep_ep.Buffer.low_latency_combine) == ["x", "topk_idx", "topk_weights", "handle", "use_logfmt", "zero_copy",
                                                            "async_finish", "return_recv_hook", "out", "combine_wait_recv_cost_stats"]
+    # V1 pair: deep_ep/buffers/legacy.py:322-331 and :408-413
+    assert _params(deep_ep.Buffer.dispatch) == ["x", "handle", "num_tokens_per_rank", "num_tokens_per_rdma_rank",
+                                                "is_token_in_rank", "num_tokens_per_expert", "topk_idx", "topk_weights",
+                                                "expert_alignment", "num_worst_tokens", "config", "previous_event",
+                                                "async_finish", "allocate_on_comm_stream"]
+    assert _params(deep_ep.Buffer.combine) == ["x", "handle", "topk_weights", "bias", "config", "previous_event",
+                                               "async_finish", "allocate_on_comm_stream"]
+    assert len(_params(_C.ElasticBuffer.intranode_dispatch)) == 17           # the binding's 16 + cached_send_head
+    assert len(_params(_C.ElasticBuffer.intranode_combine)) == 12
+    assert deep_ep.Buffer.is_sm90_compiled() and deep_ep.Config(20, 6, 256).num_sms == 20
     # the runtime keeps the positional order of the compiled binding (29 dispatch / 18 combine arguments, then extensions)
     assert len(_params(_C.ElasticBuffer.dispatch)) == 30 and _params(_C.ElasticBuffer.dispatch)[-1] == "cast_to_fp8"
     assert len(_params(_C.ElasticBuffer.combine)) == 19 and _params(_C.ElasticBuffer.combine)[-1] == "dst_buffer_slot_idx"

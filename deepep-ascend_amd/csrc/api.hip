@@ -303,11 +303,13 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
 int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_args* a, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     REQUIRE(a != nullptr, "args is NULL");
-    const bool with_topk = a->topk_idx != nullptr;
+    // An empty batch has NULL tensors: the routing mode follows num_topk, not the pointers.
+    const bool with_topk = a->num_topk > 0 || a->topk_idx != nullptr;
     const int T = a->num_tokens, H = a->hidden, R = a->num_ranks;
     REQUIRE(R >= 1 && R <= 64, "num_ranks must be in [1, 64] (got %d)", R);
     REQUIRE(!a->cached || !with_topk, "a cached dispatch takes no topk_idx");
-    REQUIRE(with_topk == (a->topk_weights != nullptr), "topk_idx and topk_weights go together");
+    REQUIRE((a->topk_idx != nullptr) == (a->topk_weights != nullptr), "topk_idx and topk_weights go together");
+    REQUIRE(!with_topk || T == 0 || a->topk_idx != nullptr, "topk_idx is NULL");
     // Routing lanes: the top-k lanes, or one lane per rank.
     const int K = with_topk ? a->num_topk : R;
     const int E = with_topk ? a->num_experts : R;
@@ -387,8 +389,9 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         hipError_t err = launch_layout_kernel(p, stream);
         if (err != hipSuccess) return hip_fail(err, "intranode dispatch layout launch");
 
-        if (a->is_token_in_rank != nullptr && (a->rank_prefix_matrix != nullptr || a->channel_prefix_matrix != nullptr ||
-                                               a->recv_channel_prefix_matrix != nullptr)) {
+        if (a->rank_prefix_matrix != nullptr || a->channel_prefix_matrix != nullptr ||
+            a->recv_channel_prefix_matrix != nullptr) {
+            REQUIRE(a->is_token_in_rank != nullptr || T == 0, "the prefix matrices are computed from is_token_in_rank");
             IntranodePrefixParams q{};
             q.mask = a->is_token_in_rank;
             q.T = T; q.R = R; q.C = a->num_channels; q.rank_idx = a->rank_idx;

@@ -192,8 +192,8 @@ typedef struct {
     int32_t payload;                /* DEEP_EP_HIP_PAYLOAD_* */
     int32_t cached;                 /* send_head is an input; topk_idx / is_token_in_rank are not read */
     int32_t num_tokens, hidden;
-    int32_t num_topk;               /* 0 when topk_idx is NULL */
-    int32_t num_experts;            /* 0 when topk_idx is NULL */
+    int32_t num_topk;               /* 0 = route by is_token_in_rank alone (no top-k tensors) */
+    int32_t num_experts;            /* 0 with num_topk == 0 */
     int32_t num_ranks, rank_idx;
     int32_t num_channels;           /* columns of the channel matrices (reference: config.num_sms / 2) */
     int32_t expert_alignment;

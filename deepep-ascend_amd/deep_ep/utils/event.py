@@ -1,6 +1,7 @@
-"""`EventOverlap`: the stream-event wrapper dispatch / combine hand back
-(surface of the reference's deep_ep/utils/event.py:8-96)."""
-from typing import Any, Callable, Optional, Tuple
+"""`EventOverlap`: what dispatch / combine hand back for stream overlap.  Same public surface as the reference's
+deep_ep/utils/event.py:8-96 (`event`, `extra_tensors`, `current_stream_wait`, `register_hook_after_wait`, call and
+`with` forms); the state machine below is this package's own."""
+from typing import Any, Callable, Optional, Sequence
 
 import torch
 
@@ -8,44 +9,45 @@ from .._C import EventHandle
 
 
 class EventOverlap:
-    """Holds the event recorded after the routing kernels, plus an optional hook that must run on
-    the waiting stream right after the wait (used by the deterministic epilogue).
+    """An event recorded behind the routing kernels of one call.
 
-    Attributes:
-        event: the captured `EventHandle` (None when the call was synchronous with the compute stream).
-        extra_tensors: tensors kept alive until the event is released.
+    `event` is None for calls that already ordered themselves with the caller's stream.  `extra_tensors` keeps the
+    tensors of an asynchronous call alive until the object goes away.  One callback can be attached; it fires on the
+    first wait (the epilogue of a deterministic call uses it).
     """
 
     def __init__(self, event: Optional[EventHandle] = None,
-                 extra_tensors: Optional[Tuple[torch.Tensor, ...]] = None) -> None:
-        self.event = event
-        self.extra_tensors = extra_tensors
-        self._release_handle_by_call = False
-        self.hook_after_wait: Optional[Callable] = None
+                 extra_tensors: Optional[Sequence[torch.Tensor]] = None) -> None:
+        self.event, self.extra_tensors = event, extra_tensors
+        self.hook_after_wait: Optional[Callable[[], Any]] = None
+        self._drop_on_exit = False
 
+    # -- waiting ---------------------------------------------------------------------------------
     def current_stream_wait(self, release_handle: bool = False) -> None:
-        """Make `torch.cuda.current_stream()` wait for the event, then run the registered hook once."""
-        assert self.event is not None
+        """Order torch's current stream behind the event; then fire the callback, once."""
+        if self.event is None:
+            raise AssertionError("this EventOverlap holds no event")
         self.event.current_stream_wait()
-        hook, self.hook_after_wait = self.hook_after_wait, None
-        if hook is not None:
-            hook()
+        pending, self.hook_after_wait = self.hook_after_wait, None
+        if callable(pending):
+            pending()
         if release_handle:
             self.event = None
 
-    def register_hook_after_wait(self, hook_after_wait: Callable) -> None:
-        assert self.hook_after_wait is None, "A hook is already registered on this `EventOverlap`"
+    def register_hook_after_wait(self, hook_after_wait: Callable[[], Any]) -> None:
+        if self.hook_after_wait is not None:
+            raise AssertionError("A hook is already registered on this `EventOverlap`")
         self.hook_after_wait = hook_after_wait
 
+    # -- `with overlap:` / `with overlap(release_handle=True):` ----------------------------------
     def __call__(self, release_handle: bool = False) -> "EventOverlap":
-        """`with event_overlap(release_handle=True): ...` drops the event after the wait."""
-        self._release_handle_by_call = release_handle
+        self._drop_on_exit = bool(release_handle)
+        return self                      # no second wrapper: the event keeps a single owner
+
+    def __enter__(self) -> "EventOverlap":
         return self
 
-    def __enter__(self) -> Any:
-        return self
-
-    def __exit__(self, exc_type: Any, exc_val: Any, exc_tb: Any) -> None:
+    def __exit__(self, *exc_info: Any) -> None:
+        drop, self._drop_on_exit = self._drop_on_exit, False
         if self.event is not None:
-            self.current_stream_wait(release_handle=self._release_handle_by_call)
-        self._release_handle_by_call = False
+            self.current_stream_wait(release_handle=drop)

@@ -9,18 +9,19 @@ from .. import _abi
 
 
 def ceil_div(x: int, y: int) -> int:
-    return (x + y - 1) // y
+    return -(-x // y)
 
 
 def align(x: int, y: int) -> int:
-    return ceil_div(x, y) * y
+    return -(-x // y) * y
 
 
 def calc_diff(x: torch.Tensor, y: torch.Tensor) -> float:
-    """1 - cosine-like similarity of (x+1, y+1) in fp64 (math.py:5-9)."""
-    x, y = x.double() + 1, y.double() + 1
-    denominator = (x * x + y * y).sum()
-    return (1 - 2 * (x * y).sum() / denominator).item()
+    """The reference's distance between two tensors (math.py:5-9): 1 - 2<a, b> / (<a, a> + <b, b>) with a = x + 1,
+    b = y + 1 in fp64."""
+    a = x.to(torch.float64) + 1.0
+    b = y.to(torch.float64) + 1.0
+    return float(1.0 - 2.0 * torch.sum(a * b) / (torch.sum(a * a) + torch.sum(b * b)))
 
 
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -39,27 +40,27 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 def per_token_cast_back(x_fp8: torch.Tensor, x_scales: torch.Tensor) -> torch.Tensor:
-    """(e4m3fn [m, n], scales [m, ceil(n/128)] fp32 or packed UE8M0 int32) -> BF16 [m, n] (math.py:42-56)."""
-    if x_fp8.numel() == 0:
-        return x_fp8.to(torch.bfloat16)
+    """(e4m3fn [m, n], scales [m, ceil(n/128)] fp32, or UE8M0 exponent bytes packed four to an int32) -> BF16 [m, n]:
+    every group of 128 channels times its scale (math.py:42-56)."""
     m, n = x_fp8.shape
-    aligned_n = align(n, 128)
-    padded = torch.nn.functional.pad(x_fp8.to(torch.float32), (0, aligned_n - n))
-    if x_scales.dtype == torch.int:
-        x_scales = (x_scales.view(dtype=torch.uint8).to(torch.int) << 23).view(dtype=torch.float)
-    out = padded.view(m, -1, 128) * x_scales.reshape(m, -1, 1)
-    return out.view(m, aligned_n).to(torch.bfloat16)[:, :n].contiguous()
+    if m * n == 0:
+        return x_fp8.to(torch.bfloat16)
+    if x_scales.dtype == torch.int32:                      # exponent byte -> fp32 power of two
+        exponents = x_scales.contiguous().view(torch.uint8).to(torch.int32)
+        x_scales = (exponents << 23).view(torch.float32)
+    groups = ceil_div(n, 128)
+    values = torch.zeros((m, groups * 128), dtype=torch.float32, device=x_fp8.device)
+    values[:, :n] = x_fp8.to(torch.float32)
+    values = values.view(m, groups, 128) * x_scales.reshape(m, groups, 1).to(torch.float32)
+    return values.view(m, groups * 128)[:, :n].to(torch.bfloat16).contiguous()
 
 
 def hash_tensor(t: torch.Tensor) -> int:
-    return t.view(torch.int).sum().item()
+    """Order-independent checksum of the raw 32-bit words."""
+    return int(t.contiguous().view(torch.int32).sum())
 
 
 def count_bytes(*tensors) -> int:
-    total = 0
-    for t in tensors:
-        if isinstance(t, (tuple, list)):
-            total += count_bytes(*t)
-        elif t is not None:
-            total += t.numel() * t.element_size()
-    return total
+    """Bytes held by tensors, tuples / lists of tensors and Nones, recursively."""
+    return sum(count_bytes(*t) if isinstance(t, (tuple, list)) else t.numel() * t.element_size()
+               for t in tensors if t is not None)

@@ -1,6 +1,8 @@
-from typing import Any, Optional
+"""Tiny argument helpers."""
 
 
-def value_or(value: Optional[Any], default: Any) -> Any:
-    """`value` unless it is None."""
-    return default if value is None else value
+def value_or(value, default):
+    """`default` stands in for a missing (None) `value`."""
+    if value is None:
+        return default
+    return value

@@ -56,6 +56,8 @@ def main():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--expanded", action="store_true", help="expert-major (expanded) receive layout")
     ap.add_argument("--bf16", action="store_true", help="BF16 dispatch instead of the fused FP8 cast")
+    ap.add_argument("--launches", type=int, default=0, choices=[0, 1, 2],
+                    help="dispatch: 0 library's choice (single launch), 1 single launch even where it does not pay, 2 layout kernel + move kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--routing", default="case", choices=["case", "sequential"],
@@ -138,8 +140,11 @@ def main():
     d.recv_topk_weights = recv_w.data_ptr()
     d.recv_capacity, d.expanded_capacity = cap, (ecap if expanded else 0)
     d.workspace, d.workspace_bytes = workspace.data_ptr(), ws_bytes
+    d.tuning = _abi.Tuning.from_env()
+    d.tuning.dispatch_launches = args.launches
 
     c = _abi.CombineArgs()
+    c.tuning = _abi.Tuning.from_env()
     c.do_expand, c.allow_multiple_reduction = int(expanded), 1
     c.num_tokens, c.hidden, c.num_topk, c.num_experts, c.num_ranks = T, H, K, E, R
     c.rank_idx, c.num_max_tokens_per_rank = 0, M
@@ -253,7 +258,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{case.name}: T={T} H={H} E={E} R={R} K={K} "
                                f"{'expanded' if expanded else 'compact'} layout, N_r={N_r}, N_e={N_e}",
-                   "l2_flush": bool(args.l2_flush), "fresh_input": bool(args.fresh_input)},
+                   "l2_flush": bool(args.l2_flush), "fresh_input": bool(args.fresh_input),
+                   "dispatch_launches": args.launches},
         "us_per_single_launch": dist,
         "us_per_call": {"dispatch": round(dispatch_us, 2), "dispatch_layout": round(layout_us, 2),
                         "dispatch_move": round(move_us, 2), "combine": round(combine_us, 2)},

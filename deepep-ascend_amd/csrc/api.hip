@@ -7,7 +7,7 @@
 #include <cstring>
 
 #include "../../include/deep_ep_hip.h"
-#include "common.cuh"
+#include "device_utils.h"
 #include "kernels.h"
 
 namespace deep_ep_hip {
@@ -45,6 +45,55 @@ int check_routing_shape(int T, int K, int E, int R) {
     return DEEP_EP_HIP_OK;
 }
 
+// How a dispatch call is cut into launches.
+struct LaunchPlan {
+    int chunks, chunks_padded;
+    bool fused;       // one launch: counting workgroups at the front of the move kernel
+};
+
+// Past this many mover workgroups the per-workgroup cost of the single-launch protocol (a look at a gate, one
+// atomic, a workgroup barrier) outweighs the launch it saves: 28 672 workgroups of 8192 BF16 rows of 14 KB take
+// 180 us in one launch against 140 us in two; 8 192 workgroups of the same rows cast to FP8 take 92 us against 97 us.
+constexpr int64_t kMaxFusedMovers = 16384;
+
+LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_move, int payload, int H, int row_bytes,
+                         const deep_ep_hip_tuning& tuning) {
+    LaunchPlan q{};
+    q.chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
+    q.chunks_padded = (q.chunks + 3) / 4 * 4;
+    q.fused = do_layout && do_move && T > 0 && K <= 8 && (R + E) <= 512 && R * q.chunks_padded <= 1024 &&
+              tuning.dispatch_launches != 2;
+    if (q.fused && tuning.dispatch_launches != 1) {
+        MoveParams probe{};
+        probe.T = T; probe.H = H; probe.row_bytes = row_bytes; probe.payload = payload;
+        probe.cast_pairs = tuning.cast_pairs; probe.copy_vecs = tuning.copy_vecs;
+        q.fused = dispatch_move_workgroups(probe) <= kMaxFusedMovers;
+    }
+    return q;
+}
+
+LayoutTables carve_tables(uint8_t* ws, const WorkspaceLayout& w, int num_tokens, int num_experts) {
+    LayoutTables t{};
+    t.rank_counts = reinterpret_cast<int32_t*>(ws + w.rank_counts);
+    t.rank_bases = reinterpret_cast<int32_t*>(ws + w.rank_bases);
+    t.expert_counts = reinterpret_cast<int32_t*>(ws + w.expert_counts);
+    t.expert_bases = reinterpret_cast<int32_t*>(ws + w.expert_bases);
+    const int chunks = num_tokens > 0 ? (num_tokens + kLayoutChunk - 1) / kLayoutChunk : 1;
+    t.chunks_padded = (chunks + 3) / 4 * 4;
+    t.experts_padded = (num_experts + 31) / 32 * 32;
+    return t;
+}
+
+void fill_fused(MoveParams& m, const LayoutParams& lay, const LaunchPlan& plan, uint8_t* ws, const WorkspaceLayout& w) {
+    m.fused = 1;
+    m.count_blocks = plan.chunks;
+    m.lay = lay;
+    m.lay.count_only = 1;
+    m.lay.vec_idx = (reinterpret_cast<uintptr_t>(lay.topk_idx) % 16 == 0) ? 1 : 0;
+    m.chunk_done = reinterpret_cast<int32_t*>(ws + w.chunk_done);
+    m.gates = reinterpret_cast<uint32_t*>(ws + w.gates);
+}
+
 }  // namespace
 
 WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_experts, int num_ranks) {
@@ -58,8 +107,14 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.done_counter = off + 4;
     w.totals = off + 8;
     off = 256;
+    w.chunk_done = off;    off = align_up(off + size_t(kMaxCountBlocks) * 2 * 4, 256);
+    w.gates = off;         off = align_up(off + size_t(kDispatchGates) * kDispatchGateStride * 4, 256);
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
-    w.chunk_counts = off;  off = align_up(off + chunks_padded * n * 4, 256);
+    const size_t experts_padded = (size_t(num_experts) + 31) / 32 * 32;
+    w.rank_counts = off;   off = align_up(off + chunks_padded * num_ranks * 4, 256);
+    w.rank_bases = off;    off = align_up(off + chunks_padded * num_ranks * 4, 256);
+    w.expert_counts = off; off = align_up(off + chunks * experts_padded * 4, 256);
+    w.expert_bases = off;  off = align_up(off + chunks * experts_padded * 4, 256);
     w.pos = off;           off = align_up(off + lanes * 4, 256);
     w.total_bytes = off;
     return w;
@@ -81,6 +136,8 @@ size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_exp
 }
 
 size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
+
+size_t deep_ep_hip_workspace_control_bytes(void) { return make_workspace_layout(1, 1, 1, 1).expert_start; }
 
 int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
     REQUIRE(a != nullptr, "args is NULL");
@@ -105,7 +162,9 @@ int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
     p.pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
     p.status = reinterpret_cast<int32_t*>(ws + w.status);
     p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
-    p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
+    p.tab = carve_tables(ws, w, p.T, p.E);
+    p.tab.rank_bases = nullptr;       // a layout-only call publishes counts, not row bases
+    p.tab.expert_bases = nullptr;
     hipError_t err = launch_layout_kernel(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "layout launch");
     return DEEP_EP_HIP_OK;
@@ -155,6 +214,8 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         REQUIRE(a->dst_buffer_slot_idx != nullptr || T == 0, "dst_buffer_slot_idx is NULL");
         REQUIRE(a->recv_capacity >= 0 && a->expanded_capacity >= 0, "negative capacity");
         REQUIRE(a->recv_capacity < (int64_t(1) << 31) && a->expanded_capacity < (int64_t(1) << 31), "capacity overflows int32 rows");
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_BF16)
+            REQUIRE(a->num_sf_packs == 0 && a->sf == nullptr && a->recv_sf == nullptr, "a BF16 payload carries no scale factors");
         if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8) {
             REQUIRE(a->num_sf_packs >= 0, "num_sf_packs must be >= 0");
             REQUIRE(a->num_sf_packs == 0 || (a->sf != nullptr && a->recv_sf != nullptr) || T == 0, "sf / recv_sf is NULL");
@@ -178,31 +239,24 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
     pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
 
-    // The layout kernel leaves per-chunk totals [bucket][chunk]; the wavefronts of the move kernel prefix-sum
-    // what they need from them (the whole per-rank part at once while R * chunks <= 1024, single rows
-    // otherwise).  When layout and move run in one call on the compact layout ("light"), the layout kernel
-    // only counts and workgroup 0 of the move kernel publishes the handle tensors: no ticket, no fences and
-    // no serial tail on the critical path.
-    const int chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
-    const int chunks_padded = (chunks + 3) / 4 * 4;
-    const int flat = R * chunks_padded;
-    const int flat_per = flat <= 256 ? 4 : flat <= 512 ? 8 : 16;
-    const bool flat_ok = T > 0 && flat <= 1024 && !a->cached;
-    const bool light = do_layout && do_move && !a->do_expand && flat_ok && (R + E) <= 512 &&
-                       getenv("DEEP_EP_HIP_NO_LIGHT_LAYOUT") == nullptr;
+    // The layout pass leaves, per (token, lane), a position inside the token's 256-token chunk and, per (bucket,
+    // chunk), the first row of that chunk's share of the bucket; the move kernel adds the two.  Layout and move in
+    // one call: the counting workgroups ride at the front of the move kernel (one launch); shapes that does not
+    // cover run the layout kernel first.
+    const LaunchPlan plan = plan_launches(T, K, E, R, do_layout, do_move, a->payload, H, H * elem_in, a->tuning);
+    LayoutParams lay{};
+    lay.topk_idx = a->topk_idx;
+    lay.T = T; lay.K = K; lay.E = E; lay.R = R; lay.E_l = E / R;
+    lay.copied_topk_idx = a->copied_topk_idx;
+    lay.pub = pub;
+    lay.status = status;
+    lay.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
+    lay.tab = carve_tables(ws, w, T, E);
+    lay.expert_bases = a->do_expand ? 1 : 0;
+    lay.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
 
-    if (do_layout) {
-        LayoutParams p{};
-        p.topk_idx = a->topk_idx;
-        p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
-        p.light = light ? 1 : 0;
-        p.copied_topk_idx = a->copied_topk_idx;
-        p.pub = pub;
-        p.status = status;
-        p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
-        p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
-            p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
-        hipError_t err = launch_layout_kernel(p, stream);
+    if (do_layout && !plan.fused) {
+        hipError_t err = launch_layout_kernel(lay, stream);
         if (err != hipSuccess) return hip_fail(err, "dispatch layout launch");
     }
 
@@ -233,13 +287,13 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         m.do_expand = a->do_expand ? 1 : 0;
         m.payload = a->payload;
         m.row_bytes = H * elem_in;
-        m.flat = flat_ok ? 1 : 0;
-        m.publish = light ? 1 : 0;
-        m.chunks_padded = chunks_padded;
-        m.flat_per = flat_per;
-        m.chunk_counts_t = reinterpret_cast<const int32_t*>(ws + w.chunk_counts);
+        m.tab = lay.tab;
         m.pub = pub;
         m.status = status;
+        m.cast_pairs = a->tuning.cast_pairs; m.copy_vecs = a->tuning.copy_vecs;
+        m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
+        if (plan.fused) fill_fused(m, lay, plan, ws, w);
+
         hipError_t err = launch_dispatch_move(m, stream);
         if (err != hipSuccess) return hip_fail(err, "dispatch move launch");
 
@@ -295,6 +349,7 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
     p.do_expand = a->do_expand ? 1 : 0;
     p.multi_red = a->allow_multiple_reduction ? 1 : 0;
     p.status = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a->workspace));
+    p.vecs = a->tuning.combine_vecs;
     hipError_t err = launch_combine_kernel(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "combine launch");
     return DEEP_EP_HIP_OK;
@@ -349,6 +404,9 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         REQUIRE(a->recv_capacity >= 0 && a->recv_capacity < (int64_t(1) << 31), "recv_capacity out of range");
         REQUIRE(a->recv_x != nullptr || a->recv_capacity == 0, "recv_x is NULL");
         REQUIRE(a->send_head != nullptr || T == 0, "send_head is NULL");
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_BF16)
+            REQUIRE(a->num_scales == 0 && a->x_scales == nullptr && a->recv_x_scales == nullptr,
+                    "a BF16 payload carries no scales");
         if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8)
             REQUIRE(a->num_scales >= 0 && (a->num_scales == 0 || T == 0 || (a->x_scales != nullptr && a->recv_x_scales != nullptr)),
                     "x_scales / recv_x_scales is NULL");
@@ -367,27 +425,23 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
     pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
 
-    const int chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
-    const int chunks_padded = (chunks + 3) / 4 * 4;
-    const int flat = R * chunks_padded;
-    const int flat_per = flat <= 256 ? 4 : flat <= 512 ? 8 : 16;
-    const bool flat_ok = T > 0 && flat <= 1024 && !a->cached;
-    const bool light = do_layout && do_move && flat_ok && (R + E) <= 512 &&
-                       getenv("DEEP_EP_HIP_NO_LIGHT_LAYOUT") == nullptr;
+    const LaunchPlan plan = plan_launches(T, K, E, R, do_layout, do_move, a->payload, H, H * elem_in, a->tuning);
+    LayoutParams lay{};
+    lay.topk_idx = a->topk_idx;
+    lay.route_mask = with_topk ? nullptr : a->is_token_in_rank;
+    lay.T = T; lay.K = K; lay.E = E; lay.R = R; lay.E_l = E / R;
+    lay.pub = pub;
+    lay.status = status;
+    lay.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
+    lay.tab = carve_tables(ws, w, T, E);
+    lay.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
 
     if (do_layout) {
-        LayoutParams p{};
-        p.topk_idx = a->topk_idx;
-        p.route_mask = with_topk ? nullptr : a->is_token_in_rank;
-        p.T = T; p.K = K; p.E = E; p.R = R; p.E_l = E / R;
-        p.light = light ? 1 : 0;
-        p.pub = pub;
-        p.status = status;
-        p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
-        p.chunk_counts = reinterpret_cast<int32_t*>(ws + w.chunk_counts);
-            p.pos = reinterpret_cast<uint32_t*>(ws + w.pos);
-        hipError_t err = launch_layout_kernel(p, stream);
-        if (err != hipSuccess) return hip_fail(err, "intranode dispatch layout launch");
+        hipError_t err = hipSuccess;
+        if (!plan.fused) {
+            err = launch_layout_kernel(lay, stream);
+            if (err != hipSuccess) return hip_fail(err, "intranode dispatch layout launch");
+        }
 
         if (a->rank_prefix_matrix != nullptr || a->channel_prefix_matrix != nullptr ||
             a->recv_channel_prefix_matrix != nullptr) {
@@ -431,13 +485,13 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.do_expand = 0;
         m.payload = a->payload;
         m.row_bytes = H * elem_in;
-        m.flat = flat_ok ? 1 : 0;
-        m.publish = light ? 1 : 0;
-        m.chunks_padded = chunks_padded;
-        m.flat_per = flat_per;
-        m.chunk_counts_t = reinterpret_cast<const int32_t*>(ws + w.chunk_counts);
+        m.tab = lay.tab;
         m.pub = pub;
         m.status = status;
+        m.cast_pairs = a->tuning.cast_pairs; m.copy_vecs = a->tuning.copy_vecs;
+        m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
+        if (plan.fused) fill_fused(m, lay, plan, ws, w);
+
         m.rank_lanes = with_topk ? 0 : 1;
         m.slot_is_row = a->cached ? 1 : 0;
         m.zero_nonlocal_w = 1;
@@ -484,6 +538,7 @@ int deep_ep_hip_launch_intranode_combine(const deep_ep_hip_intranode_combine_arg
     p.rank_mode = 1;
     p.Kw = a->num_topk;
     p.status = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a->workspace));
+    p.vecs = a->tuning.combine_vecs;
     hipError_t err = launch_combine_kernel(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "intranode combine launch");
     return DEEP_EP_HIP_OK;
@@ -550,6 +605,7 @@ int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* a, void* 
     p.chunk_counts = reinterpret_cast<int32_t*>(ws + off); off = align_up(off + chunks * p.E_l * 4, 256);
     p.chunk_base = reinterpret_cast<int32_t*>(ws + off);   off = align_up(off + chunks * p.E_l * 4, 256);
     p.pos_expert = reinterpret_cast<int32_t*>(ws + off);
+    p.pairs = a->tuning.ll_pairs; p.threads = a->tuning.ll_threads; p.two_kernels = a->tuning.ll_two_kernels;
     hipError_t err = launch_ll_dispatch(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "low-latency dispatch launch");
     return DEEP_EP_HIP_OK;
@@ -582,6 +638,7 @@ int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* a, void* st
     p.lane_slot = a->lane_rows;
     p.out = static_cast<uint8_t*>(a->combined_x);
     p.status = reinterpret_cast<int32_t*>(a->workspace);
+    p.vecs = a->tuning.ll_combine_vecs;
     hipError_t err = launch_ll_combine(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "low-latency combine launch");
     return DEEP_EP_HIP_OK;

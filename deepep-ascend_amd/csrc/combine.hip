@@ -13,7 +13,7 @@
 // own term, in lane order.
 //
 // One wavefront owns one (token, column tile of kVecs * 512 channels).
-#include "common.cuh"
+#include "device_utils.h"
 #include "kernels.h"
 #include "../../include/deep_ep_hip.h"
 
@@ -223,8 +223,7 @@ hipError_t launch(CombineParams p, hipStream_t stream) {
 
 hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
-    const char* env = getenv("DEEP_EP_HIP_COMBINE_VECS");
-    int vecs = env != nullptr ? atoi(env) : 0;
+    int vecs = p.vecs;
     if (vecs == 0) vecs = (p.H * 2 <= 1024) ? 1 : 2;
     switch (vecs) {
         case 1: return launch<1>(p, stream);

@@ -142,10 +142,37 @@ __device__ __forceinline__ int small_div(int x, float rcp_d) {
     return int((float(x) + 0.5f) * rcp_d);
 }
 
-// Agent-scope relaxed load/store that bypass the per-CU vector cache, for values another
-// workgroup of the same launch has just produced.
+// Agent-scope relaxed load / store (no caching that another XCD's workgroups could not see through), for words
+// workgroups of one launch hand to each other.
 __device__ __forceinline__ int load_agent(const int* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(int* p, int v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// kThrough: an agent-scope (write-through) store; otherwise an ordinary one.
+template <bool kThrough>
+__device__ __forceinline__ void store_word(int* p, int v) {
+    if constexpr (kThrough) store_agent(p, v);
+    else *p = v;
+}
+template <bool kAgent>
+__device__ __forceinline__ int load_word(const int* p) {
+    if constexpr (kAgent) return load_agent(p);
+    else return *p;
+}
+// 16-byte agent-scope (write-through) store.  Written as an instruction because the language offers atomics of at
+// most 8 bytes; a store has no result register, so nothing the compiler tracks depends on its completion.
+__device__ __forceinline__ void store16_agent(void* p, const vec16& v) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(t) : "memory");
+}
+
+// Waits until every store this wavefront has issued is acknowledged.  After agent-scope stores this is all a
+// workgroup needs before it raises a flag for another workgroup: no cache-wide write-back is involved.
+__device__ __forceinline__ void wait_for_own_stores() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace deep_ep_hip

@@ -10,11 +10,19 @@
 //
 // Work decomposition: one wavefront owns one (token, column tile).  All 16-byte loads of the tile
 // are issued first, then the routing metadata is resolved while they are in flight, then the tile
-// is stored to each destination with 16-byte stores.  No LDS, no barriers.
-#include "common.cuh"
-#include "cast.cuh"
+// is stored to each destination with 16-byte stores.
+//
+// Single-launch mode ("fused"): the first workgroups of the grid are counting workgroups (one 256-token
+// chunk each, the code of the layout kernel); the last of them to finish publishes the handle tensors.
+// Mover workgroups issue their payload loads, then wait (first wavefront polls an agent-scope word, the
+// others sit at a workgroup barrier) until the counts are complete, and read what the counting
+// workgroups wrote with agent-scope loads.  Counting workgroups have the lowest workgroup ids, wait for
+// nothing and are therefore resident before any mover can wait for them; every wait is bounded.
+#include "device_utils.h"
+#include "fp8_cast.h"
 #include "kernels.h"
-#include "publish.cuh"
+#include "layout_count.h"
+#include "publish.h"
 #include "../../include/deep_ep_hip.h"
 
 namespace deep_ep_hip {
@@ -37,35 +45,56 @@ struct Route {
     float w;
 };
 
-__device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int lane, bool first_tile) {
-    Route r{-1, -1, -1, -1, -1, 0.f};
+// A word of the layout tables.  In a single-launch dispatch they were written by counting workgroups of the same
+// launch, possibly through another XCD's L2: the writers release them (write back) before any gate opens, and no
+// mover touches a table line before it has passed its gate, so this XCD's caches cannot hold an older copy of
+// the line and an ordinary load fetches what was written.  (Each table line has a single writer.)
+template <bool kFused>
+__device__ __forceinline__ int layout_word(const int32_t* at) {
+    return *at;
+}
+
+// What the caller gave for one (token, lane): independent of the layout pass, so a single-launch dispatch loads
+// it together with the payload, before it knows that the layout is complete.
+struct RouteInputs {
+    int64_t raw;         // topk_idx entry
+    uint8_t mask_byte;   // is_token_in_rank entry (mask routing)
+    float w;             // topk_weights entry
+};
+
+__device__ __forceinline__ RouteInputs load_route_inputs(const MoveParams& p, int t, int lane) {
+    RouteInputs in{-1, 0, 0.f};
+    if (lane < p.K) {
+        const int64_t at = int64_t(t) * p.K + lane;
+        if (p.route_mask != nullptr) in.mask_byte = p.route_mask[at];
+        else if (!(p.cached && p.rank_lanes)) in.raw = p.topk_idx[at];
+        if (p.topk_weights != nullptr) in.w = p.topk_weights[at];
+    }
+    return in;
+}
+
+template <bool kFused>
+__device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteInputs& in, int t, int lane, bool first_tile) {
+    Route r{-1, -1, -1, -1, -1, in.w};
     const int chunk = t / kLayoutChunk;
 
     // ---- issue every load that does not depend on another one, then consume: one memory round trip ----
-    int64_t raw = -1;
-    uint8_t mask_byte = 0;
+    int64_t raw = in.raw;
+    const uint8_t mask_byte = in.mask_byte;
     uint32_t word = 0xffffffffu;     // cached: handle slot (-1 = none); otherwise the packed positions of the layout pass
     const bool rank_lanes_cached = p.cached && p.rank_lanes;
     if (lane < p.K) {
         const int64_t at = int64_t(t) * p.K + lane;
-        if (p.route_mask != nullptr) mask_byte = p.route_mask[at];
-        else if (!rank_lanes_cached) raw = p.topk_idx[at];
-        if (p.topk_weights != nullptr) r.w = p.topk_weights[at];
-        const uint32_t* words = p.cached ? reinterpret_cast<const uint32_t*>(p.cached_slot) : p.pos;
-        word = words[at];
+        const int32_t* words = p.cached ? p.cached_slot : reinterpret_cast<const int32_t*>(p.pos);
+        word = uint32_t(layout_word<kFused>(words + at));
     }
-    // Flat mode: per-rank chunk counts, flattened [R][chunks_padded]; lane L holds entries [L * per, (L + 1) * per).
-    const int per = p.flat_per;
-    vec16 counts[4];
-    if (p.flat) {
-        const int nflat = p.R * p.chunks_padded;
-        // addresses are clamped instead of predicated (and masked only when consumed) so that the loads do not
-        // wait for each other
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            counts[u] = vec16{0, 0, 0, 0};
-            if (u * 4 < per) counts[u] = load16(p.chunk_counts_t + min(lane * per + u * 4, nflat - 4));   // uniform branch
-        }
+    // Wave lane q < R fetches the base row of (rank q, this token's chunk) and the start of rank q's bucket; the
+    // routing lanes pick theirs up by shuffle.  (More than 64 ranks: each master lane fetches its own pair below.)
+    const bool bases_by_lane = !p.cached && p.R <= kWaveSize;
+    int base_of_rank = 0, start_of_rank = 0;
+    if (bases_by_lane && lane < p.R) {
+        base_of_rank = layout_word<kFused>(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded + chunk);
+        start_of_rank = layout_word<kFused>(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded);
     }
 
     int slot = -1, epos = -1;
@@ -89,52 +118,23 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
     }
     if (r.e >= 0) r.d = small_div(r.e, p.rcp_E_l);
     else slot = -1;
-    if (p.flat) {
-        // Exclusive prefix of the per-rank chunk counts in (rank, chunk) order; a wave scan joins the lanes.
-        // The prefix at (d, chunk) is at once the start of bucket d and the rows that earlier chunks put
-        // into it, so no other table is needed.
-        int ex[16];
-        int sum = 0;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const bool held = u * 4 < per && lane * per + u * 4 < p.R * p.chunks_padded;
-            const vec16 v = held ? counts[u] : vec16{0, 0, 0, 0};
-            ex[4 * u] = sum; sum += int(v.x);
-            ex[4 * u + 1] = sum; sum += int(v.y);
-            ex[4 * u + 2] = sum; sum += int(v.z);
-            ex[4 * u + 3] = sum; sum += int(v.w);
+    if (!p.cached) {
+        int base, start;
+        if (bases_by_lane) {
+            const int from = r.d >= 0 ? r.d : 0;
+            base = __shfl(base_of_rank, from, kWaveSize);
+            start = __shfl(start_of_rank, from, kWaveSize);
+        } else {
+            const int64_t row = int64_t(r.d >= 0 && slot >= 0 ? r.d : 0) * p.tab.chunks_padded;
+            base = layout_word<kFused>(p.tab.rank_bases + row + chunk);
+            start = layout_word<kFused>(p.tab.rank_bases + row);
         }
-        const int lane_base = wave_inclusive_sum(sum) - sum;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) ex[i] += lane_base;
-        // prefix at flat position f: held by lane f / per as its entry f % per (every lane takes part)
-        auto prefix_at = [&](int f) {
-            const int owner = f / per, off = f - owner * per;
-            int got = 0;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                if (i < per) {
-                    const int v = __shfl(ex[i], owner, kWaveSize);
-                    if (i == off) got = v;
-                }
-            }
-            return got;
-        };
-        const int fd = (r.d >= 0 ? r.d : 0) * p.chunks_padded;
-        const int bucket_start = prefix_at(fd);
-        const int before = prefix_at(fd + chunk);
         if (r.d >= 0 && slot >= 0) {
-            r.row_c = before + slot;
-            slot = r.row_c - bucket_start;      // slot inside the destination bucket
+            r.row_c = base + slot;
+            slot = r.row_c - start;             // slot inside the destination bucket
         }
     } else if (r.e >= 0 && slot >= 0) {
-        if (p.slot_is_row) {
-            r.row_c = slot;
-        } else {
-            // large R * chunks: each master lane sums its own bucket's row
-            if (!p.cached) slot += row_prefix(p.chunk_counts_t, p.chunks_padded, r.d, chunk);
-            r.row_c = (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
-        }
+        r.row_c = p.slot_is_row ? slot : (r.d > 0 ? p.psum_rank[r.d - 1] : 0) + slot;
     }
     if (first_tile && !p.cached && lane < p.K && p.dst_buffer_slot_idx != nullptr)
         p.dst_buffer_slot_idx[int64_t(t) * p.K + lane] = (r.e >= 0 && slot >= 0) ? p.rank_idx * p.M + slot : -1;
@@ -155,15 +155,12 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, int t, int l
         const int rj = read_lane(r.row_c, j);
         if (r.d >= 0 && dj == r.d && rj >= 0) r.my_row = rj;
     }
-    int expert_rows_before = 0;
-    if (p.do_expand && !p.cached && r.e >= 0)    // rows that earlier chunks put into this lane's expert
-        expert_rows_before = row_prefix(p.chunk_counts_t, p.chunks_padded, p.R + r.e, chunk);
     if (p.do_expand && r.e >= 0) {
         if (p.cached) {
             if (r.my_row >= 0 && r.my_row < p.recv_capacity)
                 r.erow = p.recv_src_metadata[int64_t(r.my_row) * (p.K + 2) + 2 + lane];
         } else {
-            r.erow = p.expert_start[r.e] + expert_rows_before + epos;
+            r.erow = layout_word<kFused>(p.tab.expert_bases + int64_t(chunk) * p.tab.experts_padded + r.e) + epos;
         }
     }
     return r;
@@ -257,23 +254,143 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
     return __ballot(row_of_lane >= 0);
 }
 
-// Layout and move in one call: workgroup 0 sums the transposed chunk counts and publishes the handle tensors.
-// Every thread of the workgroup must call this before any early exit.
-__device__ __forceinline__ void publish_from_chunk_counts(const MoveParams& p) {
-    extern __shared__ int publish_lds[];
-    publish_from_transposed_counts<kThreads>(p.pub, p.chunk_counts_t, p.chunks_padded, publish_lds);
+// ---- single-launch dispatch ----
+//
+// Grid: C counting workgroups (one 256-token chunk each), one publishing workgroup, then the movers.  Hand-offs
+// between workgroups of one launch cost a trip to the memory side each (about 0.4 us on an idle GPU), so the
+// protocol keeps them few, and none of its words is touched by more than a few dozen workgroups (agent-scope
+// atomics on one address serialise at about 11 ns each):
+//   - counting workgroup c stores its chunk totals and sets counts_done[c]; then it works out and stores the
+//     positions of its tokens and sets positions_done[c];
+//   - the publisher waits for all counts_done flags, writes the rank rows of the base table and the per-rank
+//     outputs (while the counting workgroups are still busy with their positions), waits for all positions_done
+//     flags, clears both sets of flags and opens every gate (stage 1); then it publishes the per-expert outputs
+//     (and, for the expanded layout, the expert base table) and opens every gate a second time (stage 2);
+//   - mover workgroup m watches gate m % kDispatchGates (each gate a cache line of its own) until it shows the
+//     stage the launch needs (compact layout: 1; expanded layout, whose rows are placed through the published
+//     expert regions: 2), then passes it.
+// Everything handed over is stored at agent scope (written through), so a workgroup only waits for its own
+// stores before it raises a flag: no cache-wide write-back or invalidate runs while the movers stream through
+// the same L2.
+// A gate is only ever advanced with a wrapping increment (0, 1, ..., limit, 0).  Gate g is passed by n_g movers,
+// limit = 1 + n_g, and receives exactly 2 + n_g increments per launch, so it is back at 0 when the launch ends and
+// nobody has to know who was last.  No mover increments a gate before it has seen the stage it needs, hence a gate
+// value >= stage means what it says, and the wrap to 0 happens only after all of the gate's movers have passed.
+// Counting and publishing workgroups have the lowest workgroup ids and wait for nothing that is dispatched after
+// them, so every wait ends; each is bounded anyway and reports DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT.
+constexpr unsigned kLayoutSpinLimit = 1u << 22;      // polls (each with a short sleep) before giving up: seconds
+
+__device__ __forceinline__ unsigned movers_of_gate(const MoveParams& p, unsigned gate) {
+    return (p.num_movers + unsigned(kDispatchGates) - 1u - gate) / unsigned(kDispatchGates);
+}
+
+__device__ __forceinline__ void advance_gate(const MoveParams& p, unsigned gate) {
+    atomicInc(p.gates + gate * kDispatchGateStride, 1u + movers_of_gate(p, gate));
+}
+
+__device__ __forceinline__ void open_all_gates(const MoveParams& p) {
+    for (unsigned g = threadIdx.x; g < unsigned(kDispatchGates); g += kThreads) advance_gate(p, g);
+}
+
+__device__ __forceinline__ void fused_count_block(const MoveParams& p) {
+    extern __shared__ uint64_t count_lds[];
+    const int c = int(blockIdx.x);
+    int32_t* counts_done = p.chunk_done + c;
+    int32_t* positions_done = p.chunk_done + kMaxCountBlocks + c;
+    count_chunk<8, true>(p.lay, c, p.count_blocks, count_lds, [&]() {
+        wait_for_own_stores();
+        __syncthreads();
+        if (threadIdx.x == 0) store_agent(counts_done, 1);
+    });
+    wait_for_own_stores();
+    __syncthreads();
+    if (threadIdx.x == 0) store_agent(positions_done, 1);
+}
+
+// All flags[0..n) set?  Polls (bounded), then clears them for the next launch.  Every thread must call it.
+__device__ __forceinline__ void await_and_clear_flags(const MoveParams& p, int32_t* flags, int n) {
+    bool complete = true;
+    for (int i = threadIdx.x; i < n; i += kThreads) {
+        unsigned polls = 0;
+        while (load_agent(flags + i) == 0 && polls < kLayoutSpinLimit) {
+            __builtin_amdgcn_s_sleep(1);
+            ++polls;
+        }
+        if (polls == kLayoutSpinLimit) complete = false;
+        store_agent(flags + i, 0);
+    }
+    if (!complete) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+    __syncthreads();
+}
+
+__device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
+    extern __shared__ uint64_t count_lds[];
+    const PublishLds lds = carve_publish_lds(reinterpret_cast<int*>(count_lds), p.R, p.E);
+    const LayoutTables& tab = p.lay.tab;
+
+    await_and_clear_flags(p, p.chunk_done, p.count_blocks);
+    publish_ranks_flat<kThreads>(p.pub, tab, lds);
+    wait_for_own_stores();
+    await_and_clear_flags(p, p.chunk_done + kMaxCountBlocks, p.count_blocks);
+    open_all_gates(p);                                                        // stage 1
+
+    // The expert tables have one writer per cache line and this workgroup has not touched them before, so
+    // ordinary loads fetch what the counting workgroups wrote through.
+    sum_expert_columns<kThreads>(tab, p.R, p.E, p.count_blocks, lds.totals);
+    publish_experts<kThreads>(p.pub, lds);
+    if (p.do_expand) {
+        __syncthreads();
+        write_expert_bases<kThreads, true>(tab, p.E, p.count_blocks, lds);
+    }
+    wait_for_own_stores();
+    __syncthreads();
+    open_all_gates(p);                                                        // stage 2
+}
+
+// First wavefront of a mover workgroup: its first look at the gate goes out together with its payload loads (on a
+// busy GPU every trip to the memory side takes as long as they do); it then waits (bounded) until the layout is as
+// complete as this launch needs it and passes the gate.  The other wavefronts meet it at a workgroup barrier.
+__device__ __forceinline__ const int* gate_of(const MoveParams& p, unsigned mover) {
+    return reinterpret_cast<const int*>(p.gates + (mover % unsigned(kDispatchGates)) * kDispatchGateStride);
+}
+
+__device__ __forceinline__ void pass_gate(const MoveParams& p, unsigned mover, int first_look) {
+    const int* word = gate_of(p, mover);
+    const unsigned need = p.do_expand ? 2u : 1u;
+    unsigned seen = unsigned(first_look);
+    unsigned polls = 0;
+    while (seen < need && polls < kLayoutSpinLimit) {
+        __builtin_amdgcn_s_sleep(2);
+        seen = unsigned(load_agent(word));
+        ++polls;
+    }
+    if (threadIdx.x == 0) {
+        if (seen < need) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+        advance_gate(p, mover % unsigned(kDispatchGates));
+    }
 }
 
 // ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
-template <int kVecs>
+template <int kVecs, bool kFused>
 __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
-    if (p.publish && blockIdx.x == 0) publish_from_chunk_counts(p);
+    if constexpr (kFused) {
+        if (blockIdx.x <= unsigned(p.count_blocks)) {
+            if (blockIdx.x < unsigned(p.count_blocks)) fused_count_block(p);
+            else fused_publish_block(p);
+            return;
+        }
+    }
     const int lane = threadIdx.x & 63;
-    const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+    const unsigned mover = blockIdx.x - (kFused ? unsigned(p.count_blocks) + 1u : 0u);
+    int first_look = 0;
+    if constexpr (kFused)
+        if (threadIdx.x < kWaveSize) first_look = load_agent(gate_of(p, mover));
+    const unsigned block = p.xcd_remap ? xcd_contiguous_block(mover, p.num_movers) : mover;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
-    if (work >= unsigned(p.T) * unsigned(p.tiles)) return;
-    const int t = int(work / unsigned(p.tiles));
-    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
+    const bool has_work = work < unsigned(p.T) * unsigned(p.tiles);
+    if (!has_work && !kFused) return;
+    const int t = has_work ? int(work / unsigned(p.tiles)) : 0;
+    const int tile = has_work ? int(work - unsigned(t) * unsigned(p.tiles)) : 0;
 
     vec16 v[kVecs];
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
@@ -281,10 +398,19 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
     for (int i = 0; i < kVecs; ++i) {
         const int off = (tile * kVecs + i) * 1024 + lane * 16;
         v[i] = vec16{0, 0, 0, 0};
-        if (off < p.row_bytes) v[i] = load16_stream(src + off);
+        if (has_work && off < p.row_bytes) v[i] = load16_stream(src + off);
     }
 
-    const Route r = resolve_route(p, t, lane, tile == 0);
+    const RouteInputs route_in = load_route_inputs(p, t, lane);
+    if constexpr (kFused) {
+        // Payload and routing inputs are in flight; nothing that reads the layout may be issued before the first
+        // wavefront has passed the gate.
+        if (threadIdx.x < kWaveSize) pass_gate(p, mover, first_look);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (!has_work) return;
+    }
+    const Route r = resolve_route<kFused>(p, route_in, t, lane, tile == 0);
     if (tile == 0) write_token_metadata(p, r, t, lane);
 
     int row_of_lane;
@@ -308,15 +434,26 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
 }
 
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
-template <int kPairs>
+template <int kPairs, bool kFused>
 __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
-    if (p.publish && blockIdx.x == 0) publish_from_chunk_counts(p);
+    if constexpr (kFused) {
+        if (blockIdx.x <= unsigned(p.count_blocks)) {
+            if (blockIdx.x < unsigned(p.count_blocks)) fused_count_block(p);
+            else fused_publish_block(p);
+            return;
+        }
+    }
     const int lane = threadIdx.x & 63;
-    const unsigned block = p.xcd_remap ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+    const unsigned mover = blockIdx.x - (kFused ? unsigned(p.count_blocks) + 1u : 0u);
+    int first_look = 0;
+    if constexpr (kFused)
+        if (threadIdx.x < kWaveSize) first_look = load_agent(gate_of(p, mover));
+    const unsigned block = p.xcd_remap ? xcd_contiguous_block(mover, p.num_movers) : mover;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
-    if (work >= unsigned(p.T) * unsigned(p.tiles)) return;
-    const int t = int(work / unsigned(p.tiles));
-    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
+    const bool has_work = work < unsigned(p.T) * unsigned(p.tiles);
+    if (!has_work && !kFused) return;
+    const int t = has_work ? int(work / unsigned(p.tiles)) : 0;
+    const int tile = has_work ? int(work - unsigned(t) * unsigned(p.tiles)) : 0;
 
     vec16 in[kPairs][2];
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
@@ -325,7 +462,7 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
         const int elem = (tile * kPairs + q) * 1024 + lane * 16;
         in[q][0] = vec16{0, 0, 0, 0};
         in[q][1] = vec16{0, 0, 0, 0};
-        if (elem < p.H) {
+        if (has_work && elem < p.H) {
             if (p.plain_loads) {
                 in[q][0] = load16(src + int64_t(elem) * 2);
                 in[q][1] = load16(src + int64_t(elem) * 2 + 16);
@@ -336,7 +473,16 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
         }
     }
 
-    const Route r = resolve_route(p, t, lane, tile == 0);
+    const RouteInputs route_in = load_route_inputs(p, t, lane);
+    if constexpr (kFused) {
+        // Payload and routing inputs are in flight; nothing that reads the layout may be issued before the first
+        // wavefront has passed the gate.
+        if (threadIdx.x < kWaveSize) pass_gate(p, mover, first_look);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (!has_work) return;
+    }
+    const Route r = resolve_route<kFused>(p, route_in, t, lane, tile == 0);
     if (tile == 0) write_token_metadata(p, r, t, lane);
 
     vec16 out[kPairs];
@@ -461,50 +607,70 @@ __global__ __launch_bounds__(kThreads) void fill_tail_kernel(const FillTailParam
 }
 
 size_t move_lds_bytes(const MoveParams& p) {
-    return p.publish ? publish_lds_bytes(p.R, p.E, kThreads) : 0;
+    if (!p.fused) return 0;
+    const size_t publish = publish_lds_bytes(p.R, p.E, kThreads);
+    const size_t bitmap = count_lds_bytes(p.R, p.E);
+    return bitmap > publish ? bitmap : publish;
+}
+
+// Grid: the counting workgroups of a single-launch dispatch come first.
+unsigned move_grid(MoveParams& p, int64_t waves) {
+    p.num_movers = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    return p.num_movers + unsigned(p.fused ? p.count_blocks + 1 : 0);
 }
 
 template <int kVecs>
 hipError_t launch_copy(MoveParams p, hipStream_t stream) {
     p.tiles = (p.row_bytes + kVecs * 1024 - 1) / (kVecs * 1024);
-    const int64_t waves = int64_t(p.T) * p.tiles;
-    const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(dispatch_copy_kernel<kVecs>, dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    const unsigned blocks = move_grid(p, int64_t(p.T) * p.tiles);
+    if (p.fused) hipLaunchKernelGGL((dispatch_copy_kernel<kVecs, true>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    else hipLaunchKernelGGL((dispatch_copy_kernel<kVecs, false>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 
 template <int kPairs>
 hipError_t launch_cast(MoveParams p, hipStream_t stream) {
     p.tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
-    const int64_t waves = int64_t(p.T) * p.tiles;
-    const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(dispatch_cast_kernel<kPairs>, dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    const unsigned blocks = move_grid(p, int64_t(p.T) * p.tiles);
+    if (p.fused) hipLaunchKernelGGL((dispatch_cast_kernel<kPairs, true>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    else hipLaunchKernelGGL((dispatch_cast_kernel<kPairs, false>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
-}
-
-int tuning_override(const char* name) {
-    const char* v = getenv(name);
-    return v != nullptr ? atoi(v) : 0;
 }
 
 }  // namespace
 
+// Column tile of a move launch: 1024-channel segments per wavefront for the fused cast, KB of row per wavefront for
+// the pass-through payloads.
+static int move_tile(const MoveParams& p) {
+    if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
+        // Two segments (2048 channels, 8 wavefronts per SIMD) measured best at hidden 7168: 92.8 us per dispatch
+        // against 93.7 (4 segments) and 96.9 (7 segments, one wavefront per token).
+        if (p.cast_pairs != 0) return p.cast_pairs;
+        return p.H <= 1024 ? 1 : 2;
+    }
+    // Large, bandwidth-bound calls: one 1 KB segment per wavefront measured best for this write-heavy stream (8192
+    // BF16 rows of 14 KB: 143 us per dispatch against 155-159 us with 2, 4, 7 or 8 segments).  Small, latency-bound
+    // calls: up to 4 KB per wavefront, so that fewer wavefronts repeat the routing work (4096 rows of 4 KB: 26 us
+    // against 32 us with 1 KB segments).
+    if (p.copy_vecs != 0) return p.copy_vecs;
+    const int kb = (p.row_bytes + 1023) / 1024;
+    const bool large = int64_t(p.T) * p.row_bytes >= (int64_t(64) << 20);
+    return large ? 1 : (kb <= 1 ? 1 : kb <= 2 ? 2 : 4);
+}
+
+int64_t dispatch_move_workgroups(const MoveParams& p) {
+    const int tile = move_tile(p);
+    const int64_t tiles = p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8 ? (p.H + tile * 1024 - 1) / (tile * 1024)
+                                                                    : (p.row_bytes + tile * 1024 - 1) / (tile * 1024);
+    return (int64_t(p.T) * tiles + kWavesPerBlock - 1) / kWavesPerBlock;
+}
+
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
     p.rcp_E_l = 1.0f / float(p.E_l);
-    {
-        const char* v = getenv("DEEP_EP_HIP_XCD_REMAP");
-        p.xcd_remap = v != nullptr ? atoi(v) : 0;
-        const char* pl = getenv("DEEP_EP_HIP_PLAIN_LOADS");
-        p.plain_loads = pl != nullptr ? atoi(pl) : 0;
-    }
+    const int tile = move_tile(p);
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
-        // Column tile = kPairs * 1024 channels per wavefront.  Two pairs (2048 channels, 8 waves per SIMD)
-        // measured best at hidden 7168: 92.8 us per dispatch against 93.7 (4 pairs) and 96.9 (7 pairs, one
-        // wavefront per token).
-        int pairs = tuning_override("DEEP_EP_HIP_CAST_PAIRS");
-        if (pairs == 0) pairs = p.H <= 1024 ? 1 : 2;
-        switch (pairs) {
+        switch (tile) {
             case 1: return launch_cast<1>(p, stream);
             case 2: return launch_cast<2>(p, stream);
             case 7: return launch_cast<7>(p, stream);
@@ -512,17 +678,7 @@ hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
             default: return launch_cast<4>(p, stream);
         }
     }
-    // Pass-through payloads.  Large, bandwidth-bound calls: one 1 KB segment per wavefront measured best for this
-    // write-heavy stream (8192 BF16 rows of 14 KB: 143 us per dispatch against 155-159 us with 2, 4, 7 or 8
-    // segments).  Small, latency-bound calls: up to 4 KB per wavefront, so that fewer wavefronts repeat the routing
-    // work (4096 rows of 4 KB: 26 us against 32 us with 1 KB segments).
-    int vecs = tuning_override("DEEP_EP_HIP_COPY_VECS");
-    if (vecs == 0) {
-        const int kb = (p.row_bytes + 1023) / 1024;
-        const bool large = int64_t(p.T) * p.row_bytes >= (int64_t(64) << 20);
-        vecs = large ? 1 : (kb <= 1 ? 1 : kb <= 2 ? 2 : 4);
-    }
-    switch (vecs) {
+    switch (tile) {
         case 1: return launch_copy<1>(p, stream);
         case 2: return launch_copy<2>(p, stream);
         case 4: return launch_copy<4>(p, stream);

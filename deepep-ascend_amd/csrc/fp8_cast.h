@@ -7,7 +7,7 @@
 // half of all amax values, so it is not used here.)
 #pragma once
 
-#include "common.cuh"
+#include "device_utils.h"
 
 namespace deep_ep_hip {
 

@@ -8,18 +8,45 @@
 
 namespace deep_ep_hip {
 
+// Single-launch dispatch: number of gates the movers spread over, and the distance between two gates in 32-bit
+// words (one cache line each).
+constexpr int kDispatchGates = 256;
+constexpr int kDispatchGateStride = 32;
+constexpr int kMaxCountBlocks = 1024;
+
 // Byte offsets of the regions carved out of the caller's workspace.
 struct WorkspaceLayout {
     size_t status;         // int32: device status bits
     size_t done_counter;   // uint32: workgroups of the layout kernel that have finished
     size_t totals;         // int32[2]: total compact rows, total expanded rows (incl. padding)
+    size_t chunk_done;     // int32[2][1024]: per-chunk completion flags of a single-launch dispatch
+    size_t gates;          // uint32[kDispatchGates], one per 128-byte line: stage counters of a single-launch dispatch
     size_t expert_start;   // int32[E]: first expanded row of each expert
-    size_t chunk_counts;   // int32[R+E][C padded to a multiple of 4]: per-chunk totals, transposed
+    size_t rank_counts;    // int32[R][C padded to a multiple of 4]: per-chunk totals of the rank buckets, transposed
+    size_t rank_bases;     // int32[R][C padded]: first compact row of every (rank, chunk)
+    size_t expert_counts;  // int32[C][E padded to a multiple of 32]: per-chunk totals of the expert buckets
+    size_t expert_bases;   // int32[C][E padded]: first expanded row of every (chunk, expert)
     size_t pos;            // uint32[Tmax*K]: chunk-relative positions, rank slot | expert position << 16
     size_t total_bytes;
 };
 
 WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_experts, int num_ranks);
+
+// The tables the layout pass leaves in the workspace for the move kernels.  A chunk is 256 consecutive tokens.
+//   rank_counts[r][c]    rows chunk c puts into rank r's bucket (transposed: consumers prefix-sum along a row)
+//   rank_bases[r][c]     first compact row of (rank r, chunk c) = rows of lower ranks + rows of earlier chunks;
+//                        rank_bases[r][0] is the start of rank r's bucket
+//   expert_counts[c][e]  rows chunk c puts into expert e's region (one writer per cache line: chunk c's workgroup)
+//   expert_bases[c][e]   first expanded row of (chunk c, expert e) = start of the region + rows of earlier chunks
+// A row is then "base of (bucket, chunk) + position inside the chunk".
+struct LayoutTables {
+    int32_t* rank_counts;
+    int32_t* rank_bases;
+    int32_t* expert_counts;
+    int32_t* expert_bases;
+    int chunks_padded;    // row length of the rank tables (chunks rounded up to a multiple of 4)
+    int experts_padded;   // row length of the expert tables (experts rounded up to a multiple of 32)
+};
 
 // Where the public results of the layout computation go (any pointer may be NULL).
 struct PublishParams {
@@ -41,15 +68,15 @@ struct LayoutParams {
     const int64_t* topk_idx;
     const uint8_t* route_mask;       // [T, R] bool: when set, lane r of token t is "rank r, if the mask says so" (K = E = R)
     int T, K, E, R, E_l;
-    int light;            // 1: only count; the move kernel of the same call sums the chunk totals and publishes
-    int chunks_padded;    // row length of the transposed chunk counts (set by the launcher)
+    int count_only;       // 1: a counting workgroup of a single-launch dispatch (somebody else publishes)
     int vec_idx;          // topk_idx is 16-byte aligned (set by the launcher)
     uint8_t* is_token_in_rank;       // optional
     int64_t* copied_topk_idx;        // optional
     PublishParams pub;
     int32_t* status;
     uint32_t* done_counter;
-    int32_t* chunk_counts;           // [R + E][chunks_padded]
+    LayoutTables tab;                // the base tables are optional (layout-only calls have no use for them)
+    int expert_bases;                // 1: also tab.expert_bases (expanded layout)
     uint32_t* pos;                   // optional (layout-only calls skip the per-lane positions)
 };
 
@@ -83,14 +110,19 @@ struct MoveParams {
     int tiles;           // column tiles per token
     int xcd_remap;       // give each XCD a contiguous token range
     int plain_loads;     // payload loads without the non-temporal hint
-    // Row bases come from the transposed chunk counts of the layout pass.
-    int flat;            // 1: R * chunks_padded <= 1024, a wavefront prefix-sums the whole rank part at once
-    int publish;         // 1: layout and move in one call (compact layout): workgroup 0 sums and publishes
-    int chunks_padded;   // row length of chunk_counts_t
-    int flat_per;        // rank-part entries each lane scans (4, 8 or 16)
-    const int32_t* chunk_counts_t;   // [R + E][chunks_padded]
-    PublishParams pub;   // written by workgroup 0
+    int cast_pairs;      // forced column tile of the fused cast, 0 = choose
+    int copy_vecs;       // forced column tile of the pass-through kernels, 0 = choose
+    LayoutTables tab;    // written by the layout pass
+    PublishParams pub;   // single-launch dispatch: what counting workgroup 0 publishes
     int32_t* status;
+    // Single-launch dispatch: the first count_blocks workgroups of the grid count (one 256-token chunk each), the
+    // last of them to finish publishes; the movers wait on `sync` before they read any of it.
+    int fused;
+    int count_blocks;
+    unsigned num_movers;     // mover workgroups (set by the launcher)
+    LayoutParams lay;        // what the counting workgroups need (lay.pub is unused: `pub` above is published)
+    int32_t* chunk_done;     // [2][kMaxCountBlocks] flags of the counting workgroups: counts stored, positions stored
+    uint32_t* gates;         // [kDispatchGates] wrapping stage counters, kDispatchGateStride words apart
     // V1 (intranode) conventions
     int rank_lanes;          // routing lanes are ranks (mask routing or a cached send_head), K == R
     int slot_is_row;         // cached_slot holds rows of the receive buffer, not rank * M + slot
@@ -100,6 +132,8 @@ struct MoveParams {
 };
 
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream);
+// Mover workgroups launch_dispatch_move would start for p (p.T, p.H, p.row_bytes, p.payload and the tile overrides set).
+int64_t dispatch_move_workgroups(const MoveParams& p);
 
 struct PadParams {
     uint8_t* recv_x;
@@ -156,6 +190,7 @@ struct CombineParams {
     // rank order; weights [rows, Kw] are summed over the token's rows.
     int rank_mode;
     int Kw;
+    int vecs;            // forced column tile, 0 = choose
 };
 
 hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream);
@@ -190,6 +225,8 @@ struct LLDispatchParams {
     int32_t* chunk_counts;   // [C][E_l]
     int32_t* chunk_base;     // [C][E_l]
     int32_t* pos_expert;     // [S*stride*K]
+    // launch-shape overrides, 0 = choose
+    int pairs, threads, two_kernels;
 };
 
 hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream);
@@ -206,6 +243,7 @@ struct LLCombineParams {
     const int32_t* lane_slot;    // optional: what the dispatch recorded; replaces the search through src_info
     uint8_t* out;
     int32_t* status;
+    int vecs;                    // forced column tile, 0 = choose
 };
 
 hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream);

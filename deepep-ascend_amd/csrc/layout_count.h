@@ -1,0 +1,170 @@
+// Counting step of the dispatch layout, shared by the stand-alone layout kernel and by the counting workgroups
+// at the front of a single-launch dispatch.
+//
+// A workgroup of 256 threads owns a chunk of 256 consecutive tokens (one thread per token).  Each wavefront
+// sets its lane bit in an LDS bitmap word per rank and per expert (ds_or_b64), so that
+//   count  = popcount(bitmap)                      and
+//   position of token t among chunk tokens routed to the same bucket = popcount(bitmap & lanes below t)
+// with no ordering-dependent atomics: placement is a pure function of the input.  Chunk totals go to the count
+// tables of the workspace.
+//
+// Counts what csrc/kernels/legacy/layout.cu:10-122 and the notify warps of
+// deep_ep/include/deep_ep/impls/dispatch.cuh:79-199 count.
+#pragma once
+
+#include "device_utils.h"
+#include "kernels.h"
+#include "../../include/deep_ep_hip.h"
+
+namespace deep_ep_hip {
+
+static_assert(kLayoutChunk == 4 * kWaveSize, "the packed before-wave word holds three fields");
+
+// LDS the counting step needs: the bitmap words [(R + E)][4] and one packed word per bucket (see below).
+inline size_t count_lds_bytes(int R, int E) {
+    return size_t(R + E) * (kLayoutChunk / kWaveSize) * sizeof(uint64_t) + size_t(R + E) * sizeof(uint32_t);
+}
+
+struct NoHook {
+    __device__ void operator()() const {}
+};
+
+// bitmap: LDS of count_lds_bytes(R, E) bytes.  Must be called by all 256 threads of the workgroup.
+// kThrough: positions and chunk totals are stored at agent scope (a workgroup of the same launch reads them).
+// counts_stored() is called by every thread once the chunk totals have been stored, before the positions are
+// worked out.
+template <int KMAX, bool kThrough, class Hook = NoHook>
+__device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chunk, const int num_chunks,
+                                            uint64_t* bitmap, Hook counts_stored = Hook()) {
+    constexpr int kThreads = kLayoutChunk;
+    constexpr int kWaves = kThreads / kWaveSize;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int t = chunk * kThreads + tid;
+    const int n = p.R + p.E;
+    const bool active = t < p.T;
+
+    // The index loads go out first (they are the longest wait of the pass), before anything that could alias
+    // them is stored; the bitmap is cleared while they are in flight.
+    int64_t raw[KMAX];
+    if (p.route_mask != nullptr) {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+            raw[k] = (active && k < p.K && p.route_mask[int64_t(t) * p.K + k] != 0) ? int64_t(k) : int64_t(-1);
+    } else if (KMAX == 8 && p.K == 8 && p.vec_idx) {
+        if (active) {
+            const vec16* src = reinterpret_cast<const vec16*>(p.topk_idx + int64_t(t) * 8);
+            vec16 q[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) q[i] = src[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                raw[2 * i] = int64_t(uint64_t(q[i].x) | (uint64_t(q[i].y) << 32));
+                raw[2 * i + 1] = int64_t(uint64_t(q[i].z) | (uint64_t(q[i].w) << 32));
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) raw[k] = -1;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) raw[k] = (active && k < p.K) ? p.topk_idx[int64_t(t) * p.K + k] : int64_t(-1);
+    }
+
+    for (int i = tid; i < n * kWaves; i += kThreads) bitmap[i] = 0ull;
+    __syncthreads();
+
+    int e[KMAX], d[KMAX];
+    int flags = 0;
+    const float rcp_experts_per_rank = 1.0f / float(p.E_l);
+    const uint64_t my_bit = 1ull << lane;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        int ev = -1;
+        if (raw[k] >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+        else if (raw[k] >= 0) ev = int(raw[k]);
+        e[k] = ev;
+        d[k] = ev >= 0 ? small_div(ev, rcp_experts_per_rank) : -1;
+        if (ev >= 0) {
+            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[(p.R + ev) * kWaves + wave]), my_bit);
+            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[d[k] * kWaves + wave]), my_bit);
+        }
+    }
+    if (p.copied_topk_idx != nullptr && active) {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+            if (k < p.K) p.copied_topk_idx[int64_t(t) * p.K + k] = raw[k];
+    }
+    __syncthreads();
+
+    // Per bucket: the chunk total goes out and the bits set by the wavefronts before each wavefront are packed into one LDS word (three 10-bit fields),
+    // so that a position costs two independent LDS reads.
+    uint32_t* before_wave = reinterpret_cast<uint32_t*>(bitmap + n * kWaves);
+    for (int j = tid; j < n; j += kThreads) {
+        const int c0 = __popcll(bitmap[j * kWaves]), c1 = __popcll(bitmap[j * kWaves + 1]);
+        const int c2 = __popcll(bitmap[j * kWaves + 2]), c3 = __popcll(bitmap[j * kWaves + 3]);
+        before_wave[j] = uint32_t(c0) | (uint32_t(c0 + c1) << 10) | (uint32_t(c0 + c1 + c2) << 20);
+        int32_t* at = j < p.R ? p.tab.rank_counts + int64_t(j) * p.tab.chunks_padded + chunk
+                              : p.tab.expert_counts + int64_t(chunk) * p.tab.experts_padded + (j - p.R);
+        store_word<kThrough>(at, c0 + c1 + c2 + c3);
+    }
+    const int pad = p.tab.chunks_padded - num_chunks;  // the padding columns of the rank table are cleared by the first workgroup
+    if (chunk == 0)
+        for (int i = tid; i < p.R * pad; i += kThreads)
+            store_word<kThrough>(p.tab.rank_counts + int64_t(i / pad) * p.tab.chunks_padded + num_chunks + i % pad, 0);
+    counts_stored();
+    __syncthreads();
+
+    const uint64_t below = lanes_below(lane);
+    const int wave_shift = wave > 0 ? 10 * (wave - 1) : 0;
+    auto rank_in_chunk = [&](int bucket) {
+        const int earlier = wave > 0 ? int((before_wave[bucket] >> wave_shift) & 0x3ffu) : 0;
+        return __popcll(bitmap[bucket * kWaves + wave] & below) + earlier;
+    };
+
+    if (active) {
+        if (p.pos != nullptr) {
+            // One word per (token, lane): low 16 bits = slot of the token inside its chunk for the lane's
+            // destination rank (master lanes only), high 16 bits = position of the lane inside its chunk for
+            // its expert; 0xffff = none.
+            uint32_t packed[KMAX];
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) {
+                uint32_t pr = 0xffffu, pe = 0xffffu;
+                if (e[k] >= 0) {
+                    bool master = true;
+#pragma unroll
+                    for (int j = 0; j < KMAX; ++j) {
+                        if (j > k && d[j] == d[k]) master = false;
+                        if (j != k && e[j] == e[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+                    }
+                    pe = uint32_t(rank_in_chunk(p.R + e[k]));
+                    if (master) pr = uint32_t(rank_in_chunk(d[k]));
+                }
+                packed[k] = pr | (pe << 16);
+            }
+            if (KMAX == 8 && p.K == 8) {
+                vec16* dst = reinterpret_cast<vec16*>(p.pos + int64_t(t) * 8);
+                const vec16 lo{packed[0], packed[1], packed[2], packed[3]}, hi{packed[4], packed[5], packed[6], packed[7]};
+                if constexpr (kThrough) {
+                    store16_agent(dst, lo);
+                    store16_agent(dst + 1, hi);
+                } else {
+                    dst[0] = lo;
+                    dst[1] = hi;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k)
+                    if (k < p.K) store_word<kThrough>(reinterpret_cast<int*>(p.pos) + int64_t(t) * p.K + k, int(packed[k]));
+            }
+        }
+        if (p.is_token_in_rank != nullptr) {
+            for (int r = 0; r < p.R; ++r)
+                p.is_token_in_rank[int64_t(t) * p.R + r] = uint8_t((bitmap[r * kWaves + wave] >> lane) & 1ull);
+        }
+    }
+    if (flags != 0) atomicOr(p.status, flags);
+
+}
+
+}  // namespace deep_ep_hip

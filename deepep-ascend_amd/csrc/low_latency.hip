@@ -7,8 +7,8 @@
 // With every logical source resident in local HBM the send/receive phases and the RDMA staging
 // buffers disappear; slots come from a scan, so the fill order is deterministic: source rank
 // ascending, then token ascending (the reference fills in arrival order).
-#include "common.cuh"
-#include "cast.cuh"
+#include "device_utils.h"
+#include "fp8_cast.h"
 #include "kernels.h"
 #include "../../include/deep_ep_hip.h"
 
@@ -368,7 +368,8 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
     const int tile = int(work - gu * unsigned(tiles));
     const int s = int(gu / unsigned(p.src_token_stride));
     const int t = int(gu - unsigned(s) * unsigned(p.src_token_stride));
-    const int n_s = p.num_tokens_per_src != nullptr ? p.num_tokens_per_src[s] : p.src_token_stride;
+    const int n_s = p.num_tokens_per_src != nullptr ? min(max(p.num_tokens_per_src[s], 0), p.src_token_stride)
+                                                    : p.src_token_stride;
     if (t >= n_s) return;
     const int src_rank = p.src_rank_begin + s;
     const int rows_per_expert = p.R * p.M;
@@ -506,8 +507,7 @@ hipError_t launch_fused_by_width(const LLDispatchParams& p, hipStream_t stream, 
     // Up to 4 x 1024 channels per wavefront: fatter wavefronts spend longer in the (serial) cast than the
     // extra wavefronts cost to launch.
     const int segs = (p.H + 1023) / 1024;
-    const char* env = getenv("DEEP_EP_HIP_LL_PAIRS");
-    const int forced = env != nullptr ? atoi(env) : 0;
+    const int forced = p.pairs;
     switch (forced == 1 || forced == 2 || forced == 4 ? forced : segs <= 1 ? 1 : segs <= 2 ? 2 : 4) {
         case 1: return launch_fused<1, kFusedThreads>(p, stream, lds);
         case 2: return launch_fused<2, kFusedThreads>(p, stream, lds);
@@ -520,10 +520,8 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
     // Decode-sized calls: one kernel, every workgroup derives the slots itself.
     const int64_t total_tokens = int64_t(p.S) * p.src_token_stride;
     const size_t fused_lds = size_t(p.E_l) * ((total_tokens + 63) / 64) * sizeof(uint64_t);
-    if (total_tokens <= 2048 && fused_lds <= 32 * 1024 && getenv("DEEP_EP_HIP_LL_TWO_KERNELS") == nullptr)
-    {
-        const char* env = getenv("DEEP_EP_HIP_LL_THREADS");
-        const int threads = env != nullptr ? atoi(env) : 512;
+    if (total_tokens <= 2048 && fused_lds <= 32 * 1024 && !p.two_kernels) {
+        const int threads = p.threads != 0 ? p.threads : 512;
         if (threads == 256) return launch_fused_by_width<256>(p, stream, fused_lds);
         if (threads == 1024) return launch_fused_by_width<1024>(p, stream, fused_lds);
         return launch_fused_by_width<512>(p, stream, fused_lds);
@@ -543,8 +541,7 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
 
 hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream) {
     if (p.S <= 0 || p.src_token_stride <= 0) return hipSuccess;
-    const char* env = getenv("DEEP_EP_HIP_LL_COMBINE_VECS");
-    int vecs = env != nullptr ? atoi(env) : 0;
+    int vecs = p.vecs;
     if (vecs != 1 && vecs != 2 && vecs != 4)
         vecs = (p.H * 2 <= 1024 || int64_t(p.S) * p.src_token_stride <= 4096) ? 1 : 4;   // decode sizes: many small wavefronts
     const int tiles = (p.H * 2 + vecs * 1024 - 1) / (vecs * 1024);

@@ -1,0 +1,225 @@
+// Turning per-chunk totals into the public outputs of the layout computation (per-rank and per-expert counts,
+// their prefix sums - the handle tensors of dispatch - and the host mailbox) and into the base tables the move
+// kernels place rows with (struct LayoutTables).  Publishes what the notify warps of
+// deep_ep/include/deep_ep/impls/dispatch.cuh:200-257 publish.
+#pragma once
+
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace deep_ep_hip {
+
+// In-place inclusive scan of a[0..n) in LDS by the whole workgroup.  tmp holds one int per wavefront.
+template <int kThreads>
+__device__ void block_inclusive_scan(int* a, int n, int* tmp) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int per = (n + kThreads - 1) / kThreads;
+    const int begin = min(tid * per, n), end = min(begin + per, n);
+    int s = 0;
+    for (int i = begin; i < end; ++i) s += a[i];
+    const int inc = wave_inclusive_sum(s);
+    if (lane == kWaveSize - 1) tmp[wave] = inc;
+    __syncthreads();
+    int run = inc - s;
+    for (int w = 0; w < wave; ++w) run += tmp[w];
+    for (int i = begin; i < end; ++i) {
+        run += a[i];
+        a[i] = run;
+    }
+    __syncthreads();
+}
+
+// LDS of the publishing workgroup: totals[R + E] | aligned[E] | aligned_incl[E] | one int per wavefront.
+struct PublishLds {
+    int* totals;         // rank part becomes its inclusive prefix sum in publish_ranks
+    int* aligned;
+    int* aligned_incl;
+    int* scan_tmp;
+};
+
+__device__ __forceinline__ PublishLds carve_publish_lds(int* lds, int R, int E) {
+    return PublishLds{lds, lds + R + E, lds + R + 2 * E, lds + R + 3 * E};
+}
+
+inline size_t publish_lds_bytes(int R, int E, int threads) {
+    return size_t(R + 3 * E + threads / kWaveSize) * sizeof(int);
+}
+
+// ---- rank part: tables are transposed, [rank][chunk] ----
+
+// totals[r] = sum of row r of rank_counts (padding columns are zero).  Ends with a barrier.
+template <int kThreads>
+__device__ void sum_rank_rows(const LayoutTables& t, int R, int* totals) {
+    for (int j = threadIdx.x; j < R; j += kThreads) {
+        const int32_t* row = t.rank_counts + int64_t(j) * t.chunks_padded;
+        int sum = 0;
+        for (int c0 = 0; c0 < t.chunks_padded; c0 += 32) {
+            vec16 v[8];                                   // all loads of a pass in flight together
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = load16(row + min(c0 + 4 * u, t.chunks_padded - 4));
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + 4 * u < t.chunks_padded) sum += int(v[u].x) + int(v[u].y) + int(v[u].z) + int(v[u].w);
+        }
+        totals[j] = sum;
+    }
+    __syncthreads();
+}
+
+// Per-rank outputs; afterwards s.totals[0..R) holds the inclusive prefix sum.  Every thread must call it.
+template <int kThreads>
+__device__ void publish_ranks(const PublishParams& q, const PublishLds& s) {
+    for (int r = threadIdx.x; r < q.R; r += kThreads) {
+        if (q.num_tokens_per_rank != nullptr) q.num_tokens_per_rank[r] = s.totals[r];
+        if (q.host_counts != nullptr) q.host_counts[r] = -s.totals[r] - 1;
+    }
+    __syncthreads();
+    block_inclusive_scan<kThreads>(s.totals, q.R, s.scan_tmp);
+    for (int r = threadIdx.x; r < q.R; r += kThreads)
+        if (q.psum_rank != nullptr) q.psum_rank[r] = s.totals[r];
+    if (threadIdx.x == 0 && q.totals_out != nullptr) q.totals_out[0] = s.totals[q.R - 1];
+}
+
+// rank_bases[r][c] = (rows of lower ranks) + sum of rank_counts[r][0..c): one thread per rank, 32 chunks per pass
+// with all of a pass's loads in flight together.  s.totals[0..R) must hold the inclusive prefix sum of the ranks.
+template <int kThreads>
+__device__ void write_rank_bases(const LayoutTables& t, int R, const PublishLds& s) {
+    for (int j = threadIdx.x; j < R; j += kThreads) {
+        const int32_t* src = t.rank_counts + int64_t(j) * t.chunks_padded;
+        int32_t* dst = t.rank_bases + int64_t(j) * t.chunks_padded;
+        int run = j > 0 ? s.totals[j - 1] : 0;
+        for (int c0 = 0; c0 < t.chunks_padded; c0 += 32) {
+            vec16 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = load16(src + min(c0 + 4 * u, t.chunks_padded - 4));
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (c0 + 4 * u < t.chunks_padded) {
+                    vec16 o;
+                    o.x = uint32_t(run); run += int(v[u].x);
+                    o.y = uint32_t(run); run += int(v[u].y);
+                    o.z = uint32_t(run); run += int(v[u].z);
+                    o.w = uint32_t(run); run += int(v[u].w);
+                    store16(dst + c0 + 4 * u, o);
+                }
+            }
+        }
+    }
+}
+
+// The whole rank part in one pass, for the publishing workgroup of a single-launch dispatch (the movers of the
+// compact layout wait for nothing else): rank_counts, written by other workgroups of the launch and therefore read
+// at agent scope, as one flat array of R * chunks_padded <= 4 * kThreads entries; rank_bases stored at agent scope.
+template <int kThreads>
+__device__ void publish_ranks_flat(const PublishParams& q, const LayoutTables& t, const PublishLds& s) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int flat = q.R * t.chunks_padded;            // a multiple of 4: a thread's entries share a row
+    const int begin = tid * 4;
+    int v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = begin < flat ? load_agent(t.rank_counts + begin + u) : 0;
+    const int sum = v[0] + v[1] + v[2] + v[3];
+    const int inc = wave_inclusive_sum(sum);
+    if (lane == kWaveSize - 1) s.scan_tmp[wave] = inc;
+    __syncthreads();
+    int run = inc - sum;
+    for (int w = 0; w < wave; ++w) run += s.scan_tmp[w];
+    if (begin < flat) {
+        store16_agent(t.rank_bases + begin, vec16{uint32_t(run), uint32_t(run + v[0]), uint32_t(run + v[0] + v[1]),
+                                                  uint32_t(run + v[0] + v[1] + v[2])});
+        if ((begin + 4) % t.chunks_padded == 0) s.totals[begin / t.chunks_padded] = run + sum;   // inclusive prefix of the rank
+    }
+    __syncthreads();
+    for (int r = tid; r < q.R; r += kThreads) {
+        const int total = s.totals[r] - (r > 0 ? s.totals[r - 1] : 0);
+        if (q.num_tokens_per_rank != nullptr) q.num_tokens_per_rank[r] = total;
+        if (q.host_counts != nullptr) q.host_counts[r] = -total - 1;
+        if (q.psum_rank != nullptr) q.psum_rank[r] = s.totals[r];
+    }
+    if (tid == 0 && q.totals_out != nullptr) q.totals_out[0] = s.totals[q.R - 1];
+}
+
+// ---- expert part: tables are [chunk][expert], so that thread e walks column e with coalesced accesses ----
+
+// totals[R + e] = sum over chunks of expert_counts[c][e].  Ends with a barrier.
+template <int kThreads>
+__device__ void sum_expert_columns(const LayoutTables& t, int R, int E, int num_chunks, int* totals) {
+    for (int e = threadIdx.x; e < E; e += kThreads) {
+        const int32_t* col = t.expert_counts + e;
+        int sum = 0;
+        for (int c0 = 0; c0 < num_chunks; c0 += 16) {
+            int v[16];                                    // all loads of a pass in flight together
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = col[int64_t(min(c0 + u, num_chunks - 1)) * t.experts_padded];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) sum += c0 + u < num_chunks ? v[u] : 0;
+        }
+        totals[R + e] = sum;
+    }
+    __syncthreads();
+}
+
+// Per-expert outputs; afterwards the region of expert j starts at s.aligned_incl[j] - s.aligned[j].
+template <int kThreads>
+__device__ void publish_experts(const PublishParams& q, const PublishLds& s) {
+    for (int j = threadIdx.x; j < q.E; j += kThreads) {
+        const int cnt = s.totals[q.R + j];
+        const int al = (cnt + q.A - 1) / q.A * q.A;
+        s.aligned[j] = al;
+        s.aligned_incl[j] = al;
+        if (q.num_tokens_per_expert != nullptr) q.num_tokens_per_expert[j] = cnt;
+        if (q.num_unaligned != nullptr) q.num_unaligned[j] = cnt;
+        if (q.cumulative_stats != nullptr) q.cumulative_stats[j] += cnt;
+        if (q.host_counts != nullptr) q.host_counts[q.R + j] = -al - 1;
+    }
+    __syncthreads();
+    block_inclusive_scan<kThreads>(s.aligned_incl, q.E, s.scan_tmp);
+    for (int j = threadIdx.x; j < q.E; j += kThreads) {
+        const int start = s.aligned_incl[j] - s.aligned[j];
+        if (q.expert_start != nullptr) q.expert_start[j] = start;
+        if (q.psum_expert != nullptr) q.psum_expert[j] = q.do_expand ? start + s.totals[q.R + j] : s.aligned_incl[j];
+    }
+    if (threadIdx.x == 0 && q.totals_out != nullptr) q.totals_out[1] = q.E > 0 ? s.aligned_incl[q.E - 1] : 0;
+    if (q.host_counts != nullptr) __threadfence_system();
+}
+
+// expert_bases[c][e] = start of expert e's region + sum of expert_counts[0..c)[e].  kThrough: stored at agent scope.
+template <int kThreads, bool kThrough>
+__device__ void write_expert_bases(const LayoutTables& t, int E, int num_chunks, const PublishLds& s) {
+    for (int e = threadIdx.x; e < E; e += kThreads) {
+        const int32_t* col = t.expert_counts + e;
+        int32_t* out = t.expert_bases + e;
+        int run = s.aligned_incl[e] - s.aligned[e];
+        for (int c0 = 0; c0 < num_chunks; c0 += 16) {
+            int v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = col[int64_t(min(c0 + u, num_chunks - 1)) * t.experts_padded];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                if (c0 + u < num_chunks) {
+                    store_word<kThrough>(out + int64_t(c0 + u) * t.experts_padded, run);
+                    run += v[u];
+                }
+            }
+        }
+    }
+}
+
+// Everything at once, for a workgroup that publishes after all counting is over (the stand-alone layout kernel):
+// totals, public outputs, and - when the caller has room for them - the base tables.
+template <int kThreads>
+__device__ void publish_layout(const PublishParams& q, const LayoutTables& t, int num_chunks, bool expert_bases, int* lds) {
+    const PublishLds s = carve_publish_lds(lds, q.R, q.E);
+    sum_rank_rows<kThreads>(t, q.R, s.totals);
+    sum_expert_columns<kThreads>(t, q.R, q.E, num_chunks, s.totals);
+    publish_ranks<kThreads>(q, s);
+    __syncthreads();
+    if (t.rank_bases != nullptr) write_rank_bases<kThreads>(t, q.R, s);
+    publish_experts<kThreads>(q, s);
+    if (t.expert_bases != nullptr && expert_bases) {
+        __syncthreads();
+        write_expert_bases<kThreads, false>(t, q.E, num_chunks, s);
+    }
+}
+
+}  // namespace deep_ep_hip

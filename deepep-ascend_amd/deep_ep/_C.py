@@ -163,7 +163,8 @@ class ElasticBuffer:
         ws = self._workspace
         status = int(ws[:4].view(torch.int32).item())
         if status != 0:
-            ws[:4].zero_()
+            # also the launch bookkeeping words that follow: a dispatch that gave up has left them mid-protocol
+            ws[:_abi.lib.deep_ep_hip_workspace_control_bytes()].zero_()
             reasons = []
             if status & _abi.STATUS_EXPERT_OUT_OF_RANGE:
                 reasons.append("topk_idx holds an expert id >= num_experts")
@@ -171,6 +172,8 @@ class ElasticBuffer:
                 reasons.append("a token selects the same expert twice")
             if status & _abi.STATUS_ROW_OVERFLOW:
                 reasons.append("a received row did not fit the output tensors")
+            if status & _abi.STATUS_LAYOUT_TIMEOUT:
+                reasons.append("a single-launch dispatch gave up waiting for its counting workgroups (outputs invalid)")
             raise RuntimeError(f"DeepEP HIP backend: {what}: " + "; ".join(reasons))
 
     def _prologue(self, previous_event, allocate_on_comm_stream: bool, async_with_compute_stream: bool,
@@ -327,6 +330,8 @@ class ElasticBuffer:
                 copied_topk_idx = torch.empty_like(topk_idx) if do_handle_copy else None
 
             args = _abi.DispatchArgs()
+
+            args.tuning = _abi.tuning
             args.payload = payload
             args.cached = int(cached_mode)
             args.do_expand = int(do_expand)
@@ -466,6 +471,7 @@ class ElasticBuffer:
             if previous_event_before_epilogue is not None:
                 run_stream.wait_event(previous_event_before_epilogue.event)
             args = _abi.CombineArgs()
+            args.tuning = _abi.tuning
             args.do_expand = int(use_expanded_layout)
             args.allow_multiple_reduction = int(self.allow_multiple_reduction)
             args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
@@ -599,6 +605,7 @@ class ElasticBuffer:
         per_expert_list: List[int] = []
         with torch.cuda.stream(run_stream):
             args = _abi.IntranodeDispatchArgs()
+            args.tuning = _abi.tuning
             args.payload, args.cached = payload, int(cached_mode)
             args.num_tokens, args.hidden = num_tokens, hidden
             args.num_topk, args.num_experts = num_topk, (num_experts if topk_idx is not None else 0)
@@ -711,6 +718,7 @@ class ElasticBuffer:
             if topk_weights is not None:
                 recv_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
             args = _abi.IntranodeCombineArgs()
+            args.tuning = _abi.tuning
             args.num_tokens, args.hidden, args.num_ranks, args.num_topk = num_tokens, hidden, R, num_topk
             args.x, args.num_x_rows = _abi.ptr(x), num_x_rows
             args.topk_weights = _abi.ptr(topk_weights)

@@ -3,6 +3,7 @@ reference's deep_ep/__init__.py:92-109).  The HIP kernel library is loaded at im
 the import fails (there is no fallback path)."""
 from . import _abi  # noqa: F401  (loads libdeep_ep_hip.so or raises)
 from ._C import Config, EventHandle, topk_idx_t
+from ._abi import tuning
 from .buffers.elastic import ElasticBuffer, EPHandle, LogicalGroup
 from .buffers.legacy import Buffer
 from .utils.event import EventOverlap

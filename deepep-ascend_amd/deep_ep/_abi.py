@@ -8,7 +8,7 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
 LIB_NAME = "libdeep_ep_hip.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 PHASE_LAYOUT = 1
 PHASE_MOVE = 2
@@ -19,10 +19,33 @@ PAYLOAD_CAST_FP8 = 2
 STATUS_EXPERT_OUT_OF_RANGE = 1
 STATUS_DUPLICATE_EXPERT = 2
 STATUS_ROW_OVERFLOW = 4
+STATUS_LAYOUT_TIMEOUT = 8
 
 MAX_TOPK = 32
 MAX_EXPERTS = 1024
 MAX_RANKS = 512
+
+
+class Tuning(Structure):
+    """Launch-shape knobs carried by every argument block (all zero = the library's own choice).  The C library reads
+    no environment variables; this package seeds its process-wide default (`deep_ep.tuning`) from
+    DEEP_EP_HIP_<FIELD NAME IN CAPITALS> once at import."""
+    _fields_ = [
+        ("dispatch_launches", c_int32), ("cast_pairs", c_int32), ("copy_vecs", c_int32), ("plain_loads", c_int32),
+        ("xcd_remap", c_int32), ("combine_vecs", c_int32), ("ll_pairs", c_int32), ("ll_threads", c_int32),
+        ("ll_two_kernels", c_int32), ("ll_combine_vecs", c_int32), ("reserved", c_int32 * 6),
+    ]
+
+    @classmethod
+    def from_env(cls) -> "Tuning":
+        t = cls()
+        for name, _ in cls._fields_:
+            if name != "reserved":
+                setattr(t, name, int(os.environ.get("DEEP_EP_HIP_" + name.upper(), "0")))
+        return t
+
+
+tuning = Tuning.from_env()
 
 
 class LayoutArgs(Structure):
@@ -67,6 +90,7 @@ class DispatchArgs(Structure):
         ("expanded_capacity", c_int64),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("tuning", Tuning),
     ]
 
 
@@ -90,6 +114,7 @@ class CombineArgs(Structure):
         ("combined_topk_weights", c_void_p),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("tuning", Tuning),
     ]
 
 
@@ -126,6 +151,7 @@ class IntranodeDispatchArgs(Structure):
         ("recv_capacity", c_int64),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("tuning", Tuning),
     ]
 
 
@@ -143,6 +169,7 @@ class IntranodeCombineArgs(Structure):
         ("combined_topk_weights", c_void_p),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("tuning", Tuning),
     ]
 
 
@@ -169,6 +196,7 @@ class LLDispatchArgs(Structure):
         ("lane_rows", c_void_p),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("tuning", Tuning),
     ]
 
 
@@ -189,6 +217,7 @@ class LLCombineArgs(Structure):
         ("combined_x", c_void_p),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("tuning", Tuning),
     ]
 
 
@@ -207,6 +236,7 @@ EXPORTS = {
     "deep_ep_hip_last_error": (c_char_p, []),
     "deep_ep_hip_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "deep_ep_hip_workspace_status_offset": (c_size_t, []),
+    "deep_ep_hip_workspace_control_bytes": (c_size_t, []),
     "deep_ep_hip_launch_layout": (c_int, [POINTER(LayoutArgs), c_void_p]),
     "deep_ep_hip_launch_dispatch": (c_int, [POINTER(DispatchArgs), c_void_p]),
     "deep_ep_hip_launch_combine": (c_int, [POINTER(CombineArgs), c_void_p]),

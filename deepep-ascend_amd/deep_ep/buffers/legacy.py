@@ -248,6 +248,7 @@ class Buffer:
             if T > 0:
                 ws = self._workspace(_abi.lib.deep_ep_hip_ll_workspace_bytes(S, T, K, E_l))
                 args = _abi.LLDispatchArgs()
+                args.tuning = _abi.tuning
                 args.use_fp8, args.round_scale, args.use_ue8m0 = int(use_fp8), int(round_scale), int(use_ue8m0)
                 args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
                 args.num_tokens_per_src = 0
@@ -333,6 +334,7 @@ class Buffer:
             if T > 0:
                 ws = self._workspace(4096)
                 args = _abi.LLCombineArgs()
+                args.tuning = _abi.tuning
                 args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
                 args.num_tokens_per_src = 0
                 args.hidden, args.num_topk, args.num_experts = H, K, num_experts

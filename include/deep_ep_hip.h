@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define DEEP_EP_HIP_ABI_VERSION 2
+#define DEEP_EP_HIP_ABI_VERSION 3
 
 #define DEEP_EP_HIP_OK 0
 #define DEEP_EP_HIP_ERR_INVALID_ARGUMENT (-1)
@@ -59,15 +59,42 @@ extern "C" {
 #define DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE 1  /* topk_idx >= num_experts (entry ignored) */
 #define DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT 2     /* one token names an expert twice */
 #define DEEP_EP_HIP_STATUS_ROW_OVERFLOW 4         /* a row fell outside the caller's capacity (row dropped) */
+#define DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT 8       /* a single-launch dispatch gave up waiting for its own counting
+                                                     workgroups (outputs of that call are invalid) */
 
 int deep_ep_hip_abi_version(void);
 const char* deep_ep_hip_last_error(void);
+
+/* Launch-shape knobs, last member of every argument block.  All zero = the library's own choice (what the
+ * measurements behind it say is best); nothing here changes results.  The library reads no environment
+ * variables. */
+typedef struct {
+    int32_t dispatch_launches; /* dispatch with both phases in one call: 0 = a single launch (counting workgroups at
+                                  the front of the move kernel) where the shape allows it (num_topk <= 8, num_ranks +
+                                  num_experts <= 512, num_ranks * ceil(num_tokens / 256) <= 1024) and it pays (at most
+                                  16384 mover workgroups); 1 = a single launch wherever the shape allows it; 2 = always
+                                  layout kernel + move kernel */
+    int32_t cast_pairs;        /* fused FP8 cast: 1024-channel segments per wavefront (1, 2, 4, 7, 8) */
+    int32_t copy_vecs;         /* pass-through payloads: KB of row per wavefront (1, 2, 4, 7, 8) */
+    int32_t plain_loads;       /* 1: payload loads allocate in the caches (for inputs known to be cache resident) */
+    int32_t xcd_remap;         /* 1: consecutive workgroups of a dispatch share an XCD */
+    int32_t combine_vecs;      /* combine: KB of row per wavefront (1, 2, 4) */
+    int32_t ll_pairs;          /* low-latency dispatch: 1024-channel segments per wavefront (1, 2, 4) */
+    int32_t ll_threads;        /* low-latency dispatch, single-kernel path: workgroup size (256, 512, 1024) */
+    int32_t ll_two_kernels;    /* 1: low-latency dispatch always as count kernel + move kernel */
+    int32_t ll_combine_vecs;   /* low-latency combine: KB of row per wavefront (1, 2, 4) */
+    int32_t reserved[6];
+} deep_ep_hip_tuning;
 
 /* Bytes of workspace needed for dispatches of up to num_max_tokens tokens.  The workspace must
  * be zero-filled once before its first use; the kernels leave it ready for the next call. */
 size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_experts, int num_ranks);
 /* Byte offset, inside the workspace, of the int32 status word. */
 size_t deep_ep_hip_workspace_status_offset(void);
+/* Leading bytes of the workspace that hold the status word and the launch bookkeeping the kernels expect to find
+ * zero at the start of a launch (and leave zero at its end).  After DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT, zero these
+ * bytes before the workspace is used again. */
+size_t deep_ep_hip_workspace_control_bytes(void);
 
 /* ------------------------------------------------------------------------------------------
  * Dispatch layout (V1 `Buffer.get_dispatch_layout`): counts only.
@@ -141,6 +168,7 @@ typedef struct {
 
     void* workspace;
     uint64_t workspace_bytes;
+    deep_ep_hip_tuning tuning;
 } deep_ep_hip_dispatch_args;
 
 int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* args, void* stream);
@@ -168,6 +196,7 @@ typedef struct {
     float* combined_topk_weights;       /* [num_tokens, num_topk] out or NULL */
     void* workspace;
     uint64_t workspace_bytes;
+    deep_ep_hip_tuning tuning;
 } deep_ep_hip_combine_args;
 
 int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* args, void* stream);
@@ -228,6 +257,7 @@ typedef struct {
     void* workspace;                /* deep_ep_hip_workspace_bytes(num_tokens, max(num_topk, num_ranks),
                                        max(num_experts, num_ranks), num_ranks) bytes */
     uint64_t workspace_bytes;
+    deep_ep_hip_tuning tuning;
 } deep_ep_hip_intranode_dispatch_args;
 
 int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_args* args, void* stream);
@@ -247,6 +277,7 @@ typedef struct {
     float* combined_topk_weights;   /* [num_tokens, num_topk] out or NULL */
     void* workspace;                /* >= 256 bytes (status word) */
     uint64_t workspace_bytes;
+    deep_ep_hip_tuning tuning;
 } deep_ep_hip_intranode_combine_args;
 
 int deep_ep_hip_launch_intranode_combine(const deep_ep_hip_intranode_combine_args* args, void* stream);
@@ -286,6 +317,7 @@ typedef struct {
                                            packed_recv_src_info */
     void* workspace;
     uint64_t workspace_bytes;
+    deep_ep_hip_tuning tuning;
 } deep_ep_hip_ll_dispatch_args;
 
 /* Bytes of (zero-initialised, reusable) workspace a low-latency dispatch of this shape needs. */
@@ -309,6 +341,7 @@ typedef struct {
                                            source's token count are left untouched */
     void* workspace;
     uint64_t workspace_bytes;
+    deep_ep_hip_tuning tuning;
 } deep_ep_hip_ll_combine_args;
 
 int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* args, void* stream);

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(_abi.lib, name), f"{name} is declared in the header but not exported"
     assert sorted(_abi.EXPORTS) == names, "ctypes binding table and header disagree"
-    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 2
+    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 3
 
 
 def test_ctypes_structs_match_the_header_layout():
@@ -39,7 +39,8 @@ def test_ctypes_structs_match_the_header_layout():
                "deep_ep_hip_combine_args": _abi.CombineArgs,
                "deep_ep_hip_intranode_dispatch_args": _abi.IntranodeDispatchArgs,
                "deep_ep_hip_intranode_combine_args": _abi.IntranodeCombineArgs, "deep_ep_hip_ll_dispatch_args": _abi.LLDispatchArgs,
-               "deep_ep_hip_ll_combine_args": _abi.LLCombineArgs, "deep_ep_hip_cast_args": _abi.CastArgs}
+               "deep_ep_hip_ll_combine_args": _abi.LLCombineArgs, "deep_ep_hip_cast_args": _abi.CastArgs,
+               "deep_ep_hip_tuning": _abi.Tuning}
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {"]
     for cname, cls in structs.items():
         lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
@@ -63,7 +64,8 @@ def test_header_limits_match_python_constants():
     for name, value in (("DEEP_EP_HIP_MAX_TOPK", _abi.MAX_TOPK), ("DEEP_EP_HIP_MAX_EXPERTS", _abi.MAX_EXPERTS),
                         ("DEEP_EP_HIP_MAX_RANKS", _abi.MAX_RANKS), ("DEEP_EP_HIP_PHASE_LAYOUT", _abi.PHASE_LAYOUT),
                         ("DEEP_EP_HIP_PHASE_MOVE", _abi.PHASE_MOVE), ("DEEP_EP_HIP_PAYLOAD_CAST_FP8", _abi.PAYLOAD_CAST_FP8),
-                        ("DEEP_EP_HIP_STATUS_ROW_OVERFLOW", _abi.STATUS_ROW_OVERFLOW)):
+                        ("DEEP_EP_HIP_STATUS_ROW_OVERFLOW", _abi.STATUS_ROW_OVERFLOW),
+                        ("DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT", _abi.STATUS_LAYOUT_TIMEOUT)):
         assert re.search(rf"#define {name} {value}\b", text), name
 
 

@@ -1,7 +1,6 @@
-"""Every tuning knob (environment variable read at launch time) selects another instantiation or code path of the
-same kernels; the results must stay bit-identical to the oracle."""
-import os
-
+"""Every tuning knob (a field of the `tuning` member of the argument blocks, set here through the package-wide
+default `deep_ep.tuning`) selects another instantiation or code path of the same kernels; the results must stay
+bit-identical to the oracle."""
 import pytest
 import torch
 
@@ -12,22 +11,21 @@ from test_gpu_parity import _buffer, assert_equal
 pytestmark = pytest.mark.gpu
 
 KNOBS = [
-    ("DEEP_EP_HIP_XCD_REMAP", "1"), ("DEEP_EP_HIP_PLAIN_LOADS", "1"), ("DEEP_EP_HIP_NO_LIGHT_LAYOUT", "1"),
-    ("DEEP_EP_HIP_CAST_PAIRS", "1"), ("DEEP_EP_HIP_CAST_PAIRS", "4"), ("DEEP_EP_HIP_CAST_PAIRS", "7"),
-    ("DEEP_EP_HIP_CAST_PAIRS", "8"), ("DEEP_EP_HIP_COPY_VECS", "1"), ("DEEP_EP_HIP_COPY_VECS", "2"),
-    ("DEEP_EP_HIP_COPY_VECS", "7"), ("DEEP_EP_HIP_COPY_VECS", "8"), ("DEEP_EP_HIP_COMBINE_VECS", "1"),
-    ("DEEP_EP_HIP_COMBINE_VECS", "4"),
+    ("xcd_remap", 1), ("plain_loads", 1), ("dispatch_launches", 1), ("dispatch_launches", 2),
+    ("cast_pairs", 1), ("cast_pairs", 4), ("cast_pairs", 7), ("cast_pairs", 8), ("copy_vecs", 1), ("copy_vecs", 2),
+    ("copy_vecs", 7), ("copy_vecs", 8), ("combine_vecs", 1), ("combine_vecs", 4),
 ]
 
 
 @pytest.fixture
 def knob(request, monkeypatch):
+    import deep_ep
     name, value = request.param
-    monkeypatch.setenv(name, value)
+    monkeypatch.setattr(deep_ep.tuning, name, value)
     return name, value
 
 
-@pytest.mark.parametrize("knob", KNOBS, indirect=True, ids=[f"{n[12:]}={v}" for n, v in KNOBS])
+@pytest.mark.parametrize("knob", KNOBS, indirect=True, ids=[f"{n}={v}" for n, v in KNOBS])
 def test_dispatch_and_combine_under_knob(knob):
     case = rc.small("knobs", 700, 2304, 64, 8, 6, seed=40, masked_ratio=0.1)        # 2304 = 2.25 x 1024 channels: ragged tiles
     buf = _buffer(case)
@@ -58,12 +56,11 @@ def test_dispatch_and_combine_under_knob(knob):
     buf.check_device_status()
 
 
-LL_KNOBS = [("DEEP_EP_HIP_LL_THREADS", "256"), ("DEEP_EP_HIP_LL_THREADS", "1024"), ("DEEP_EP_HIP_LL_PAIRS", "1"),
-            ("DEEP_EP_HIP_LL_PAIRS", "2"), ("DEEP_EP_HIP_LL_TWO_KERNELS", "1"), ("DEEP_EP_HIP_LL_COMBINE_VECS", "2"),
-            ("DEEP_EP_HIP_LL_COMBINE_VECS", "4")]
+LL_KNOBS = [("ll_threads", 256), ("ll_threads", 1024), ("ll_pairs", 1), ("ll_pairs", 2), ("ll_two_kernels", 1),
+            ("ll_combine_vecs", 2), ("ll_combine_vecs", 4)]
 
 
-@pytest.mark.parametrize("knob", LL_KNOBS, indirect=True, ids=[f"{n[12:]}={v}" for n, v in LL_KNOBS])
+@pytest.mark.parametrize("knob", LL_KNOBS, indirect=True, ids=[f"{n}={v}" for n, v in LL_KNOBS])
 def test_low_latency_under_knob(knob):
     import deep_ep
     R, T, H, E, K, M = 4, 100, 2560, 32, 5, 128

@@ -1,0 +1,102 @@
+"""The single-launch dispatch (layout and move in one call without a host wait: counting workgroups ride at the front
+of the move kernel and hand the layout to the movers through gates in the workspace) against the CPU oracle, and
+the state it must leave behind: every launch finds and leaves the bookkeeping words of the workspace at zero."""
+import pytest
+import torch
+
+import routing_cases as rc
+import routing_oracle as oracle
+from test_gpu_parity import CASES, _buffer, assert_equal
+
+pytestmark = pytest.mark.gpu
+
+# shapes the single launch covers (num_topk <= 8, num_ranks + num_experts <= 512, num_ranks * chunks <= 1024)
+FUSED = ["C1", "C2", "tiny_masked", "one_token", "k1_e_eq_r", "ragged_chunks", "r1_world", "many_chunks"]
+
+
+def _control_words(buf):
+    from deep_ep import _abi
+    n = _abi.lib.deep_ep_hip_workspace_control_bytes()
+    words = buf.runtime._workspace[:n].view(torch.int32).cpu().clone()
+    words[2:4] = 0          # the two row totals a dispatch leaves for the kernels that follow it
+    return words
+
+
+def _check(buf, case, do_expand, payload, alignment=1):
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    if payload == "bf16":
+        src, kw = case.x, {}
+    else:
+        src, kw = oracle.per_token_cast_to_fp8(case.x), {"cast_to_fp8": True}
+    ref = oracle.dispatch(src, case.topk_idx, case.topk_weights, case.E, case.R, buf.rank_idx, case.M, do_expand=do_expand,
+                          expert_alignment=alignment)
+    recv, ridx, rw, handle, _ = buf.dispatch(x, idx, w, num_experts=case.E, do_cpu_sync=False, do_expand=do_expand,
+                                             expert_alignment=alignment, **kw)
+    n = ref.num_expanded_tokens if do_expand else ref.num_recv_tokens
+    valid = ref.expanded_row_is_valid if do_expand else torch.ones(n, dtype=torch.bool)
+    if payload == "bf16":
+        assert_equal(recv[:n].cpu()[valid], ref.recv_x[valid], "recv_x")
+    else:
+        assert_equal(recv[0][:n].cpu()[valid], ref.recv_x[valid], "recv_x (fp8)")
+        assert_equal(recv[1][:n].cpu()[valid], ref.recv_sf[valid], "recv_sf")
+    if not do_expand:
+        assert_equal(ridx[:n], ref.recv_topk_idx, "recv_topk_idx")
+        assert_equal(rw[:n], ref.recv_topk_weights, "recv_topk_weights")
+    else:
+        assert_equal(rw[:n].cpu()[valid], ref.recv_topk_weights[valid], "recv_topk_weights")
+    assert_equal(handle.psum_num_recv_tokens_per_scaleup_rank, ref.psum_num_recv_tokens_per_scaleup_rank, "psum_rank")
+    assert_equal(handle.psum_num_recv_tokens_per_expert, ref.psum_num_recv_tokens_per_expert, "psum_expert")
+    assert_equal(handle.num_unaligned_recv_tokens_per_expert, ref.num_unaligned_recv_tokens_per_expert, "unaligned")
+    assert_equal(handle.dst_buffer_slot_idx, ref.dst_buffer_slot_idx, "dst_buffer_slot_idx")
+    assert_equal(handle.recv_src_metadata[:ref.num_recv_tokens], ref.recv_src_metadata, "recv_src_metadata")
+    return handle, ref
+
+
+@pytest.mark.parametrize("name", FUSED)
+@pytest.mark.parametrize("do_expand", [False, True], ids=["compact", "expanded"])
+@pytest.mark.parametrize("payload", ["bf16", "cast_fp8"])
+def test_single_launch_matches_the_oracle(name, do_expand, payload, monkeypatch):
+    import deep_ep
+    monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", 1)
+    case = CASES[name]()
+    if payload == "cast_fp8" and case.H % 128 != 0:
+        pytest.skip("the fused cast needs hidden % 128 == 0")
+    buf = _buffer(case, rank=case.R - 1)
+    _check(buf, case, do_expand, payload, alignment=4 if do_expand else 1)
+    buf.check_device_status()
+    assert int(_control_words(buf).abs().sum()) == 0, "the launch did not leave its bookkeeping words at zero"
+
+
+def test_launches_of_changing_shape_share_one_workspace(monkeypatch):
+    """Gates, flags and tables are reused by launches of different token counts, layouts and launch modes; each must
+    find them clean."""
+    import deep_ep
+    E, R, K, H = 32, 4, 6, 512
+    buf = deep_ep.ElasticBuffer(deep_ep.LogicalGroup(1, R), num_max_tokens_per_rank=4096, hidden=H, num_topk=K)
+    shapes = [1, 2, 255, 256, 257, 700, 4096, 3, 1025]
+    for round_ in range(2):
+        for i, T in enumerate(shapes):
+            case = rc.small(f"seq{T}", T, H, E, R, K, seed=100 + T, masked_ratio=0.1)
+            case.M = 4096
+            monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", (1, 2, 0)[(i + round_) % 3])
+            handle, ref = _check(buf, case, do_expand=bool((i + round_) % 2), payload=("bf16", "cast_fp8")[i % 2])
+            assert int(_control_words(buf).abs().sum()) == 0, f"bookkeeping words not zero after T={T}"
+    buf.check_device_status()
+
+
+def test_many_back_to_back_launches_without_host_sync(monkeypatch):
+    """50 single-launch dispatches queued without a host wait in between: the gates of launch n must have wrapped to
+    zero before launch n + 1 reads them (stream order), whatever the number of movers per gate."""
+    import deep_ep
+    monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", 1)
+    case = rc.small("b2b", 1500, 1024, 64, 8, 8, seed=77, masked_ratio=0.05)
+    buf = _buffer(case)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    ref = oracle.dispatch(case.x, case.topk_idx, case.topk_weights, case.E, case.R, 0, case.M)
+    outs = [buf.dispatch(x, idx, w, num_experts=case.E, do_cpu_sync=False) for _ in range(50)]
+    torch.cuda.synchronize()
+    for recv, ridx, rw, handle, _ in outs[::7] + [outs[-1]]:
+        assert_equal(recv[:ref.num_recv_tokens], ref.recv_x, "recv_x")
+        assert_equal(handle.dst_buffer_slot_idx, ref.dst_buffer_slot_idx, "dst_buffer_slot_idx")
+    buf.check_device_status()
+    assert int(_control_words(buf).abs().sum()) == 0

@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/deep_ep_hip.h"
 #include "device_utils.h"
@@ -124,55 +125,45 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
 
 using namespace deep_ep_hip;
 
-extern "C" {
+// ---- the workspace of deep_ep_hip_launch_dispatch_static: device memory that exists without any allocation ----
+constexpr size_t kStaticWorkspaceBytes = DEEP_EP_HIP_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
 
-int deep_ep_hip_abi_version(void) { return DEEP_EP_HIP_ABI_VERSION; }
+namespace {
 
-const char* deep_ep_hip_last_error(void) { return g_last_error; }
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];          // address of `scratch` on each device (every GPU holds its own copy)
+bool g_scratch_ready[kMaxDevices];
+std::mutex g_scratch_mutex;
 
-size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_experts, int num_ranks) {
-    if (num_max_tokens < 0 || num_topk < 1 || num_experts < 1 || num_ranks < 1) return 0;
-    return make_workspace_layout(num_max_tokens, num_topk, num_experts, num_ranks).total_bytes;
+__global__ void clear_words_kernel(uint32_t* words, size_t n) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) words[i] = 0u;
 }
 
-size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
-
-size_t deep_ep_hip_workspace_control_bytes(void) { return make_workspace_layout(1, 1, 1, 1).expert_start; }
-
-int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
-    REQUIRE(a != nullptr, "args is NULL");
-    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
-    REQUIRE(a->num_tokens == 0 || a->topk_idx != nullptr, "topk_idx is NULL");
-    REQUIRE(a->num_tokens_per_rank != nullptr && a->num_tokens_per_expert != nullptr, "count outputs are NULL");
-    REQUIRE(a->workspace != nullptr, "workspace is NULL");
-    const WorkspaceLayout w = make_workspace_layout(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks);
-    if (a->workspace_bytes < w.total_bytes)
-        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
-                    (unsigned long long)a->workspace_bytes, w.total_bytes);
-    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
-    LayoutParams p{};
-    p.topk_idx = a->topk_idx;
-    p.T = a->num_tokens; p.K = a->num_topk; p.E = a->num_experts; p.R = a->num_ranks;
-    p.E_l = p.E / p.R;
-    p.is_token_in_rank = a->is_token_in_rank;
-    p.pub.R = p.R; p.pub.E = p.E; p.pub.A = 1;
-    p.pub.num_tokens_per_rank = a->num_tokens_per_rank;
-    p.pub.num_tokens_per_expert = a->num_tokens_per_expert;
-    p.pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
-    p.pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
-    p.status = reinterpret_cast<int32_t*>(ws + w.status);
-    p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
-    p.tab = carve_tables(ws, w, p.T, p.E);
-    p.tab.rank_bases = nullptr;       // a layout-only call publishes counts, not row bases
-    p.tab.expert_bases = nullptr;
-    hipError_t err = launch_layout_kernel(p, static_cast<hipStream_t>(stream));
-    if (err != hipSuccess) return hip_fail(err, "layout launch");
+// Device address of `scratch` on the current device.  First use on a device resolves the address and clears the
+// bookkeeping words with a small kernel on `stream` (no memset: the call may be under graph capture).
+int static_workspace(hipStream_t stream, void** out) {
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return hip_fail(err, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(DEEP_EP_HIP_ERR_UNSUPPORTED, "device index %d is beyond %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ready[dev]) {
+        void* ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || ptr == nullptr) return hip_fail(err, "hipGetSymbolAddress(scratch)");
+        const size_t control_words = make_workspace_layout(1, 1, 1, 1).expert_start / 4;
+        hipLaunchKernelGGL(clear_words_kernel, dim3(16), dim3(256), 0, stream, static_cast<uint32_t*>(ptr), control_words);
+        err = hipGetLastError();
+        if (err != hipSuccess) return hip_fail(err, "clearing the static workspace");
+        g_scratch_ptr[dev] = ptr;
+        g_scratch_ready[dev] = true;
+    }
+    *out = g_scratch_ptr[dev];
     return DEEP_EP_HIP_OK;
 }
 
-int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
-    REQUIRE(a != nullptr, "args is NULL");
+int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace, uint64_t workspace_bytes, hipStream_t stream) {
     if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
     const int T = a->num_tokens, H = a->hidden, K = a->num_topk, E = a->num_experts, R = a->num_ranks;
     const bool do_layout = (a->phases & DEEP_EP_HIP_PHASE_LAYOUT) != 0;
@@ -186,14 +177,14 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
     REQUIRE(a->expert_alignment >= 1, "expert_alignment must be >= 1");
     REQUIRE(!a->do_zero_padding || a->do_expand, "do_zero_padding requires do_expand");
     REQUIRE(T == 0 || a->topk_idx != nullptr, "topk_idx is NULL");
-    REQUIRE(a->workspace != nullptr, "workspace is NULL");
+    REQUIRE(workspace != nullptr, "workspace is NULL");
     REQUIRE(a->psum_num_recv_tokens_per_rank != nullptr && a->psum_num_recv_tokens_per_expert != nullptr &&
             a->num_unaligned_recv_tokens_per_expert != nullptr, "handle prefix-sum tensors are NULL");
     const WorkspaceLayout w = make_workspace_layout(T, K, E, R);
-    if (a->workspace_bytes < w.total_bytes)
+    if (workspace_bytes < w.total_bytes)
         return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
-                    (unsigned long long)a->workspace_bytes, w.total_bytes);
-    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+                    (unsigned long long)workspace_bytes, w.total_bytes);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
     int32_t* status = reinterpret_cast<int32_t*>(ws + w.status);
 
     int elem_in = 2, elem_out = 2;
@@ -314,6 +305,74 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
         }
     }
     return DEEP_EP_HIP_OK;
+}
+
+}  // namespace
+
+
+extern "C" {
+
+int deep_ep_hip_abi_version(void) { return DEEP_EP_HIP_ABI_VERSION; }
+
+const char* deep_ep_hip_last_error(void) { return g_last_error; }
+
+size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_experts, int num_ranks) {
+    if (num_max_tokens < 0 || num_topk < 1 || num_experts < 1 || num_ranks < 1) return 0;
+    return make_workspace_layout(num_max_tokens, num_topk, num_experts, num_ranks).total_bytes;
+}
+
+size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
+
+size_t deep_ep_hip_workspace_control_bytes(void) { return make_workspace_layout(1, 1, 1, 1).expert_start; }
+
+int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
+    REQUIRE(a->num_tokens == 0 || a->topk_idx != nullptr, "topk_idx is NULL");
+    REQUIRE(a->num_tokens_per_rank != nullptr && a->num_tokens_per_expert != nullptr, "count outputs are NULL");
+    REQUIRE(a->workspace != nullptr, "workspace is NULL");
+    const WorkspaceLayout w = make_workspace_layout(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks);
+    if (a->workspace_bytes < w.total_bytes)
+        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed",
+                    (unsigned long long)a->workspace_bytes, w.total_bytes);
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    LayoutParams p{};
+    p.topk_idx = a->topk_idx;
+    p.T = a->num_tokens; p.K = a->num_topk; p.E = a->num_experts; p.R = a->num_ranks;
+    p.E_l = p.E / p.R;
+    p.is_token_in_rank = a->is_token_in_rank;
+    p.pub.R = p.R; p.pub.E = p.E; p.pub.A = 1;
+    p.pub.num_tokens_per_rank = a->num_tokens_per_rank;
+    p.pub.num_tokens_per_expert = a->num_tokens_per_expert;
+    p.pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
+    p.pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
+    p.status = reinterpret_cast<int32_t*>(ws + w.status);
+    p.done_counter = reinterpret_cast<uint32_t*>(ws + w.done_counter);
+    p.tab = carve_tables(ws, w, p.T, p.E);
+    p.tab.rank_bases = nullptr;       // a layout-only call publishes counts, not row bases
+    p.tab.expert_bases = nullptr;
+    hipError_t err = launch_layout_kernel(p, static_cast<hipStream_t>(stream));
+    if (err != hipSuccess) return hip_fail(err, "layout launch");
+    return DEEP_EP_HIP_OK;
+}
+
+int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream) {
+    REQUIRE(a != nullptr, "args is NULL");
+    return dispatch_with_workspace(a, a->workspace, a->workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int deep_ep_hip_launch_dispatch_static(const deep_ep_hip_dispatch_args* a, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    REQUIRE(a != nullptr, "args is NULL");
+    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
+    const size_t need = make_workspace_layout(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks).total_bytes;
+    if (need > kStaticWorkspaceBytes)
+        return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL,
+                    "this shape needs %zu bytes of workspace, the built-in one has %zu: pass a workspace of your own to "
+                    "deep_ep_hip_launch_dispatch", need, kStaticWorkspaceBytes);
+    void* ws = nullptr;
+    if (int rc = static_workspace(stream, &ws)) return rc;
+    return dispatch_with_workspace(a, ws, kStaticWorkspaceBytes, stream);
 }
 
 int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) {

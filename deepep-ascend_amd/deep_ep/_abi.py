@@ -24,6 +24,7 @@ STATUS_LAYOUT_TIMEOUT = 8
 MAX_TOPK = 32
 MAX_EXPERTS = 1024
 MAX_RANKS = 512
+STATIC_WORKSPACE_BYTES = 1 << 20
 
 
 class Tuning(Structure):
@@ -239,6 +240,7 @@ EXPORTS = {
     "deep_ep_hip_workspace_control_bytes": (c_size_t, []),
     "deep_ep_hip_launch_layout": (c_int, [POINTER(LayoutArgs), c_void_p]),
     "deep_ep_hip_launch_dispatch": (c_int, [POINTER(DispatchArgs), c_void_p]),
+    "deep_ep_hip_launch_dispatch_static": (c_int, [POINTER(DispatchArgs), c_void_p]),
     "deep_ep_hip_launch_combine": (c_int, [POINTER(CombineArgs), c_void_p]),
     "deep_ep_hip_launch_intranode_dispatch": (c_int, [POINTER(IntranodeDispatchArgs), c_void_p]),
     "deep_ep_hip_launch_intranode_combine": (c_int, [POINTER(IntranodeCombineArgs), c_void_p]),

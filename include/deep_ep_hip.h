@@ -173,6 +173,18 @@ typedef struct {
 
 int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* args, void* stream);
 
+/* The same dispatch for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  args->workspace and
+ * args->workspace_bytes are ignored: the workspace is a device-resident array built into the library,
+ * DEEP_EP_HIP_STATIC_WORKSPACE_BYTES long, of which every GPU the library runs on holds one copy until the process
+ * ends.  Shapes with deep_ep_hip_workspace_bytes(num_tokens, num_topk, num_experts, num_ranks) beyond that are
+ * rejected with DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL.  The call allocates and frees nothing; the caller still passes
+ * every input and output.  The device the stream belongs to must be current.  All calls on one GPU share that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race, and the two phases of a split call must
+ * both come through this entry point.  Status bits raised by these calls are kept in the array's own status word. */
+#define DEEP_EP_HIP_STATIC_WORKSPACE_BYTES (1u << 20)
+int deep_ep_hip_launch_dispatch_static(const deep_ep_hip_dispatch_args* args, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Combine (V2 `ElasticBuffer.combine`): per origin token, fp32 sum of bias_0, bias_1 and the
  * rows that came back, in ascending master-lane order, one round-to-nearest-even BF16 store.

@@ -1,0 +1,626 @@
+// Host side of dispatch / combine for the HIP backend: the class the `deep_ep._C` extension registers as
+// `ElasticBuffer` (the role of csrc/elastic/buffer.hpp:83-1345 on CUDA and csrc/backends/ascend/elastic_buffer.hpp on
+// Ascend).  It checks arguments, allocates the outputs, sequences the launches on the right stream and returns the
+// reference's tuples.  Torch types stop here: below this class everything goes through the C ABI of
+// include/deep_ep_hip.h (plain pointers, sizes and a stream).
+//
+// One GPU, logical ranks: `num_ranks` only decides which bucket (destination rank) an expert belongs to; every
+// bucket lives in this GPU's HBM.  One call moves the tokens of the logical source rank `rank_idx`.
+#pragma once
+
+#include <c10/hip/HIPFunctions.h>
+#include <pybind11/pybind11.h>
+#include <torch/types.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <optional>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "../../../include/deep_ep_hip.h"
+#include "event.hpp"
+
+namespace deep_ep::hip {
+
+// Host checks raise what the reference's EP_HOST_ASSERT raises: an exception Python sees as RuntimeError
+// (deep_ep/include/deep_ep/common/exception.cuh:11-34).
+class EPException : public std::runtime_error {
+public:
+    using std::runtime_error::runtime_error;
+};
+
+#define EP_HIP_HOST_ASSERT(cond)                                                                      \
+    do {                                                                                              \
+        if (!(cond)) throw ::deep_ep::hip::EPException(std::string("Assertion failed: ") + #cond);    \
+    } while (0)
+
+inline int64_t align_up(int64_t x, int64_t y) { return (x + y - 1) / y * y; }
+
+constexpr int64_t kBufferAlignmentBytes = 2 * 1024 * 1024;   // symmetric::kNumAlignmentBytes (csrc/elastic/buffer.hpp:1363-1365)
+constexpr int64_t kRecordAlignBytes = 32;                    // ptx::kNumTMAAlignBytes, used only by the size calculus
+
+// Launch-shape knobs every call passes down (all zero = the library's own choice); seeded from DEEP_EP_HIP_<NAME>.
+inline deep_ep_hip_tuning& process_tuning() {
+    static deep_ep_hip_tuning tuning = [] {
+        deep_ep_hip_tuning t{};
+        auto env = [](const char* name) {
+            const char* v = std::getenv(name);
+            return v != nullptr ? std::atoi(v) : 0;
+        };
+        t.dispatch_launches = env("DEEP_EP_HIP_DISPATCH_LAUNCHES");
+        t.cast_pairs = env("DEEP_EP_HIP_CAST_PAIRS");
+        t.copy_vecs = env("DEEP_EP_HIP_COPY_VECS");
+        t.plain_loads = env("DEEP_EP_HIP_PLAIN_LOADS");
+        t.xcd_remap = env("DEEP_EP_HIP_XCD_REMAP");
+        t.combine_vecs = env("DEEP_EP_HIP_COMBINE_VECS");
+        t.ll_pairs = env("DEEP_EP_HIP_LL_PAIRS");
+        t.ll_threads = env("DEEP_EP_HIP_LL_THREADS");
+        t.ll_two_kernels = env("DEEP_EP_HIP_LL_TWO_KERNELS");
+        t.ll_combine_vecs = env("DEEP_EP_HIP_LL_COMBINE_VECS");
+        return t;
+    }();
+    return tuning;
+}
+
+inline int32_t* tuning_field(const std::string& name) {
+    deep_ep_hip_tuning& t = process_tuning();
+    if (name == "dispatch_launches") return &t.dispatch_launches;
+    if (name == "cast_pairs") return &t.cast_pairs;
+    if (name == "copy_vecs") return &t.copy_vecs;
+    if (name == "plain_loads") return &t.plain_loads;
+    if (name == "xcd_remap") return &t.xcd_remap;
+    if (name == "combine_vecs") return &t.combine_vecs;
+    if (name == "ll_pairs") return &t.ll_pairs;
+    if (name == "ll_threads") return &t.ll_threads;
+    if (name == "ll_two_kernels") return &t.ll_two_kernels;
+    if (name == "ll_combine_vecs") return &t.ll_combine_vecs;
+    throw EPException("unknown tuning field: " + name);
+}
+
+inline void check_abi(int rc, const char* what) {
+    if (rc != 0) {
+        std::ostringstream msg;
+        msg << "DeepEP HIP backend: " << what << " failed (code " << rc << "): " << deep_ep_hip_last_error();
+        throw EPException(msg.str());
+    }
+}
+
+template <class T>
+inline T* ptr_of(const std::optional<torch::Tensor>& t) {
+    return t.has_value() ? static_cast<T*>(t->data_ptr()) : nullptr;
+}
+
+class ElasticBuffer {
+public:
+    using cpu_comm_t = pybind11::object;      // there is no CPU communicator on one GPU; whatever is passed is ignored
+
+    ElasticBuffer(int rank_idx, int num_ranks, int64_t /*comm_handle*/, cpu_comm_t /*cpu_comm*/, int64_t num_buffer_bytes,
+                  int64_t num_cpu_buffer_bytes, bool allow_hybrid_mode, bool allow_multiple_reduction,
+                  bool prefer_overlap_with_compute, int /*sl_idx*/, int /*num_allocated_qps*/, int num_cpu_timeout_secs,
+                  int /*num_gpu_timeout_secs*/, bool explicitly_destroy)
+        : rank_idx_(rank_idx), num_ranks_(num_ranks), num_buffer_bytes_(num_buffer_bytes),
+          allow_hybrid_mode_(allow_hybrid_mode), allow_multiple_reduction_(allow_multiple_reduction),
+          prefer_overlap_with_compute_(prefer_overlap_with_compute), num_cpu_timeout_secs_(num_cpu_timeout_secs),
+          explicitly_destroy_(explicitly_destroy), comm_stream_(make_comm_stream()), last_stream_(comm_stream_) {
+        EP_HIP_HOST_ASSERT(0 <= rank_idx and rank_idx < num_ranks);
+        EP_HIP_HOST_ASSERT(num_ranks <= DEEP_EP_HIP_MAX_RANKS);
+        EP_HIP_HOST_ASSERT(num_buffer_bytes > 0 and num_buffer_bytes % kBufferAlignmentBytes == 0);
+        EP_HIP_HOST_ASSERT(num_cpu_buffer_bytes == 0);      // CPU buffers are not supported by the HIP backend
+        device_ = torch::Device(torch::kCUDA, comm_stream_.device_index());
+    }
+
+    // ---- lifetime ----
+    void destroy() {
+        EP_HIP_HOST_ASSERT(explicitly_destroy_);
+        EP_HIP_HOST_ASSERT(not destroyed_);
+        c10::hip::device_synchronize();
+        workspace_.reset();
+        destroyed_ = true;
+    }
+
+    bool is_destroyed() const { return destroyed_; }
+
+    c10::Stream get_comm_stream() const { return comm_stream_.unwrap(); }
+
+    // (RDMA ranks, load/store-reachable ranks): every logical rank is local
+    std::tuple<int, int> get_physical_domain_size() const { return {1, num_ranks_}; }
+
+    // (scale-out ranks, scale-up ranks)
+    std::tuple<int, int> get_logical_domain_size() const { return {1, num_ranks_}; }
+
+    void barrier(bool use_comm_stream, bool with_cpu_sync, bool /*sequential*/) {
+        // One process, one GPU: ordering between logical ranks is stream ordering.
+        if (with_cpu_sync) c10::hip::device_synchronize();
+        if (use_comm_stream) {
+            const Stream compute = current_stream();
+            if (compute != comm_stream_) {
+                stream_wait(comm_stream_, compute);
+                stream_wait(compute, comm_stream_);
+            }
+        }
+        if (with_cpu_sync) c10::hip::device_synchronize();
+    }
+
+    // Size the reference would ask for (csrc/elastic/buffer.hpp:588-688, direct mode, peers reachable by load/store).
+    // This backend scatters straight into the output tensors and needs no staging buffer; the number is kept so that
+    // `num_bytes` / `get_buffer_size_hint` stay drop-in.  `comm_handle` is the logical rank count here.
+    static int64_t calculate_buffer_size(int64_t comm_handle, int num_max_tokens_per_rank, int hidden, int num_topk,
+                                         bool use_fp8_dispatch, bool /*allow_hybrid_mode*/, bool allow_multiple_reduction) {
+        EP_HIP_HOST_ASSERT(num_max_tokens_per_rank > 0 and hidden > 0);
+        EP_HIP_HOST_ASSERT((hidden + 31) / 32 * 4 <= hidden);
+        const int64_t ranks = comm_handle > 0 ? comm_handle : 1;
+        const int64_t topk = num_topk == 0 ? 32 : num_topk;
+        auto record = [&](int64_t hidden_bytes, int64_t sf_bytes, bool with_metadata) {
+            // deep_ep/include/deep_ep/common/layout.cuh:187-208
+            const int64_t meta = topk * 8 + (with_metadata ? (1 + topk) * 4 : 0);
+            return align_up(hidden_bytes, kRecordAlignBytes) + align_up(sf_bytes, kRecordAlignBytes) + align_up(meta, kRecordAlignBytes);
+        };
+        const int64_t sf_packs = use_fp8_dispatch ? (hidden + 31) / 32 : 0;
+        const int64_t dispatch_bytes = ranks * num_max_tokens_per_rank * record(int64_t(hidden) * (use_fp8_dispatch ? 1 : 2), sf_packs * 4, true);
+        const int64_t tokens_in_layout = allow_multiple_reduction ? std::min<int64_t>(ranks, topk) : topk;
+        const int64_t combine_bytes = tokens_in_layout * num_max_tokens_per_rank * record(int64_t(hidden) * 2, 0, false);
+        return align_up(std::max(dispatch_bytes, combine_bytes), kBufferAlignmentBytes);
+    }
+
+    // ---- dispatch: argument order and the 16-tuple follow csrc/elastic/buffer.hpp:695-728,1166-1178 ----
+    // `cast_to_fp8` (extension): `x` is BF16 and the FP8 e4m3 cast with per-1x128 fp32 scales is fused into the
+    // scatter; the result equals casting first and dispatching the pair.
+    std::tuple<torch::Tensor, std::optional<torch::Tensor>, std::optional<torch::Tensor>, std::optional<torch::Tensor>,
+               std::optional<torch::Tensor>, int, int, std::vector<int>, torch::Tensor, torch::Tensor, torch::Tensor,
+               torch::Tensor, torch::Tensor, std::optional<torch::Tensor>, std::optional<torch::Tensor>,
+               std::optional<EventHandle>>
+    dispatch(const torch::Tensor& x, const std::optional<torch::Tensor>& sf, const torch::Tensor& topk_idx,
+             const std::optional<torch::Tensor>& topk_weights,
+             const std::optional<torch::Tensor>& cumulative_local_expert_recv_stats,
+             const std::optional<int>& cached_num_recv_tokens, const std::optional<int>& cached_num_expanded_tokens,
+             const std::optional<std::vector<int>>& cached_num_recv_tokens_per_expert_list,
+             const std::optional<torch::Tensor>& cached_psum_num_recv_tokens_per_scaleup_rank,
+             const std::optional<torch::Tensor>& cached_psum_num_recv_tokens_per_expert,
+             const std::optional<torch::Tensor>& cached_num_unaligned_recv_tokens_per_expert,
+             const std::optional<torch::Tensor>& cached_dst_buffer_slot_idx,
+             const std::optional<torch::Tensor>& /*cached_token_metadata_at_forward*/,
+             const std::optional<torch::Tensor>& cached_recv_src_metadata,
+             const std::optional<torch::Tensor>& /*cached_channel_linked_list*/, int num_max_tokens_per_rank,
+             int num_experts, int expert_alignment, int /*num_sms*/, int /*num_qps*/,
+             const std::optional<EventHandle>& previous_event,
+             const std::optional<EventHandle>& previous_event_before_epilogue, bool async_with_compute_stream,
+             bool allocate_on_comm_stream, bool do_handle_copy, bool do_cpu_sync, bool do_expand, bool do_zero_padding,
+             bool use_tma_aligned_col_major_sf, bool cast_to_fp8) {
+        EP_HIP_HOST_ASSERT(not destroyed_);
+        EP_HIP_HOST_ASSERT(not do_zero_padding or do_expand);
+        const bool cached_mode = cached_num_recv_tokens.has_value();
+        if (cached_mode) {
+            EP_HIP_HOST_ASSERT(cached_num_recv_tokens_per_expert_list.has_value());
+            EP_HIP_HOST_ASSERT(cached_num_expanded_tokens.has_value());
+            EP_HIP_HOST_ASSERT(cached_psum_num_recv_tokens_per_scaleup_rank.has_value());
+            EP_HIP_HOST_ASSERT(cached_psum_num_recv_tokens_per_expert.has_value());
+            EP_HIP_HOST_ASSERT(cached_num_unaligned_recv_tokens_per_expert.has_value());
+            EP_HIP_HOST_ASSERT(cached_dst_buffer_slot_idx.has_value());
+            EP_HIP_HOST_ASSERT(cached_recv_src_metadata.has_value());
+            EP_HIP_HOST_ASSERT(not do_cpu_sync);                                       // no CPU sync with a cached handle
+            EP_HIP_HOST_ASSERT(not cumulative_local_expert_recv_stats.has_value());    // statistics need a fresh layout
+        }
+
+        EP_HIP_HOST_ASSERT(x.dim() == 2 and x.is_cuda() and x.is_contiguous());
+        const int num_tokens = static_cast<int>(x.size(0)), hidden = static_cast<int>(x.size(1));
+        EP_HIP_HOST_ASSERT((hidden * x.element_size()) % 16 == 0);
+        EP_HIP_HOST_ASSERT(num_tokens <= num_max_tokens_per_rank);
+        const int R = num_ranks_;
+        EP_HIP_HOST_ASSERT(num_experts % R == 0);
+        EP_HIP_HOST_ASSERT(num_experts <= DEEP_EP_HIP_MAX_EXPERTS);
+
+        int payload, num_sf_packs = 0;
+        int64_t sf_ts = 0, sf_hs = 0;
+        torch::ScalarType out_dtype = x.scalar_type();
+        std::optional<torch::ScalarType> sf_dtype;
+        if (cast_to_fp8) {
+            EP_HIP_HOST_ASSERT(not sf.has_value() and x.scalar_type() == torch::kBFloat16);
+            EP_HIP_HOST_ASSERT(hidden % 128 == 0);
+            payload = DEEP_EP_HIP_PAYLOAD_CAST_FP8;
+            num_sf_packs = hidden / 128;
+            out_dtype = torch::kFloat8_e4m3fn;
+            sf_dtype = torch::kFloat32;
+        } else if (sf.has_value()) {
+            EP_HIP_HOST_ASSERT(x.element_size() == 1);
+            EP_HIP_HOST_ASSERT(sf->dim() == 2 and sf->is_cuda() and sf->size(0) == num_tokens);
+            EP_HIP_HOST_ASSERT(sf->element_size() == 4);                 // fp32, or four packed UE8M0 exponents
+            payload = DEEP_EP_HIP_PAYLOAD_FP8;
+            num_sf_packs = static_cast<int>(sf->size(1));
+            sf_dtype = sf->scalar_type();
+            sf_ts = sf->stride(0);
+            sf_hs = sf->stride(1);
+        } else {
+            EP_HIP_HOST_ASSERT(x.scalar_type() == torch::kBFloat16);
+            payload = DEEP_EP_HIP_PAYLOAD_BF16;
+        }
+
+        EP_HIP_HOST_ASSERT(topk_idx.dim() == 2 and topk_idx.size(0) == num_tokens);
+        const int num_topk = static_cast<int>(topk_idx.size(1));
+        EP_HIP_HOST_ASSERT(1 <= num_topk and num_topk <= DEEP_EP_HIP_MAX_TOPK);
+        EP_HIP_HOST_ASSERT(topk_idx.scalar_type() == torch::kInt64);
+        EP_HIP_HOST_ASSERT(topk_idx.is_cuda() and topk_idx.is_contiguous());
+        if (topk_weights.has_value()) {
+            EP_HIP_HOST_ASSERT(topk_weights->dim() == 2 and topk_weights->size(0) == num_tokens and topk_weights->size(1) == num_topk);
+            EP_HIP_HOST_ASSERT(topk_weights->is_cuda() and topk_weights->is_contiguous() and topk_weights->scalar_type() == torch::kFloat32);
+        }
+        if (cumulative_local_expert_recv_stats.has_value()) {
+            const auto& s = *cumulative_local_expert_recv_stats;
+            EP_HIP_HOST_ASSERT(s.dim() == 1 and s.size(0) == num_experts and s.scalar_type() == torch::kInt32 and s.is_cuda() and s.is_contiguous());
+        }
+
+        StreamScope scope(*this, previous_event, allocate_on_comm_stream, async_with_compute_stream);
+        const Stream& run = scope.run_stream;
+        const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(device_);
+        torch::Tensor workspace = acquire_workspace(run, num_tokens, num_topk, num_experts);
+
+        torch::Tensor counts, psum_rank, psum_expert, num_unaligned, dst_slot;
+        std::optional<torch::Tensor> copied_topk_idx;
+        {
+            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);      // allocations below belong to the run stream
+            if (cached_mode) {
+                psum_rank = *cached_psum_num_recv_tokens_per_scaleup_rank;
+                psum_expert = *cached_psum_num_recv_tokens_per_expert;
+                num_unaligned = *cached_num_unaligned_recv_tokens_per_expert;
+                EP_HIP_HOST_ASSERT(psum_rank.dim() == 1 and psum_rank.size(0) == R and psum_rank.scalar_type() == torch::kInt32 and psum_rank.is_cuda());
+                EP_HIP_HOST_ASSERT(psum_expert.dim() == 1 and psum_expert.size(0) == num_experts and psum_expert.scalar_type() == torch::kInt32);
+                EP_HIP_HOST_ASSERT(num_unaligned.dim() == 1 and num_unaligned.size(0) == num_experts);
+                dst_slot = *cached_dst_buffer_slot_idx;
+                EP_HIP_HOST_ASSERT(dst_slot.dim() == 2 and dst_slot.size(0) == num_tokens and dst_slot.size(1) == num_topk and
+                                   dst_slot.scalar_type() == torch::kInt32 and dst_slot.is_contiguous());
+            } else {
+                counts = torch::empty({R + 2 * int64_t(num_experts)}, i32);     // one allocation, one D2H copy when syncing
+                psum_rank = counts.slice(0, 0, R);
+                psum_expert = counts.slice(0, R, R + num_experts);
+                num_unaligned = counts.slice(0, R + num_experts, R + 2 * int64_t(num_experts));
+                dst_slot = torch::empty({num_tokens, num_topk}, i32);
+                if (do_handle_copy) copied_topk_idx = torch::empty_like(topk_idx);
+            }
+        }
+
+        deep_ep_hip_dispatch_args args{};
+        args.payload = payload;
+        args.cached = cached_mode ? 1 : 0;
+        args.do_expand = do_expand ? 1 : 0;
+        args.do_zero_padding = do_zero_padding ? 1 : 0;
+        args.num_tokens = num_tokens; args.hidden = hidden; args.num_topk = num_topk;
+        args.num_experts = num_experts; args.num_ranks = R; args.rank_idx = rank_idx_;
+        args.num_max_tokens_per_rank = num_max_tokens_per_rank;
+        args.expert_alignment = expert_alignment;
+        args.x = x.data_ptr();
+        args.sf = sf.has_value() ? sf->data_ptr() : nullptr;
+        args.sf_token_stride = sf_ts; args.sf_hidden_stride = sf_hs;
+        args.num_sf_packs = num_sf_packs;
+        args.topk_idx = static_cast<const int64_t*>(topk_idx.data_ptr());
+        args.topk_weights = ptr_of<const float>(topk_weights);
+        args.copied_topk_idx = ptr_of<int64_t>(copied_topk_idx);
+        args.psum_num_recv_tokens_per_rank = static_cast<int32_t*>(psum_rank.data_ptr());
+        args.psum_num_recv_tokens_per_expert = static_cast<int32_t*>(psum_expert.data_ptr());
+        args.num_unaligned_recv_tokens_per_expert = static_cast<int32_t*>(num_unaligned.data_ptr());
+        args.cumulative_local_expert_recv_stats = ptr_of<int32_t>(cumulative_local_expert_recv_stats);
+        args.host_counts = nullptr;
+        args.dst_buffer_slot_idx = static_cast<int32_t*>(dst_slot.data_ptr());
+        args.workspace = workspace.data_ptr();
+        args.workspace_bytes = static_cast<uint64_t>(workspace.numel());
+        args.tuning = process_tuning();
+        void* stream_ptr = run.stream();
+
+        // Sizes of the outputs
+        int num_recv_tokens, num_expanded_tokens;
+        std::vector<int> per_expert_list;
+        if (cached_mode) {
+            num_recv_tokens = *cached_num_recv_tokens;
+            num_expanded_tokens = *cached_num_expanded_tokens;
+            per_expert_list = *cached_num_recv_tokens_per_expert_list;
+        } else if (do_cpu_sync) {
+            args.phases = DEEP_EP_HIP_PHASE_LAYOUT;
+            check_abi(deep_ep_hip_launch_dispatch(&args, stream_ptr), "dispatch layout");
+            torch::Tensor host;
+            {
+                c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
+                host = counts.cpu();                               // waits for the layout kernel
+            }
+            read_and_clear_status(workspace, "dispatch");
+            const int32_t* h = host.data_ptr<int32_t>();
+            num_recv_tokens = h[R - 1];
+            num_expanded_tokens = 0;
+            per_expert_list.resize(num_experts);
+            for (int e = 0; e < num_experts; ++e) {
+                const int aligned = (h[R + num_experts + e] + expert_alignment - 1) / expert_alignment * expert_alignment;
+                per_expert_list[e] = aligned;
+                num_expanded_tokens += aligned;
+            }
+        } else {
+            num_recv_tokens = num_max_tokens_per_rank * R;
+            num_expanded_tokens = num_max_tokens_per_rank * std::min(num_topk, num_experts) + (expert_alignment - 1) * num_experts;
+            num_expanded_tokens = static_cast<int>(align_up(num_expanded_tokens, expert_alignment));
+        }
+
+        const int64_t num_allocated = do_expand ? num_expanded_tokens : num_recv_tokens;
+        torch::Tensor recv_x, recv_src_metadata;
+        std::optional<torch::Tensor> recv_sf, recv_topk_idx, recv_topk_weights;
+        int64_t rsf_ts = 0, rsf_hs = 0;
+        {
+            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
+            recv_x = torch::empty({num_allocated, hidden}, torch::TensorOptions().dtype(out_dtype).device(device_));
+            recv_src_metadata = cached_mode ? *cached_recv_src_metadata : torch::empty({num_recv_tokens, num_topk + 2}, i32);
+            if (sf_dtype.has_value()) {
+                if (not use_tma_aligned_col_major_sf) {
+                    rsf_ts = num_sf_packs; rsf_hs = 1;
+                } else {
+                    rsf_ts = 1; rsf_hs = align_up(num_allocated, 4);        // column-major, rows padded to 4 (csrc/elastic/buffer.hpp:1092-1101)
+                }
+                recv_sf = torch::empty_strided({num_allocated, num_sf_packs}, {rsf_ts, rsf_hs},
+                                               torch::TensorOptions().dtype(*sf_dtype).device(device_));
+            }
+            if (not do_expand) recv_topk_idx = torch::empty({num_allocated, num_topk}, topk_idx.options());
+            if (topk_weights.has_value()) {
+                const auto f32 = torch::TensorOptions().dtype(torch::kFloat32).device(device_);
+                recv_topk_weights = do_expand ? torch::empty({num_allocated}, f32) : torch::empty({num_allocated, num_topk}, f32);
+            }
+        }
+
+        if (previous_event_before_epilogue.has_value()) stream_wait(run, *previous_event_before_epilogue);
+
+        args.phases = (cached_mode or do_cpu_sync) ? DEEP_EP_HIP_PHASE_MOVE : (DEEP_EP_HIP_PHASE_LAYOUT | DEEP_EP_HIP_PHASE_MOVE);
+        args.recv_src_metadata = static_cast<int32_t*>(recv_src_metadata.data_ptr());
+        args.recv_x = recv_x.data_ptr();
+        args.recv_sf = recv_sf.has_value() ? recv_sf->data_ptr() : nullptr;
+        args.recv_sf_token_stride = rsf_ts; args.recv_sf_hidden_stride = rsf_hs;
+        args.recv_topk_idx = ptr_of<int64_t>(recv_topk_idx);
+        args.recv_topk_weights = ptr_of<float>(recv_topk_weights);
+        args.recv_capacity = recv_src_metadata.size(0);
+        args.expanded_capacity = do_expand ? num_expanded_tokens : 0;
+        check_abi(deep_ep_hip_launch_dispatch(&args, stream_ptr), "dispatch");
+
+        std::optional<EventHandle> event = scope.finish(
+            {x, sf, topk_idx, topk_weights, recv_x, recv_sf, recv_topk_idx, recv_topk_weights,
+             cumulative_local_expert_recv_stats, copied_topk_idx, psum_rank, psum_expert, num_unaligned, recv_src_metadata,
+             dst_slot, workspace});
+        return {recv_x, recv_sf, recv_topk_idx, recv_topk_weights, copied_topk_idx, num_recv_tokens, num_expanded_tokens,
+                per_expert_list, psum_rank, psum_expert, num_unaligned, recv_src_metadata, dst_slot, std::nullopt,
+                std::nullopt, event};
+    }
+
+    // ---- combine: argument order and the 3-tuple follow csrc/elastic/buffer.hpp:1181-1198,1344 ----
+    // `dst_buffer_slot_idx` (the handle's token -> received-row map) is what lets a single GPU gather instead of
+    // routing rows back through a buffer; the Python wrapper passes it.
+    std::tuple<torch::Tensor, std::optional<torch::Tensor>, std::optional<EventHandle>>
+    combine(const torch::Tensor& x, const std::optional<torch::Tensor>& topk_weights, const std::optional<torch::Tensor>& bias_0,
+            const std::optional<torch::Tensor>& bias_1, const torch::Tensor& src_metadata, const torch::Tensor& combined_topk_idx,
+            const torch::Tensor& psum_num_recv_tokens_per_scaleup_rank,
+            const std::optional<torch::Tensor>& /*token_metadata_at_forward*/,
+            const std::optional<torch::Tensor>& /*channel_linked_list*/, int num_experts, int num_max_tokens_per_rank,
+            int /*num_sms*/, int /*num_qps*/, const std::optional<EventHandle>& previous_event,
+            const std::optional<EventHandle>& previous_event_before_epilogue, bool async_with_compute_stream,
+            bool allocate_on_comm_stream, bool use_expanded_layout, const std::optional<torch::Tensor>& dst_buffer_slot_idx) {
+        EP_HIP_HOST_ASSERT(not destroyed_);
+        EP_HIP_HOST_ASSERT(dst_buffer_slot_idx.has_value());
+        EP_HIP_HOST_ASSERT(x.dim() == 2 and x.is_cuda() and x.is_contiguous());
+        EP_HIP_HOST_ASSERT(x.scalar_type() == torch::kBFloat16);
+        const int64_t num_x_rows = x.size(0);
+        const int hidden = static_cast<int>(x.size(1));
+        EP_HIP_HOST_ASSERT((hidden * 2) % 16 == 0);
+        EP_HIP_HOST_ASSERT(combined_topk_idx.dim() == 2 and combined_topk_idx.scalar_type() == torch::kInt64 and combined_topk_idx.is_contiguous());
+        const int num_tokens = static_cast<int>(combined_topk_idx.size(0)), num_topk = static_cast<int>(combined_topk_idx.size(1));
+        EP_HIP_HOST_ASSERT(dst_buffer_slot_idx->dim() == 2 and dst_buffer_slot_idx->size(0) == num_tokens and dst_buffer_slot_idx->size(1) == num_topk);
+        EP_HIP_HOST_ASSERT(src_metadata.dim() == 2 and src_metadata.size(1) == num_topk + 2);
+        if (topk_weights.has_value()) {
+            EP_HIP_HOST_ASSERT(topk_weights->scalar_type() == torch::kFloat32 and topk_weights->is_cuda() and topk_weights->is_contiguous());
+            if (use_expanded_layout) EP_HIP_HOST_ASSERT(topk_weights->dim() == 1 and topk_weights->size(0) == num_x_rows);
+            else EP_HIP_HOST_ASSERT(topk_weights->dim() == 2 and topk_weights->size(0) == num_x_rows and topk_weights->size(1) == num_topk);
+        }
+        for (const auto* b : {&bias_0, &bias_1}) {
+            if (b->has_value()) {
+                const auto& t = **b;
+                EP_HIP_HOST_ASSERT(t.scalar_type() == x.scalar_type() and t.dim() == 2 and t.size(0) == num_tokens and t.size(1) == hidden and
+                                   t.is_cuda() and t.is_contiguous());
+            }
+        }
+        EP_HIP_HOST_ASSERT(bias_0.has_value() or not bias_1.has_value());
+
+        StreamScope scope(*this, previous_event, allocate_on_comm_stream, async_with_compute_stream);
+        const Stream& run = scope.run_stream;
+        torch::Tensor workspace = acquire_workspace(run, num_tokens, num_topk, num_experts);
+        torch::Tensor combined_x;
+        std::optional<torch::Tensor> combined_topk_weights;
+        {
+            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
+            combined_x = torch::empty({num_tokens, hidden}, x.options());
+            if (topk_weights.has_value())
+                combined_topk_weights = torch::empty({num_tokens, num_topk}, torch::TensorOptions().dtype(torch::kFloat32).device(device_));
+        }
+        if (previous_event_before_epilogue.has_value()) stream_wait(run, *previous_event_before_epilogue);
+
+        deep_ep_hip_combine_args args{};
+        args.do_expand = use_expanded_layout ? 1 : 0;
+        args.allow_multiple_reduction = allow_multiple_reduction_ ? 1 : 0;
+        args.num_tokens = num_tokens; args.hidden = hidden; args.num_topk = num_topk;
+        args.num_experts = num_experts; args.num_ranks = num_ranks_;
+        args.rank_idx = rank_idx_; args.num_max_tokens_per_rank = num_max_tokens_per_rank;
+        args.x = x.data_ptr();
+        args.num_x_rows = num_x_rows;
+        args.topk_weights = ptr_of<const float>(topk_weights);
+        args.bias_0 = bias_0.has_value() ? bias_0->data_ptr() : nullptr;
+        args.bias_1 = bias_1.has_value() ? bias_1->data_ptr() : nullptr;
+        args.topk_idx = static_cast<const int64_t*>(combined_topk_idx.data_ptr());
+        args.dst_buffer_slot_idx = static_cast<const int32_t*>(dst_buffer_slot_idx->data_ptr());
+        args.recv_src_metadata = static_cast<const int32_t*>(src_metadata.data_ptr());
+        args.num_recv_rows = src_metadata.size(0);
+        args.psum_num_recv_tokens_per_rank = static_cast<const int32_t*>(psum_num_recv_tokens_per_scaleup_rank.data_ptr());
+        args.combined_x = combined_x.data_ptr();
+        args.combined_topk_weights = ptr_of<float>(combined_topk_weights);
+        args.workspace = workspace.data_ptr();
+        args.workspace_bytes = static_cast<uint64_t>(workspace.numel());
+        args.tuning = process_tuning();
+        check_abi(deep_ep_hip_launch_combine(&args, run.stream()), "combine");
+
+        std::optional<EventHandle> event = scope.finish({x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx,
+                                                         psum_num_recv_tokens_per_scaleup_rank, dst_buffer_slot_idx, combined_x,
+                                                         combined_topk_weights, workspace});
+        return {combined_x, combined_topk_weights, event};
+    }
+
+    // ---- V1 `Buffer.get_dispatch_layout` on this buffer (csrc/legacy/buffer.hpp:337-404) ----
+    std::tuple<torch::Tensor, std::optional<torch::Tensor>, torch::Tensor, torch::Tensor, std::optional<EventHandle>>
+    get_dispatch_layout(const torch::Tensor& topk_idx, int num_experts, const std::optional<EventHandle>& previous_event,
+                        bool async_finish, bool allocate_on_comm_stream) {
+        EP_HIP_HOST_ASSERT(topk_idx.dim() == 2 and topk_idx.is_contiguous() and topk_idx.is_cuda());
+        EP_HIP_HOST_ASSERT(topk_idx.scalar_type() == torch::kInt64);
+        EP_HIP_HOST_ASSERT(num_experts > 0 and num_experts % num_ranks_ == 0);
+        const int num_tokens = static_cast<int>(topk_idx.size(0)), num_topk = static_cast<int>(topk_idx.size(1));
+        StreamScope scope(*this, previous_event, allocate_on_comm_stream, async_finish);
+        const Stream& run = scope.run_stream;
+        torch::Tensor workspace = acquire_workspace(run, num_tokens, num_topk, num_experts);
+        torch::Tensor per_rank, per_expert, in_rank;
+        {
+            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
+            const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(device_);
+            per_rank = torch::empty({num_ranks_}, i32);
+            per_expert = torch::empty({num_experts}, i32);
+            in_rank = torch::empty({num_tokens, num_ranks_}, torch::TensorOptions().dtype(torch::kBool).device(device_));
+        }
+        deep_ep_hip_layout_args args{};
+        args.topk_idx = static_cast<const int64_t*>(topk_idx.data_ptr());
+        args.num_tokens = num_tokens; args.num_topk = num_topk; args.num_experts = num_experts; args.num_ranks = num_ranks_;
+        args.num_tokens_per_rank = static_cast<int32_t*>(per_rank.data_ptr());
+        args.num_tokens_per_expert = static_cast<int32_t*>(per_expert.data_ptr());
+        args.is_token_in_rank = static_cast<uint8_t*>(in_rank.data_ptr());
+        args.workspace = workspace.data_ptr();
+        args.workspace_bytes = static_cast<uint64_t>(workspace.numel());
+        check_abi(deep_ep_hip_launch_layout(&args, run.stream()), "get_dispatch_layout");
+        std::optional<EventHandle> event = scope.finish({topk_idx, per_rank, per_expert, in_rank, workspace});
+        return {per_rank, std::nullopt, per_expert, in_rank, event};
+    }
+
+    // Synchronise and raise if a kernel flagged bad routing input or a row that did not fit the outputs.
+    void check_device_status(const std::string& what) {
+        c10::hip::device_synchronize();
+        if (workspace_.has_value()) read_and_clear_status(*workspace_, what.c_str());
+    }
+
+    // The status word as the GPU has it now (every launch queued so far has finished): 0 = nothing flagged.
+    int device_status() {
+        c10::hip::device_synchronize();
+        return workspace_.has_value() ? workspace_->slice(0, 0, 4).view(torch::kInt32).item<int>() : 0;
+    }
+
+    // The bookkeeping words at the head of the workspace (status, launch protocol), copied to the host after a full
+    // synchronisation: between launches everything but the status word and the two row totals reads zero.
+    torch::Tensor workspace_control_words() {
+        c10::hip::device_synchronize();
+        const int64_t n = static_cast<int64_t>(deep_ep_hip_workspace_control_bytes());
+        if (not workspace_.has_value()) return torch::zeros({n / 4}, torch::kInt32);
+        return workspace_->slice(0, 0, n).view(torch::kInt32).cpu();
+    }
+
+private:
+    // The one communication stream of the buffer, at the default priority.  Fails loudly when there is no GPU.
+    static Stream make_comm_stream() {
+        if (c10::hip::device_count() <= 0) throw EPException("DeepEP HIP backend: no GPU is visible");
+        return c10::hip::getStreamFromPoolMasqueradingAsCUDA(false);
+    }
+
+    // Stream choreography of one call (csrc/elastic/buffer.hpp:528-586).  The reference always runs on its comm
+    // stream; when nothing asks for overlap the same ordering is had, without two cross-stream waits, by running on
+    // the caller's stream.  The destructor restores the current stream whatever happens in between.
+    struct StreamScope {
+        ElasticBuffer& buffer;
+        Stream compute_stream, run_stream;
+        bool allocate_on_comm_stream, async_with_compute_stream, switched = false;
+
+        StreamScope(ElasticBuffer& b, const std::optional<EventHandle>& previous_event, bool allocate_on_comm, bool async)
+            : buffer(b), compute_stream(current_stream()), run_stream(compute_stream), allocate_on_comm_stream(allocate_on_comm),
+              async_with_compute_stream(async) {
+            if (previous_event.has_value()) EP_HIP_HOST_ASSERT(allocate_on_comm_stream);
+            const bool overlap = previous_event.has_value() or allocate_on_comm_stream or async_with_compute_stream;
+            if (not overlap) return;
+            run_stream = buffer.comm_stream_;
+            if (allocate_on_comm_stream) {
+                c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(buffer.comm_stream_);
+                switched = true;
+            }
+            if (previous_event.has_value()) stream_wait(run_stream, *previous_event);
+            else if (run_stream != compute_stream) stream_wait(run_stream, compute_stream);
+        }
+
+        ~StreamScope() {
+            if (switched) c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(compute_stream);
+        }
+
+        std::optional<EventHandle> finish(std::initializer_list<std::optional<torch::Tensor>> tensors) {
+            buffer.last_stream_ = run_stream;
+            std::optional<EventHandle> event;
+            if (run_stream != compute_stream) {
+                if (async_with_compute_stream) {
+                    event = EventHandle(run_stream);
+                    const char* avoid = std::getenv("EP_AVOID_RECORD_STREAM");
+                    if (avoid != nullptr and std::atoi(avoid) != 0) {
+                        for (const auto& t : tensors)
+                            if (t.has_value()) event->tensors_to_record.push_back(t);
+                    } else {
+                        for (const auto& t : tensors) {
+                            if (t.has_value() and t->is_cuda()) {
+                                t->record_stream(compute_stream.unwrap());
+                                t->record_stream(run_stream.unwrap());
+                            }
+                        }
+                    }
+                } else {
+                    stream_wait(compute_stream, run_stream);
+                }
+            } else if (async_with_compute_stream) {
+                event = EventHandle(run_stream);
+            }
+            return event;
+        }
+    };
+
+    // The workspace is shared by every call on this buffer and is not re-entrant: a call that runs on another
+    // stream than the previous one first waits for everything queued there.  It grows geometrically, so that
+    // steady-state calls never allocate; a replaced workspace stays reserved for the stream that last used it.
+    torch::Tensor acquire_workspace(const Stream& run, int num_tokens, int num_topk, int num_experts) {
+        if (last_stream_ != run) stream_wait(run, last_stream_);
+        const int64_t need = static_cast<int64_t>(deep_ep_hip_workspace_bytes(std::max(num_tokens, 1), num_topk, num_experts, num_ranks_));
+        if (not workspace_.has_value() or workspace_->numel() < need) {
+            const int64_t size = std::max(need, 2 * (workspace_.has_value() ? workspace_->numel() : int64_t(0)));
+            if (workspace_.has_value()) workspace_->record_stream(last_stream_.unwrap());
+            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
+            workspace_ = torch::zeros({size}, torch::TensorOptions().dtype(torch::kUInt8).device(device_));
+        }
+        return *workspace_;
+    }
+
+    void read_and_clear_status(const torch::Tensor& workspace, const char* what) {
+        const int status = workspace.slice(0, 0, 4).view(torch::kInt32).item<int>();
+        if (status == 0) return;
+        // also the launch bookkeeping words that follow: a dispatch that gave up has left them mid-protocol
+        workspace.slice(0, 0, static_cast<int64_t>(deep_ep_hip_workspace_control_bytes())).zero_();
+        std::string reasons;
+        auto add = [&](int bit, const char* text) {
+            if (status & bit) reasons += (reasons.empty() ? "" : "; ") + std::string(text);
+        };
+        add(DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE, "topk_idx holds an expert id >= num_experts");
+        add(DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT, "a token selects the same expert twice");
+        add(DEEP_EP_HIP_STATUS_ROW_OVERFLOW, "a received row did not fit the output tensors");
+        add(DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT, "a single-launch dispatch gave up waiting for its counting workgroups (outputs invalid)");
+        throw EPException(std::string("DeepEP HIP backend: ") + what + ": " + reasons);
+    }
+
+    int rank_idx_, num_ranks_;
+    int64_t num_buffer_bytes_;
+    bool allow_hybrid_mode_, allow_multiple_reduction_, prefer_overlap_with_compute_;
+    int num_cpu_timeout_secs_;
+    bool explicitly_destroy_;
+    bool destroyed_ = false;
+    Stream comm_stream_;
+    Stream last_stream_;                     // stream of the last launch that used the workspace
+    torch::Device device_ = torch::Device(torch::kCUDA, 0);
+    std::optional<torch::Tensor> workspace_;
+};
+
+}  // namespace deep_ep::hip

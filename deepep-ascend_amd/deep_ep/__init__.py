@@ -2,8 +2,8 @@
 reference's deep_ep/__init__.py:92-109).  The HIP kernel library is loaded at import; without it
 the import fails (there is no fallback path)."""
 from . import _abi  # noqa: F401  (loads libdeep_ep_hip.so or raises)
-from ._C import Config, EventHandle, topk_idx_t
-from ._abi import tuning
+from ._binding import EventHandle, topk_idx_t, tuning
+from ._runtime import Config
 from .buffers.elastic import ElasticBuffer, EPHandle, LogicalGroup
 from .buffers.legacy import Buffer
 from .utils.event import EventOverlap
@@ -11,4 +11,4 @@ from .utils.event import EventOverlap
 __version__ = "2.0.0+hip"
 
 __all__ = ["ElasticBuffer", "EPHandle", "EventOverlap", "EventHandle", "Buffer", "Config", "LogicalGroup", "topk_idx_t",
-           "__version__"]
+           "tuning", "__version__"]

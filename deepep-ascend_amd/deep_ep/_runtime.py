@@ -1,10 +1,12 @@
-"""Host runtime of the HIP backend: the objects the reference exposes from its compiled
-`deep_ep._C` module (csrc/python_api.cpp:37-54, csrc/elastic/binding.hpp:9-44), written over the
-C ABI in include/deep_ep_hip.h.  PyTorch supplies device memory and streams only.
+"""Host runtime of the HIP backend in Python, over the ctypes binding of the C ABI (include/deep_ep_hip.h): a second
+binding of the same ABI beside the compiled `deep_ep._C` extension (csrc/host/), with the same names and the same
+argument and tuple contracts (csrc/python_api.cpp:37-54, csrc/elastic/binding.hpp:9-44 of the reference).  The V2
+`ElasticBuffer` uses the compiled extension when it is built and this module otherwise (or when
+DEEP_EP_HIP_BINDING=ctypes); the V1 `Buffer` surface (intranode dispatch / combine, low latency) always runs on this
+module.  PyTorch supplies device memory and streams only.
 
-Public names (same set as the reference's binding contract, tests/platform/api_contract.py):
-`get_platform`, `topk_idx_t`, `EventHandle`, `ElasticBuffer`, `calculate_elastic_buffer_size`,
-plus `get_elastic_buffer_alignment`.
+Public names: `get_platform`, `topk_idx_t`, `EventHandle`, `ElasticBuffer`, `calculate_elastic_buffer_size`,
+`get_elastic_buffer_alignment`, `Config`.
 
 One GPU, logical ranks: `num_ranks` only decides which bucket (destination rank) an expert
 belongs to; every bucket lives in this GPU's HBM.  One call moves the tokens of the logical
@@ -57,6 +59,12 @@ class EventHandle:
 
     def current_stream_wait(self) -> None:
         torch.cuda.current_stream().wait_event(self.event)
+
+
+def _stream_wait_event(stream: torch.cuda.Stream, event) -> None:
+    """`stream` waits for `event`, an EventHandle of this module or of the compiled extension."""
+    with torch.cuda.stream(stream):
+        event.current_stream_wait()
 
 
 def _token_record_bytes(hidden_bytes: int, sf_bytes: int, num_topk: int, with_metadata: bool) -> int:
@@ -116,6 +124,7 @@ class ElasticBuffer:
         self.device = torch.device("cuda", torch.cuda.current_device())
         self.comm_stream = torch.cuda.Stream(device=self.device)
         self._workspace: Optional[torch.Tensor] = None
+        self._last_stream: Optional[torch.cuda.Stream] = None      # stream of the last launch that used the workspace
         self._destroyed = False
 
     # ---- lifetime ----
@@ -151,13 +160,40 @@ class ElasticBuffer:
             torch.cuda.synchronize(self.device)
 
     # ---- helpers ----
-    def _get_workspace(self, num_tokens: int, num_topk: int, num_experts: int) -> torch.Tensor:
+    def _get_workspace(self, run_stream: torch.cuda.Stream, num_tokens: int, num_topk: int, num_experts: int) -> torch.Tensor:
+        """The workspace is shared by every call on this buffer and is not re-entrant: a call that runs on another
+        stream than the previous one first waits for everything queued there.  It grows geometrically, so that
+        steady-state calls never allocate; a replaced workspace stays reserved for the stream that last used it."""
+        if self._last_stream is not None and self._last_stream != run_stream:
+            run_stream.wait_stream(self._last_stream)
         need = _abi.lib.deep_ep_hip_workspace_bytes(max(num_tokens, 1), num_topk, num_experts, self.num_ranks)
         if self._workspace is None or self._workspace.numel() < need:
-            # grow geometrically so steady-state calls never allocate
             size = max(need, 2 * (self._workspace.numel() if self._workspace is not None else 0))
-            self._workspace = torch.zeros(size, dtype=torch.uint8, device=self.device)
+            if self._workspace is not None and self._last_stream is not None:
+                self._workspace.record_stream(self._last_stream)
+            with torch.cuda.stream(run_stream):
+                self._workspace = torch.zeros(size, dtype=torch.uint8, device=self.device)
+        self._last_stream = run_stream
         return self._workspace
+
+    def check_device_status(self, what: str = "routing") -> None:
+        """Synchronise and raise if a kernel flagged bad routing input or a row that did not fit the outputs."""
+        torch.cuda.synchronize(self.device)
+        if self._workspace is not None:
+            self._read_and_clear_status(what)
+
+    def workspace_control_words(self) -> torch.Tensor:
+        """The bookkeeping words at the head of the workspace (status, launch protocol), copied to the host after a full
+        synchronisation: between launches everything but the status word and the two row totals reads zero."""
+        torch.cuda.synchronize(self.device)
+        n = _abi.lib.deep_ep_hip_workspace_control_bytes()
+        if self._workspace is None:
+            return torch.zeros(n // 4, dtype=torch.int32)
+        return self._workspace[:n].view(torch.int32).cpu()
+
+    def device_status(self) -> int:
+        torch.cuda.synchronize(self.device)
+        return 0 if self._workspace is None else int(self._workspace[:4].view(torch.int32).item())
 
     def _read_and_clear_status(self, what: str) -> None:
         ws = self._workspace
@@ -193,7 +229,7 @@ class ElasticBuffer:
         if allocate_on_comm_stream:
             torch.cuda.set_stream(self.comm_stream)
         if previous_event is not None:
-            self.comm_stream.wait_event(previous_event.event)
+            _stream_wait_event(self.comm_stream, previous_event)
         else:
             self.comm_stream.wait_stream(compute_stream)
         return compute_stream, self.comm_stream
@@ -215,8 +251,6 @@ class ElasticBuffer:
                 compute_stream.wait_stream(run_stream)
         elif async_with_compute_stream:
             event = EventHandle(run_stream)
-        if allocate_on_comm_stream:
-            torch.cuda.set_stream(compute_stream)
         return event
 
     # ---- dispatch ----
@@ -302,125 +336,129 @@ class ElasticBuffer:
                          s.is_contiguous(), "cumulative_local_expert_recv_stats is int32 [num_experts] on device")
 
         compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_with_compute_stream)
-        dev = self.device
-        i32 = dict(dtype=torch.int32, device=dev)
-        workspace = self._get_workspace(num_tokens, num_topk, num_experts)
+        try:
+            dev = self.device
+            i32 = dict(dtype=torch.int32, device=dev)
+            workspace = self._get_workspace(run_stream, num_tokens, num_topk, num_experts)
 
-        with torch.cuda.stream(run_stream):
-            if cached_mode:
-                psum_rank = cached_psum_num_recv_tokens_per_scaleup_rank
-                psum_expert = cached_psum_num_recv_tokens_per_expert
-                num_unaligned = cached_num_unaligned_recv_tokens_per_expert
-                _host_assert(psum_rank.shape == (R,) and psum_rank.dtype == torch.int32 and psum_rank.is_cuda,
-                             "cached psum per rank is int32 [num_ranks]")
-                _host_assert(psum_expert.shape == (num_experts,) and psum_expert.dtype == torch.int32,
-                             "cached psum per expert is int32 [num_experts]")
-                _host_assert(num_unaligned is not None and num_unaligned.shape == (num_experts,),
-                             "cached unaligned counts are int32 [num_experts]")
-                dst_slot = cached_dst_buffer_slot_idx
-                _host_assert(tuple(dst_slot.shape) == (num_tokens, num_topk) and dst_slot.dtype == torch.int32 and
-                             dst_slot.is_contiguous(), "cached dst_buffer_slot_idx is int32 [num_tokens, num_topk]")
-                copied_topk_idx = None
-            else:
-                counts = torch.empty(R + 2 * num_experts, **i32)   # one allocation, one D2H copy when syncing
-                psum_rank = counts[:R]
-                psum_expert = counts[R:R + num_experts]
-                num_unaligned = counts[R + num_experts:]
-                dst_slot = torch.empty((num_tokens, num_topk), **i32)
-                copied_topk_idx = torch.empty_like(topk_idx) if do_handle_copy else None
-
-            args = _abi.DispatchArgs()
-
-            args.tuning = _abi.tuning
-            args.payload = payload
-            args.cached = int(cached_mode)
-            args.do_expand = int(do_expand)
-            args.do_zero_padding = int(do_zero_padding)
-            args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
-            args.num_experts, args.num_ranks, args.rank_idx = num_experts, R, self.rank_idx
-            args.num_max_tokens_per_rank = num_max_tokens_per_rank
-            args.expert_alignment = expert_alignment
-            args.x = _abi.ptr(x)
-            args.sf = _abi.ptr(sf)
-            args.sf_token_stride, args.sf_hidden_stride = sf_ts, sf_hs
-            args.num_sf_packs = num_sf_packs
-            args.topk_idx = _abi.ptr(topk_idx)
-            args.topk_weights = _abi.ptr(topk_weights)
-            args.copied_topk_idx = _abi.ptr(copied_topk_idx)
-            args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_rank)
-            args.psum_num_recv_tokens_per_expert = _abi.ptr(psum_expert)
-            args.num_unaligned_recv_tokens_per_expert = _abi.ptr(num_unaligned)
-            args.cumulative_local_expert_recv_stats = _abi.ptr(cumulative_local_expert_recv_stats)
-            args.host_counts = 0
-            args.dst_buffer_slot_idx = _abi.ptr(dst_slot)
-            args.workspace = _abi.ptr(workspace)
-            args.workspace_bytes = workspace.numel()
-            stream_ptr = run_stream.cuda_stream
-
-            # Sizes of the outputs
-            if cached_mode:
-                num_recv_tokens = cached_num_recv_tokens
-                num_expanded_tokens = cached_num_expanded_tokens
-                per_expert_list = list(cached_num_recv_tokens_per_expert_list)
-            elif do_cpu_sync:
-                args.phases = _abi.PHASE_LAYOUT
-                _abi.check(_abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(args), stream_ptr), "dispatch layout")
-                host = counts.cpu()                                  # waits for the layout kernel
-                self._read_and_clear_status("dispatch")
-                num_recv_tokens = int(host[R - 1])
-                unaligned = host[R + num_experts:]
-                aligned = (unaligned + (expert_alignment - 1)) // expert_alignment * expert_alignment
-                per_expert_list = aligned.tolist()
-                num_expanded_tokens = int(aligned.sum())
-            else:
-                num_recv_tokens = num_max_tokens_per_rank * R
-                num_expanded_tokens = num_max_tokens_per_rank * min(num_topk, num_experts) + \
-                    (expert_alignment - 1) * num_experts
-                num_expanded_tokens = _align(num_expanded_tokens, expert_alignment)
-                per_expert_list = []
-
-            num_allocated = num_expanded_tokens if do_expand else num_recv_tokens
-            recv_x = torch.empty((num_allocated, hidden), dtype=out_dtype, device=dev)
-            recv_src_metadata = cached_recv_src_metadata if cached_mode else \
-                torch.empty((num_recv_tokens, num_topk + 2), **i32)
-            recv_sf = None
-            rsf_ts = rsf_hs = 0
-            if sf_dtype is not None:
-                if not use_tma_aligned_col_major_sf:
-                    rsf_ts, rsf_hs = num_sf_packs, 1
+            with torch.cuda.stream(run_stream):
+                if cached_mode:
+                    psum_rank = cached_psum_num_recv_tokens_per_scaleup_rank
+                    psum_expert = cached_psum_num_recv_tokens_per_expert
+                    num_unaligned = cached_num_unaligned_recv_tokens_per_expert
+                    _host_assert(psum_rank.shape == (R,) and psum_rank.dtype == torch.int32 and psum_rank.is_cuda,
+                                 "cached psum per rank is int32 [num_ranks]")
+                    _host_assert(psum_expert.shape == (num_experts,) and psum_expert.dtype == torch.int32,
+                                 "cached psum per expert is int32 [num_experts]")
+                    _host_assert(num_unaligned is not None and num_unaligned.shape == (num_experts,),
+                                 "cached unaligned counts are int32 [num_experts]")
+                    dst_slot = cached_dst_buffer_slot_idx
+                    _host_assert(tuple(dst_slot.shape) == (num_tokens, num_topk) and dst_slot.dtype == torch.int32 and
+                                 dst_slot.is_contiguous(), "cached dst_buffer_slot_idx is int32 [num_tokens, num_topk]")
+                    copied_topk_idx = None
                 else:
-                    rsf_ts, rsf_hs = 1, _align(num_allocated, 4)
-                recv_sf = torch.empty_strided((num_allocated, num_sf_packs), (rsf_ts, rsf_hs), dtype=sf_dtype, device=dev)
-            recv_topk_idx = torch.empty((num_allocated, num_topk), dtype=topk_idx.dtype, device=dev) if not do_expand else None
-            recv_topk_weights = None
-            if topk_weights is not None:
-                recv_topk_weights = torch.empty((num_allocated,) if do_expand else (num_allocated, num_topk),
-                                                dtype=torch.float32, device=dev)
+                    counts = torch.empty(R + 2 * num_experts, **i32)   # one allocation, one D2H copy when syncing
+                    psum_rank = counts[:R]
+                    psum_expert = counts[R:R + num_experts]
+                    num_unaligned = counts[R + num_experts:]
+                    dst_slot = torch.empty((num_tokens, num_topk), **i32)
+                    copied_topk_idx = torch.empty_like(topk_idx) if do_handle_copy else None
 
-            if previous_event_before_epilogue is not None:
-                run_stream.wait_event(previous_event_before_epilogue.event)
+                args = _abi.DispatchArgs()
 
-            args.phases = _abi.PHASE_MOVE if (cached_mode or do_cpu_sync) else (_abi.PHASE_LAYOUT | _abi.PHASE_MOVE)
-            args.recv_src_metadata = _abi.ptr(recv_src_metadata)
-            args.recv_x = _abi.ptr(recv_x)
-            args.recv_sf = _abi.ptr(recv_sf)
-            args.recv_sf_token_stride, args.recv_sf_hidden_stride = rsf_ts, rsf_hs
-            args.recv_topk_idx = _abi.ptr(recv_topk_idx)
-            args.recv_topk_weights = _abi.ptr(recv_topk_weights)
-            args.recv_capacity = recv_src_metadata.shape[0]
-            args.expanded_capacity = num_expanded_tokens if do_expand else 0
-            _abi.check(_abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(args), stream_ptr), "dispatch")
+                args.tuning = _abi.tuning
+                args.payload = payload
+                args.cached = int(cached_mode)
+                args.do_expand = int(do_expand)
+                args.do_zero_padding = int(do_zero_padding)
+                args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
+                args.num_experts, args.num_ranks, args.rank_idx = num_experts, R, self.rank_idx
+                args.num_max_tokens_per_rank = num_max_tokens_per_rank
+                args.expert_alignment = expert_alignment
+                args.x = _abi.ptr(x)
+                args.sf = _abi.ptr(sf)
+                args.sf_token_stride, args.sf_hidden_stride = sf_ts, sf_hs
+                args.num_sf_packs = num_sf_packs
+                args.topk_idx = _abi.ptr(topk_idx)
+                args.topk_weights = _abi.ptr(topk_weights)
+                args.copied_topk_idx = _abi.ptr(copied_topk_idx)
+                args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_rank)
+                args.psum_num_recv_tokens_per_expert = _abi.ptr(psum_expert)
+                args.num_unaligned_recv_tokens_per_expert = _abi.ptr(num_unaligned)
+                args.cumulative_local_expert_recv_stats = _abi.ptr(cumulative_local_expert_recv_stats)
+                args.host_counts = 0
+                args.dst_buffer_slot_idx = _abi.ptr(dst_slot)
+                args.workspace = _abi.ptr(workspace)
+                args.workspace_bytes = workspace.numel()
+                stream_ptr = run_stream.cuda_stream
 
-        event = self._epilogue(
-            [x, sf, topk_idx, topk_weights, recv_x, recv_sf, recv_topk_idx, recv_topk_weights,
-             cumulative_local_expert_recv_stats, copied_topk_idx, psum_rank, psum_expert, num_unaligned,
-             recv_src_metadata, dst_slot, workspace],
-            compute_stream, run_stream, allocate_on_comm_stream, async_with_compute_stream)
+                # Sizes of the outputs
+                if cached_mode:
+                    num_recv_tokens = cached_num_recv_tokens
+                    num_expanded_tokens = cached_num_expanded_tokens
+                    per_expert_list = list(cached_num_recv_tokens_per_expert_list)
+                elif do_cpu_sync:
+                    args.phases = _abi.PHASE_LAYOUT
+                    _abi.check(_abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(args), stream_ptr), "dispatch layout")
+                    host = counts.cpu()                                  # waits for the layout kernel
+                    self._read_and_clear_status("dispatch")
+                    num_recv_tokens = int(host[R - 1])
+                    unaligned = host[R + num_experts:]
+                    aligned = (unaligned + (expert_alignment - 1)) // expert_alignment * expert_alignment
+                    per_expert_list = aligned.tolist()
+                    num_expanded_tokens = int(aligned.sum())
+                else:
+                    num_recv_tokens = num_max_tokens_per_rank * R
+                    num_expanded_tokens = num_max_tokens_per_rank * min(num_topk, num_experts) + \
+                        (expert_alignment - 1) * num_experts
+                    num_expanded_tokens = _align(num_expanded_tokens, expert_alignment)
+                    per_expert_list = []
 
-        return (recv_x, recv_sf, recv_topk_idx, recv_topk_weights, copied_topk_idx,
-                num_recv_tokens, num_expanded_tokens, per_expert_list,
-                psum_rank, psum_expert, num_unaligned, recv_src_metadata, dst_slot,
-                None, None, event)
+                num_allocated = num_expanded_tokens if do_expand else num_recv_tokens
+                recv_x = torch.empty((num_allocated, hidden), dtype=out_dtype, device=dev)
+                recv_src_metadata = cached_recv_src_metadata if cached_mode else \
+                    torch.empty((num_recv_tokens, num_topk + 2), **i32)
+                recv_sf = None
+                rsf_ts = rsf_hs = 0
+                if sf_dtype is not None:
+                    if not use_tma_aligned_col_major_sf:
+                        rsf_ts, rsf_hs = num_sf_packs, 1
+                    else:
+                        rsf_ts, rsf_hs = 1, _align(num_allocated, 4)
+                    recv_sf = torch.empty_strided((num_allocated, num_sf_packs), (rsf_ts, rsf_hs), dtype=sf_dtype, device=dev)
+                recv_topk_idx = torch.empty((num_allocated, num_topk), dtype=topk_idx.dtype, device=dev) if not do_expand else None
+                recv_topk_weights = None
+                if topk_weights is not None:
+                    recv_topk_weights = torch.empty((num_allocated,) if do_expand else (num_allocated, num_topk),
+                                                    dtype=torch.float32, device=dev)
+
+                if previous_event_before_epilogue is not None:
+                    _stream_wait_event(run_stream, previous_event_before_epilogue)
+
+                args.phases = _abi.PHASE_MOVE if (cached_mode or do_cpu_sync) else (_abi.PHASE_LAYOUT | _abi.PHASE_MOVE)
+                args.recv_src_metadata = _abi.ptr(recv_src_metadata)
+                args.recv_x = _abi.ptr(recv_x)
+                args.recv_sf = _abi.ptr(recv_sf)
+                args.recv_sf_token_stride, args.recv_sf_hidden_stride = rsf_ts, rsf_hs
+                args.recv_topk_idx = _abi.ptr(recv_topk_idx)
+                args.recv_topk_weights = _abi.ptr(recv_topk_weights)
+                args.recv_capacity = recv_src_metadata.shape[0]
+                args.expanded_capacity = num_expanded_tokens if do_expand else 0
+                _abi.check(_abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(args), stream_ptr), "dispatch")
+
+            event = self._epilogue(
+                [x, sf, topk_idx, topk_weights, recv_x, recv_sf, recv_topk_idx, recv_topk_weights,
+                 cumulative_local_expert_recv_stats, copied_topk_idx, psum_rank, psum_expert, num_unaligned,
+                 recv_src_metadata, dst_slot, workspace],
+                compute_stream, run_stream, allocate_on_comm_stream, async_with_compute_stream)
+
+            return (recv_x, recv_sf, recv_topk_idx, recv_topk_weights, copied_topk_idx,
+                    num_recv_tokens, num_expanded_tokens, per_expert_list,
+                    psum_rank, psum_expert, num_unaligned, recv_src_metadata, dst_slot,
+                    None, None, event)
+        finally:
+            if allocate_on_comm_stream:
+                torch.cuda.set_stream(compute_stream)
 
     # ---- combine ----
     def combine(self, x: torch.Tensor, topk_weights: Optional[torch.Tensor],
@@ -462,41 +500,45 @@ class ElasticBuffer:
         _host_assert(bias_0 is not None or bias_1 is None, "bias_1 needs bias_0")
 
         compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_with_compute_stream)
-        workspace = self._get_workspace(num_tokens, num_topk, num_experts)
-        with torch.cuda.stream(run_stream):
-            combined_x = torch.empty((num_tokens, hidden), dtype=x.dtype, device=self.device)
-            combined_topk_weights = None
-            if topk_weights is not None:
-                combined_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
-            if previous_event_before_epilogue is not None:
-                run_stream.wait_event(previous_event_before_epilogue.event)
-            args = _abi.CombineArgs()
-            args.tuning = _abi.tuning
-            args.do_expand = int(use_expanded_layout)
-            args.allow_multiple_reduction = int(self.allow_multiple_reduction)
-            args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
-            args.num_experts, args.num_ranks = num_experts, self.num_ranks
-            args.rank_idx, args.num_max_tokens_per_rank = self.rank_idx, num_max_tokens_per_rank
-            args.x = _abi.ptr(x)
-            args.num_x_rows = num_x_rows
-            args.topk_weights = _abi.ptr(topk_weights)
-            args.bias_0, args.bias_1 = _abi.ptr(bias_0), _abi.ptr(bias_1)
-            args.topk_idx = _abi.ptr(combined_topk_idx)
-            args.dst_buffer_slot_idx = _abi.ptr(dst_buffer_slot_idx)
-            args.recv_src_metadata = _abi.ptr(src_metadata)
-            args.num_recv_rows = src_metadata.shape[0]
-            args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_num_recv_tokens_per_scaleup_rank)
-            args.combined_x = _abi.ptr(combined_x)
-            args.combined_topk_weights = _abi.ptr(combined_topk_weights)
-            args.workspace = _abi.ptr(workspace)
-            args.workspace_bytes = workspace.numel()
-            _abi.check(_abi.lib.deep_ep_hip_launch_combine(ctypes.byref(args), run_stream.cuda_stream), "combine")
+        try:
+            workspace = self._get_workspace(run_stream, num_tokens, num_topk, num_experts)
+            with torch.cuda.stream(run_stream):
+                combined_x = torch.empty((num_tokens, hidden), dtype=x.dtype, device=self.device)
+                combined_topk_weights = None
+                if topk_weights is not None:
+                    combined_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
+                if previous_event_before_epilogue is not None:
+                    _stream_wait_event(run_stream, previous_event_before_epilogue)
+                args = _abi.CombineArgs()
+                args.tuning = _abi.tuning
+                args.do_expand = int(use_expanded_layout)
+                args.allow_multiple_reduction = int(self.allow_multiple_reduction)
+                args.num_tokens, args.hidden, args.num_topk = num_tokens, hidden, num_topk
+                args.num_experts, args.num_ranks = num_experts, self.num_ranks
+                args.rank_idx, args.num_max_tokens_per_rank = self.rank_idx, num_max_tokens_per_rank
+                args.x = _abi.ptr(x)
+                args.num_x_rows = num_x_rows
+                args.topk_weights = _abi.ptr(topk_weights)
+                args.bias_0, args.bias_1 = _abi.ptr(bias_0), _abi.ptr(bias_1)
+                args.topk_idx = _abi.ptr(combined_topk_idx)
+                args.dst_buffer_slot_idx = _abi.ptr(dst_buffer_slot_idx)
+                args.recv_src_metadata = _abi.ptr(src_metadata)
+                args.num_recv_rows = src_metadata.shape[0]
+                args.psum_num_recv_tokens_per_rank = _abi.ptr(psum_num_recv_tokens_per_scaleup_rank)
+                args.combined_x = _abi.ptr(combined_x)
+                args.combined_topk_weights = _abi.ptr(combined_topk_weights)
+                args.workspace = _abi.ptr(workspace)
+                args.workspace_bytes = workspace.numel()
+                _abi.check(_abi.lib.deep_ep_hip_launch_combine(ctypes.byref(args), run_stream.cuda_stream), "combine")
 
-        event = self._epilogue(
-            [x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx,
-             psum_num_recv_tokens_per_scaleup_rank, dst_buffer_slot_idx, combined_x, combined_topk_weights, workspace],
-            compute_stream, run_stream, allocate_on_comm_stream, async_with_compute_stream)
-        return combined_x, combined_topk_weights, event
+            event = self._epilogue(
+                [x, topk_weights, bias_0, bias_1, src_metadata, combined_topk_idx,
+                 psum_num_recv_tokens_per_scaleup_rank, dst_buffer_slot_idx, combined_x, combined_topk_weights, workspace],
+                compute_stream, run_stream, allocate_on_comm_stream, async_with_compute_stream)
+            return combined_x, combined_topk_weights, event
+        finally:
+            if allocate_on_comm_stream:
+                torch.cuda.set_stream(compute_stream)
 
     # ---- V1 surface kept on the same runtime ----
     def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
@@ -509,23 +551,27 @@ class ElasticBuffer:
         _host_assert(num_experts > 0 and num_experts % self.num_ranks == 0, "num_experts % num_ranks == 0")
         num_tokens, num_topk = topk_idx.shape
         compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_finish)
-        workspace = self._get_workspace(num_tokens, num_topk, num_experts)
-        with torch.cuda.stream(run_stream):
-            num_tokens_per_rank = torch.empty((self.num_ranks,), dtype=torch.int32, device=self.device)
-            num_tokens_per_expert = torch.empty((num_experts,), dtype=torch.int32, device=self.device)
-            is_token_in_rank = torch.empty((num_tokens, self.num_ranks), dtype=torch.bool, device=self.device)
-            args = _abi.LayoutArgs()
-            args.topk_idx = _abi.ptr(topk_idx)
-            args.num_tokens, args.num_topk, args.num_experts, args.num_ranks = num_tokens, num_topk, num_experts, self.num_ranks
-            args.num_tokens_per_rank = _abi.ptr(num_tokens_per_rank)
-            args.num_tokens_per_expert = _abi.ptr(num_tokens_per_expert)
-            args.is_token_in_rank = _abi.ptr(is_token_in_rank)
-            args.workspace = _abi.ptr(workspace)
-            args.workspace_bytes = workspace.numel()
-            _abi.check(_abi.lib.deep_ep_hip_launch_layout(ctypes.byref(args), run_stream.cuda_stream), "get_dispatch_layout")
-        event = self._epilogue([topk_idx, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, workspace],
-                               compute_stream, run_stream, allocate_on_comm_stream, async_finish)
-        return num_tokens_per_rank, None, num_tokens_per_expert, is_token_in_rank, event
+        try:
+            workspace = self._get_workspace(run_stream, num_tokens, num_topk, num_experts)
+            with torch.cuda.stream(run_stream):
+                num_tokens_per_rank = torch.empty((self.num_ranks,), dtype=torch.int32, device=self.device)
+                num_tokens_per_expert = torch.empty((num_experts,), dtype=torch.int32, device=self.device)
+                is_token_in_rank = torch.empty((num_tokens, self.num_ranks), dtype=torch.bool, device=self.device)
+                args = _abi.LayoutArgs()
+                args.topk_idx = _abi.ptr(topk_idx)
+                args.num_tokens, args.num_topk, args.num_experts, args.num_ranks = num_tokens, num_topk, num_experts, self.num_ranks
+                args.num_tokens_per_rank = _abi.ptr(num_tokens_per_rank)
+                args.num_tokens_per_expert = _abi.ptr(num_tokens_per_expert)
+                args.is_token_in_rank = _abi.ptr(is_token_in_rank)
+                args.workspace = _abi.ptr(workspace)
+                args.workspace_bytes = workspace.numel()
+                _abi.check(_abi.lib.deep_ep_hip_launch_layout(ctypes.byref(args), run_stream.cuda_stream), "get_dispatch_layout")
+            event = self._epilogue([topk_idx, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, workspace],
+                                   compute_stream, run_stream, allocate_on_comm_stream, async_finish)
+            return num_tokens_per_rank, None, num_tokens_per_expert, is_token_in_rank, event
+        finally:
+            if allocate_on_comm_stream:
+                torch.cuda.set_stream(compute_stream)
 
     def intranode_dispatch(self, x: torch.Tensor, x_scales: Optional[torch.Tensor],
                            topk_idx: Optional[torch.Tensor], topk_weights: Optional[torch.Tensor],
@@ -599,85 +645,89 @@ class ElasticBuffer:
             _host_assert(cached_mode or topk_idx is not None, "num_worst_tokens needs the top-k tensors")
 
         compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_finish, v1_rules=True)
-        route_lanes = num_topk if topk_idx is not None else R
-        route_experts = num_experts if topk_idx is not None else R
-        workspace = self._get_workspace(num_tokens, route_lanes, route_experts)
-        per_expert_list: List[int] = []
-        with torch.cuda.stream(run_stream):
-            args = _abi.IntranodeDispatchArgs()
-            args.tuning = _abi.tuning
-            args.payload, args.cached = payload, int(cached_mode)
-            args.num_tokens, args.hidden = num_tokens, hidden
-            args.num_topk, args.num_experts = num_topk, (num_experts if topk_idx is not None else 0)
-            args.num_ranks, args.rank_idx = R, self.rank_idx
-            args.num_channels, args.expert_alignment = num_channels, expert_alignment
-            args.x, args.x_scales = _abi.ptr(x), _abi.ptr(x_scales)
-            args.scale_token_stride, args.scale_hidden_stride, args.num_scales = scale_ts, scale_hs, num_scales
-            args.topk_idx, args.topk_weights = _abi.ptr(topk_idx), _abi.ptr(topk_weights)
-            args.is_token_in_rank = _abi.ptr(is_token_in_rank)
-            args.workspace, args.workspace_bytes = _abi.ptr(workspace), workspace.numel()
-            stream_ptr = run_stream.cuda_stream
+        try:
+            route_lanes = num_topk if topk_idx is not None else R
+            route_experts = num_experts if topk_idx is not None else R
+            workspace = self._get_workspace(run_stream, num_tokens, route_lanes, route_experts)
+            per_expert_list: List[int] = []
+            with torch.cuda.stream(run_stream):
+                args = _abi.IntranodeDispatchArgs()
+                args.tuning = _abi.tuning
+                args.payload, args.cached = payload, int(cached_mode)
+                args.num_tokens, args.hidden = num_tokens, hidden
+                args.num_topk, args.num_experts = num_topk, (num_experts if topk_idx is not None else 0)
+                args.num_ranks, args.rank_idx = R, self.rank_idx
+                args.num_channels, args.expert_alignment = num_channels, expert_alignment
+                args.x, args.x_scales = _abi.ptr(x), _abi.ptr(x_scales)
+                args.scale_token_stride, args.scale_hidden_stride, args.num_scales = scale_ts, scale_hs, num_scales
+                args.topk_idx, args.topk_weights = _abi.ptr(topk_idx), _abi.ptr(topk_weights)
+                args.is_token_in_rank = _abi.ptr(is_token_in_rank)
+                args.workspace, args.workspace_bytes = _abi.ptr(workspace), workspace.numel()
+                stream_ptr = run_stream.cuda_stream
 
-            if cached_mode:
-                num_recv_tokens = cached_num_recv_tokens
-                rank_prefix_matrix, channel_prefix_matrix = cached_rank_prefix_matrix, cached_channel_prefix_matrix
-                recv_channel_prefix_matrix = torch.empty((R, num_channels), **i32)
-                send_head = cached_send_head
-                recv_src_idx = torch.empty((num_recv_tokens,), **i32)
-                args.phases = _abi.PHASE_MOVE
-            else:
-                rank_prefix_matrix = torch.empty((R, R), **i32)
-                channel_prefix_matrix = torch.empty((R, num_channels), **i32)
-                recv_channel_prefix_matrix = torch.empty((R, num_channels), **i32)
-                send_head = torch.empty((num_tokens, R), **i32)
-                counts = torch.empty(R + max(num_experts, 1), **i32)
-                args.rank_prefix_matrix = _abi.ptr(rank_prefix_matrix)
-                args.channel_prefix_matrix = _abi.ptr(channel_prefix_matrix)
-                args.recv_channel_prefix_matrix = _abi.ptr(recv_channel_prefix_matrix)
-                args.psum_num_recv_tokens_per_rank = _abi.ptr(counts)
-                args.num_recv_tokens_per_expert = _abi.ptr(counts[R:]) if topk_idx is not None else 0
-                if num_worst_tokens > 0:
-                    num_recv_tokens = num_worst_tokens
-                    args.phases = _abi.PHASE_LAYOUT | _abi.PHASE_MOVE
-                    args.fill_unused_topk_idx = 1
-                else:
-                    # The reference spins on host-mapped counters here (csrc/legacy/buffer.hpp:580-600)
-                    args.phases = _abi.PHASE_LAYOUT
-                    _abi.check(_abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(args), stream_ptr),
-                               "intranode dispatch layout")
-                    if topk_idx is None:
-                        host = torch.cat([counts[:R], num_tokens_per_expert]).cpu()
-                    else:
-                        host = counts.cpu()
-                        self._read_and_clear_status("dispatch")
-                    num_recv_tokens = int(host[R - 1])
-                    per_expert = host[R:R + num_experts]
-                    per_expert_list = ((per_expert + (expert_alignment - 1)) // expert_alignment * expert_alignment).tolist()
+                if cached_mode:
+                    num_recv_tokens = cached_num_recv_tokens
+                    rank_prefix_matrix, channel_prefix_matrix = cached_rank_prefix_matrix, cached_channel_prefix_matrix
+                    recv_channel_prefix_matrix = torch.empty((R, num_channels), **i32)
+                    send_head = cached_send_head
+                    recv_src_idx = torch.empty((num_recv_tokens,), **i32)
                     args.phases = _abi.PHASE_MOVE
-                recv_src_idx = torch.empty((num_recv_tokens,), **i32)
+                else:
+                    rank_prefix_matrix = torch.empty((R, R), **i32)
+                    channel_prefix_matrix = torch.empty((R, num_channels), **i32)
+                    recv_channel_prefix_matrix = torch.empty((R, num_channels), **i32)
+                    send_head = torch.empty((num_tokens, R), **i32)
+                    counts = torch.empty(R + max(num_experts, 1), **i32)
+                    args.rank_prefix_matrix = _abi.ptr(rank_prefix_matrix)
+                    args.channel_prefix_matrix = _abi.ptr(channel_prefix_matrix)
+                    args.recv_channel_prefix_matrix = _abi.ptr(recv_channel_prefix_matrix)
+                    args.psum_num_recv_tokens_per_rank = _abi.ptr(counts)
+                    args.num_recv_tokens_per_expert = _abi.ptr(counts[R:]) if topk_idx is not None else 0
+                    if num_worst_tokens > 0:
+                        num_recv_tokens = num_worst_tokens
+                        args.phases = _abi.PHASE_LAYOUT | _abi.PHASE_MOVE
+                        args.fill_unused_topk_idx = 1
+                    else:
+                        # The reference spins on host-mapped counters here (csrc/legacy/buffer.hpp:580-600)
+                        args.phases = _abi.PHASE_LAYOUT
+                        _abi.check(_abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(args), stream_ptr),
+                                   "intranode dispatch layout")
+                        if topk_idx is None:
+                            host = torch.cat([counts[:R], num_tokens_per_expert]).cpu()
+                        else:
+                            host = counts.cpu()
+                            self._read_and_clear_status("dispatch")
+                        num_recv_tokens = int(host[R - 1])
+                        per_expert = host[R:R + num_experts]
+                        per_expert_list = ((per_expert + (expert_alignment - 1)) // expert_alignment * expert_alignment).tolist()
+                        args.phases = _abi.PHASE_MOVE
+                    recv_src_idx = torch.empty((num_recv_tokens,), **i32)
 
-            recv_x = torch.empty((num_recv_tokens, hidden), dtype=x.dtype, device=self.device)
-            recv_x_scales = recv_topk_idx = recv_topk_weights = None
-            if topk_idx is not None:
-                recv_topk_idx = torch.empty((num_recv_tokens, num_topk), dtype=topk_idx.dtype, device=self.device)
-                recv_topk_weights = torch.empty((num_recv_tokens, num_topk), dtype=torch.float32, device=self.device)
-            if x_scales is not None:
-                recv_x_scales = torch.empty((num_recv_tokens, num_scales), dtype=x_scales.dtype, device=self.device)
-                args.recv_scale_token_stride, args.recv_scale_hidden_stride = num_scales, 1
-            args.send_head = _abi.ptr(send_head)
-            args.recv_src_idx = _abi.ptr(recv_src_idx)
-            args.recv_x, args.recv_x_scales = _abi.ptr(recv_x), _abi.ptr(recv_x_scales)
-            args.recv_topk_idx, args.recv_topk_weights = _abi.ptr(recv_topk_idx), _abi.ptr(recv_topk_weights)
-            args.recv_capacity = num_recv_tokens
-            _abi.check(_abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(args), stream_ptr), "intranode dispatch")
+                recv_x = torch.empty((num_recv_tokens, hidden), dtype=x.dtype, device=self.device)
+                recv_x_scales = recv_topk_idx = recv_topk_weights = None
+                if topk_idx is not None:
+                    recv_topk_idx = torch.empty((num_recv_tokens, num_topk), dtype=topk_idx.dtype, device=self.device)
+                    recv_topk_weights = torch.empty((num_recv_tokens, num_topk), dtype=torch.float32, device=self.device)
+                if x_scales is not None:
+                    recv_x_scales = torch.empty((num_recv_tokens, num_scales), dtype=x_scales.dtype, device=self.device)
+                    args.recv_scale_token_stride, args.recv_scale_hidden_stride = num_scales, 1
+                args.send_head = _abi.ptr(send_head)
+                args.recv_src_idx = _abi.ptr(recv_src_idx)
+                args.recv_x, args.recv_x_scales = _abi.ptr(recv_x), _abi.ptr(recv_x_scales)
+                args.recv_topk_idx, args.recv_topk_weights = _abi.ptr(recv_topk_idx), _abi.ptr(recv_topk_weights)
+                args.recv_capacity = num_recv_tokens
+                _abi.check(_abi.lib.deep_ep_hip_launch_intranode_dispatch(ctypes.byref(args), stream_ptr), "intranode dispatch")
 
-        event = self._epilogue(
-            [x, x_scales, topk_idx, topk_weights, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
-             rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_x, recv_x_scales, recv_src_idx,
-             recv_topk_idx, recv_topk_weights, send_head, workspace],
-            compute_stream, run_stream, allocate_on_comm_stream, async_finish)
-        return (recv_x, recv_x_scales, recv_topk_idx, recv_topk_weights, per_expert_list, rank_prefix_matrix,
-                channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, send_head, event)
+            event = self._epilogue(
+                [x, x_scales, topk_idx, topk_weights, num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank,
+                 rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_x, recv_x_scales, recv_src_idx,
+                 recv_topk_idx, recv_topk_weights, send_head, workspace],
+                compute_stream, run_stream, allocate_on_comm_stream, async_finish)
+            return (recv_x, recv_x_scales, recv_topk_idx, recv_topk_weights, per_expert_list, rank_prefix_matrix,
+                    channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, send_head, event)
+        finally:
+            if allocate_on_comm_stream:
+                torch.cuda.set_stream(compute_stream)
 
     def intranode_combine(self, x: torch.Tensor, topk_weights: Optional[torch.Tensor],
                           bias_0: Optional[torch.Tensor], bias_1: Optional[torch.Tensor],
@@ -711,27 +761,31 @@ class ElasticBuffer:
         _host_assert(bias_0 is not None or bias_1 is None, "bias_1 needs bias_0")
 
         compute_stream, run_stream = self._prologue(previous_event, allocate_on_comm_stream, async_finish, v1_rules=True)
-        workspace = self._get_workspace(1, 1, R)
-        with torch.cuda.stream(run_stream):
-            recv_x = torch.empty((num_tokens, hidden), dtype=x.dtype, device=self.device)
-            recv_topk_weights = None
-            if topk_weights is not None:
-                recv_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
-            args = _abi.IntranodeCombineArgs()
-            args.tuning = _abi.tuning
-            args.num_tokens, args.hidden, args.num_ranks, args.num_topk = num_tokens, hidden, R, num_topk
-            args.x, args.num_x_rows = _abi.ptr(x), num_x_rows
-            args.topk_weights = _abi.ptr(topk_weights)
-            args.bias_0, args.bias_1 = _abi.ptr(bias_0), _abi.ptr(bias_1)
-            args.send_head = _abi.ptr(send_head)
-            args.combined_x, args.combined_topk_weights = _abi.ptr(recv_x), _abi.ptr(recv_topk_weights)
-            args.workspace, args.workspace_bytes = _abi.ptr(workspace), workspace.numel()
-            _abi.check(_abi.lib.deep_ep_hip_launch_intranode_combine(ctypes.byref(args), run_stream.cuda_stream),
-                       "intranode combine")
-        event = self._epilogue([x, topk_weights, bias_0, bias_1, src_idx, send_head, rank_prefix_matrix,
-                                channel_prefix_matrix, recv_x, recv_topk_weights, workspace],
-                               compute_stream, run_stream, allocate_on_comm_stream, async_finish)
-        return recv_x, recv_topk_weights, event
+        try:
+            workspace = self._get_workspace(run_stream, 1, 1, R)
+            with torch.cuda.stream(run_stream):
+                recv_x = torch.empty((num_tokens, hidden), dtype=x.dtype, device=self.device)
+                recv_topk_weights = None
+                if topk_weights is not None:
+                    recv_topk_weights = torch.empty((num_tokens, num_topk), dtype=torch.float32, device=self.device)
+                args = _abi.IntranodeCombineArgs()
+                args.tuning = _abi.tuning
+                args.num_tokens, args.hidden, args.num_ranks, args.num_topk = num_tokens, hidden, R, num_topk
+                args.x, args.num_x_rows = _abi.ptr(x), num_x_rows
+                args.topk_weights = _abi.ptr(topk_weights)
+                args.bias_0, args.bias_1 = _abi.ptr(bias_0), _abi.ptr(bias_1)
+                args.send_head = _abi.ptr(send_head)
+                args.combined_x, args.combined_topk_weights = _abi.ptr(recv_x), _abi.ptr(recv_topk_weights)
+                args.workspace, args.workspace_bytes = _abi.ptr(workspace), workspace.numel()
+                _abi.check(_abi.lib.deep_ep_hip_launch_intranode_combine(ctypes.byref(args), run_stream.cuda_stream),
+                           "intranode combine")
+            event = self._epilogue([x, topk_weights, bias_0, bias_1, src_idx, send_head, rank_prefix_matrix,
+                                    channel_prefix_matrix, recv_x, recv_topk_weights, workspace],
+                                   compute_stream, run_stream, allocate_on_comm_stream, async_finish)
+            return recv_x, recv_topk_weights, event
+        finally:
+            if allocate_on_comm_stream:
+                torch.cuda.set_stream(compute_stream)
 
 
 class Config:

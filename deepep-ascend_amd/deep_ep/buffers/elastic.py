@@ -14,8 +14,8 @@ from typing import List, Optional, Tuple, Union
 
 import torch
 
-from .. import _C
-from .._C import EventHandle
+from .. import _binding as _C
+from .._binding import EventHandle
 from ..platform import capture_event, unwrap_event
 from ..utils.event import EventOverlap
 from ..utils.semantic import value_or
@@ -129,7 +129,7 @@ class ElasticBuffer:
         self.num_max_tokens_per_rank = num_max_tokens_per_rank
         self.num_allocated_qps = num_allocated_qps
         self.explicitly_destroy = explicitly_destroy
-        self.runtime = _C.ElasticBuffer(self.rank_idx, self.num_ranks, 0, [], num_bytes, num_cpu_bytes,
+        self.runtime = _C.ElasticBuffer(self.rank_idx, self.num_ranks, 0, None, num_bytes, num_cpu_bytes,
                                         allow_hybrid_mode, allow_multiple_reduction, prefer_overlap_with_compute,
                                         sl_idx, num_allocated_qps, num_cpu_timeout_secs, num_gpu_timeout_secs,
                                         explicitly_destroy)
@@ -171,7 +171,10 @@ class ElasticBuffer:
         return capture_event()
 
     def get_comm_stream(self) -> torch.cuda.Stream:
-        return self.runtime.get_comm_stream()
+        ts = self.runtime.get_comm_stream()
+        if isinstance(ts, torch.cuda.Stream):
+            return ts
+        return torch.cuda.Stream(stream_id=ts.stream_id, device_index=ts.device_index, device_type=ts.device_type)
 
     def get_physical_domain_size(self) -> Tuple[int, int]:
         return self.runtime.get_physical_domain_size()
@@ -181,7 +184,7 @@ class ElasticBuffer:
 
     def get_theoretical_num_sms(self, num_experts: int, num_topk: int, *args, **kwargs) -> int:
         """The routing kernels are bandwidth bound and always launched over the whole GPU."""
-        return torch.cuda.get_device_properties(self.runtime.device).multi_processor_count
+        return torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
 
     def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
                             previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
@@ -311,6 +314,4 @@ class ElasticBuffer:
         """Synchronise and raise if a kernel flagged bad routing input (an expert id outside
         [0, num_experts), one expert named twice by a token) or a row that did not fit the outputs.
         Calls with `do_cpu_sync=True` check this themselves."""
-        torch.cuda.synchronize()
-        if self.runtime._workspace is not None:
-            self.runtime._read_and_clear_status("routing")
+        self.runtime.check_device_status("routing")

@@ -22,7 +22,8 @@ from typing import Callable, List, Optional, Tuple, Union
 
 import torch
 
-from .. import _C, _abi
+from .. import _abi, _binding
+from .. import _runtime as _C
 from ..platform import unwrap_event
 from ..utils.event import EventOverlap
 
@@ -54,7 +55,7 @@ class Buffer:
 
     @staticmethod
     def capture() -> EventOverlap:
-        return EventOverlap(_C.EventHandle())
+        return EventOverlap(_binding.EventHandle())
 
     @staticmethod
     def is_sm90_compiled() -> bool:

@@ -2,24 +2,25 @@
 deep_ep/platform.py:9-80, which only knows "cuda" and "ascend")."""
 import torch
 
-from . import _C
+from . import _binding, _runtime
 
 
 def get_platform() -> str:
-    return _C.get_platform()
+    return _binding.get_platform()
 
 
 def is_hip() -> bool:
     return get_platform() == "hip"
 
 
-def capture_event() -> "_C.EventHandle":
-    return _C.EventHandle()
+def capture_event():
+    return _binding.EventHandle()
 
 
 def unwrap_event(event):
     """EventOverlap or EventHandle or None -> EventHandle or None."""
-    return getattr(event, "event", event) if event is not None and not isinstance(event, _C.EventHandle) else event
+    is_handle = isinstance(event, (_binding.EventHandle, _runtime.EventHandle))
+    return getattr(event, "event", event) if event is not None and not is_handle else event
 
 
 def synchronize() -> None:

@@ -5,7 +5,7 @@ from typing import Any, Callable, Optional, Sequence
 
 import torch
 
-from .._C import EventHandle
+from .._binding import EventHandle
 
 
 class EventOverlap:

@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "deep_ep_hip.h")
 
 import deep_ep
-from deep_ep import _C, _abi
+from deep_ep import _C, _abi, _runtime
 
 
 def header_functions():
@@ -183,24 +183,75 @@ def test_no_product_module_touches_the_oracle():
     pkg = os.path.join(ROOT, "deepep-ascend_amd")
     for dirpath, _, files in os.walk(pkg):
         for f in files:
-            if f.endswith((".py", ".hip", ".cuh", ".h", ".cpp")):
+            if f.endswith((".py", ".hip", ".h", ".hpp", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "routing_oracle" not in text and "fp8_ref" not in text and "/oracle" not in text, f
 
 
 # ---- Python surface (names and signatures of the reference: deep_ep/__init__.py:92-109,
 # deep_ep/buffers/elastic.py:331-349,1391-1412,1616-1626; binding contract tests/platform/api_contract.py:1-42)
+# The reference's binding contract (tests/platform/api_contract.py:1-42): names every platform's `_C` has, and what
+# this platform adds (the Ascend build adds `is_destroyed` in the same way).
+COMMON_MODULE_NAMES = {"get_platform", "topk_idx_t", "EventHandle", "ElasticBuffer", "calculate_elastic_buffer_size"}
+COMMON_BUFFER_METHODS = {"destroy", "get_comm_stream", "get_physical_domain_size", "get_logical_domain_size", "barrier",
+                         "dispatch", "combine"}
+HIP_ONLY_MODULE_NAMES = {"EPException", "get_elastic_buffer_alignment", "set_tuning", "get_tuning", "abi_version"}
+HIP_ONLY_BUFFER_METHODS = {"is_destroyed", "get_dispatch_layout", "check_device_status", "device_status",
+                           "workspace_control_words"}
+
+
+def _public(obj):
+    return {n for n in dir(obj) if not n.startswith("_")}
+
+
+def test_compiled_extension_has_exactly_the_contract_names():
+    """`deep_ep._C` is the compiled extension (csrc/host/binding.cpp), loaded by file like the reference's contract
+    test loads a built extension; its public names are the common contract plus this platform's additions."""
+    assert _C.__file__.endswith(".so") and deep_ep._binding.name == "pybind" and deep_ep._binding.compiled is _C
+    assert _C.get_platform() == "hip" and deep_ep.platform.get_platform() == "hip"
+    assert _C.topk_idx_t == torch.int64 == deep_ep.topk_idx_t
+    assert _public(_C) == COMMON_MODULE_NAMES | HIP_ONLY_MODULE_NAMES
+    assert _public(_C.ElasticBuffer) == COMMON_BUFFER_METHODS | HIP_ONLY_BUFFER_METHODS
+    assert _public(_C.EventHandle) == {"current_stream_wait"} and hasattr(_C.EventHandle, "__copy__")
+    assert _C.abi_version() == _abi.ABI_VERSION
+    with pytest.raises(RuntimeError):          # host checks surface as RuntimeError (exception.cuh:11-34)
+        _C.calculate_elastic_buffer_size(8, 0, 7168, 8, False, True, True)
+    with pytest.raises(TypeError):             # the 14-argument constructor of binding.hpp:24-27
+        _C.ElasticBuffer(0, 8)
+    _C.set_tuning("cast_pairs", 4)
+    assert _C.get_tuning("cast_pairs") == 4
+    _C.set_tuning("cast_pairs", 0)
+    with pytest.raises(RuntimeError):
+        _C.set_tuning("no_such_knob", 1)
+
+
+def test_ctypes_binding_can_be_selected():
+    env = dict(os.environ, DEEP_EP_HIP_BINDING="ctypes", PYTHONPATH=os.path.join(ROOT, "deepep-ascend_amd"))
+    code = "import deep_ep; print(deep_ep._binding.name, deep_ep.EventHandle.__module__)"
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True)
+    assert res.returncode == 0 and res.stdout.split() == ["ctypes", "deep_ep._runtime"], res.stderr
+
+
 def test_module_surface():
     for name in ("ElasticBuffer", "EPHandle", "EventOverlap", "EventHandle", "Buffer", "topk_idx_t", "__version__"):
         assert hasattr(deep_ep, name)
     assert deep_ep.topk_idx_t == torch.int64
-    for name in ("get_platform", "topk_idx_t", "EventHandle", "ElasticBuffer", "calculate_elastic_buffer_size"):
-        assert hasattr(_C, name)
-    assert _C.get_platform() == "hip"
-    for m in ("destroy", "get_comm_stream", "get_physical_domain_size", "get_logical_domain_size", "barrier", "dispatch", "combine"):
-        assert callable(getattr(_C.ElasticBuffer, m))
-    assert callable(_C.EventHandle.current_stream_wait) and hasattr(_C.EventHandle, "__copy__")
-    assert hasattr(_C.ElasticBuffer, "cpu_comm_t")
+    for runtime in (_C, _runtime):
+        assert COMMON_MODULE_NAMES <= _public(runtime)
+        assert runtime.get_platform() == "hip"
+        assert COMMON_BUFFER_METHODS <= _public(runtime.ElasticBuffer)
+        assert callable(runtime.EventHandle.current_stream_wait) and hasattr(runtime.EventHandle, "__copy__")
+    assert hasattr(_runtime.ElasticBuffer, "cpu_comm_t")
+
+
+def test_tuning_reaches_both_runtimes():
+    deep_ep.tuning.combine_vecs = 4
+    try:
+        assert _abi.tuning.combine_vecs == 4 and _C.get_tuning("combine_vecs") == 4 and deep_ep.tuning.combine_vecs == 4
+    finally:
+        deep_ep.tuning.combine_vecs = 0
+    with pytest.raises(AttributeError):
+        deep_ep.tuning.no_such_knob = 1
 
 
 def _params(fn):
@@ -238,13 +289,18 @@ def test_signatures_are_drop_in():
                                                 "async_finish", "allocate_on_comm_stream"]
     assert _params(deep_ep.Buffer.combine) == ["x", "handle", "topk_weights", "bias", "config", "previous_event",
                                                "async_finish", "allocate_on_comm_stream"]
-    assert len(_params(_C.ElasticBuffer.intranode_dispatch)) == 17           # the binding's 16 + cached_send_head
-    assert len(_params(_C.ElasticBuffer.intranode_combine)) == 12
+    assert len(_params(_runtime.ElasticBuffer.intranode_dispatch)) == 17     # the binding's 16 + cached_send_head
+    assert len(_params(_runtime.ElasticBuffer.intranode_combine)) == 12
     assert deep_ep.Buffer.is_sm90_compiled() and deep_ep.Config(20, 6, 256).num_sms == 20
-    # the runtime keeps the positional order of the compiled binding (29 dispatch / 18 combine arguments, then extensions)
-    assert len(_params(_C.ElasticBuffer.dispatch)) == 30 and _params(_C.ElasticBuffer.dispatch)[-1] == "cast_to_fp8"
-    assert len(_params(_C.ElasticBuffer.combine)) == 19 and _params(_C.ElasticBuffer.combine)[-1] == "dst_buffer_slot_idx"
-    assert len(_params(_C.ElasticBuffer.__init__)) == 14
+    # the Python runtime keeps the positional order of the compiled binding (29 dispatch / 18 combine arguments, then
+    # extensions); pybind prints the compiled signatures into the docstrings
+    R = _runtime.ElasticBuffer
+    assert len(_params(R.dispatch)) == 30 and _params(R.dispatch)[-1] == "cast_to_fp8"
+    assert len(_params(R.combine)) == 19 and _params(R.combine)[-1] == "dst_buffer_slot_idx"
+    assert len(_params(R.__init__)) == 14
+    assert _C.ElasticBuffer.dispatch.__doc__.split("->")[0].count("arg") == 30
+    assert _C.ElasticBuffer.combine.__doc__.split("->")[0].count("arg") == 19
+    assert _C.ElasticBuffer.__init__.__doc__.split("->")[0].count("arg") == 14
 
 
 def test_handle_fields():
@@ -261,11 +317,12 @@ def test_handle_fields():
 def test_buffer_size_calculus_worked_numbers():
     # T=8192 per rank, H=7168, K=8, R=8 (Appendix A of the reference's calculus): BF16 904 MiB, FP8 max(512, 900) MiB
     mib = 1 << 20
-    assert _C.calculate_elastic_buffer_size(8, 8192, 7168, 8, False, True, True) == 904 * mib
-    assert _C.calculate_elastic_buffer_size(8, 8192, 7168, 8, True, True, True) == 900 * mib
-    assert _C.calculate_elastic_buffer_size(8, 128, 1024, 0, False, True, True) % _C.get_elastic_buffer_alignment() == 0
-    with pytest.raises(RuntimeError):
-        _C.calculate_elastic_buffer_size(8, 0, 7168, 8, False, True, True)
+    for rt in (_C, _runtime):
+        assert rt.calculate_elastic_buffer_size(8, 8192, 7168, 8, False, True, True) == 904 * mib
+        assert rt.calculate_elastic_buffer_size(8, 8192, 7168, 8, True, True, True) == 900 * mib
+        assert rt.calculate_elastic_buffer_size(8, 128, 1024, 0, False, True, True) % rt.get_elastic_buffer_alignment() == 0
+        with pytest.raises(RuntimeError):
+            rt.calculate_elastic_buffer_size(8, 0, 7168, 8, False, True, True)
     g = deep_ep.LogicalGroup(3, 8)
     assert (g.rank(), g.size()) == (3, 8)
     assert deep_ep.ElasticBuffer.get_buffer_size_hint(g, 8192, 7168, 8) == 904 * mib

@@ -15,9 +15,7 @@ FUSED = ["C1", "C2", "tiny_masked", "one_token", "k1_e_eq_r", "ragged_chunks", "
 
 
 def _control_words(buf):
-    from deep_ep import _abi
-    n = _abi.lib.deep_ep_hip_workspace_control_bytes()
-    words = buf.runtime._workspace[:n].view(torch.int32).cpu().clone()
+    words = buf.runtime.workspace_control_words().clone()
     words[2:4] = 0          # the two row totals a dispatch leaves for the kernels that follow it
     return words
 

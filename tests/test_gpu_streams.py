@@ -123,3 +123,75 @@ def test_host_argument_errors():
     # the buffer still works after the rejected inputs
     rx, _, _, _, _ = buf.dispatch(x, idx, w, num_experts=case.E)
     assert rx.shape[0] == oracle.dispatch(case.x, case.topk_idx, case.topk_weights, case.E, case.R, 0, case.M).num_recv_tokens
+
+
+def test_calls_on_two_streams_share_the_workspace_in_order():
+    """An asynchronous dispatch on the communication stream that nobody has waited for yet, followed at once by plain
+    calls on the compute stream with other routing: the buffer's workspace (positions, tables, gates) is shared, so the
+    second call has to queue behind the first by itself.  Both results are checked against the oracle."""
+    a = rc.small("two_streams_a", 3000, 1024, 64, 8, 8, seed=61, masked_ratio=0.05)
+    b = rc.small("two_streams_b", 2900, 1024, 64, 8, 8, seed=62, masked_ratio=0.3)
+    b.M = a.M
+    buf = _buf(a)
+    ref_a = oracle.dispatch(a.x, a.topk_idx, a.topk_weights, a.E, a.R, 0, a.M)
+    ref_b = oracle.dispatch(b.x, b.topk_idx, b.topk_weights, b.E, b.R, 0, b.M)
+    xa, ia, wa = a.x.cuda(), a.topk_idx.cuda(), a.topk_weights.cuda()
+    xb, ib, wb = b.x.cuda(), b.topk_idx.cuda(), b.topk_weights.cuda()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        ra, ria, rwa, ha, ev = buf.dispatch(xa, ia, wa, num_experts=a.E, do_cpu_sync=False, async_with_compute_stream=True)
+        rb, rib, rwb, hb, _ = buf.dispatch(xb, ib, wb, num_experts=b.E, do_cpu_sync=False)          # compute stream, no wait
+        per_rank, _, per_expert, _, _ = buf.get_dispatch_layout(ia, a.E)                            # and a layout call on top
+        ev.current_stream_wait()
+        torch.cuda.synchronize()
+        assert_equal(ra[:ref_a.num_recv_tokens], ref_a.recv_x, "recv_x of the asynchronous call")
+        assert_equal(ha.dst_buffer_slot_idx, ref_a.dst_buffer_slot_idx, "slots of the asynchronous call")
+        assert_equal(rb[:ref_b.num_recv_tokens], ref_b.recv_x, "recv_x of the call that followed")
+        assert_equal(hb.dst_buffer_slot_idx, ref_b.dst_buffer_slot_idx, "slots of the call that followed")
+        assert_equal(per_expert, oracle.layout(a.topk_idx, a.E, a.R)[1], "layout counts")
+    buf.check_device_status()
+
+
+def test_current_stream_is_restored_when_a_call_fails():
+    case = rc.small("restore", 64, 256, 8, 2, 2, seed=63)
+    buf = _buf(case)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    before = torch.cuda.current_stream()
+    with pytest.raises(RuntimeError):
+        buf.dispatch(x, idx, w, num_experts=case.E, num_max_tokens_per_rank=4, allocate_on_comm_stream=True,
+                     previous_event=buf.capture(), async_with_compute_stream=True)
+    bad = idx.clone()
+    bad[0, 0] = case.E + 1
+    with pytest.raises(RuntimeError, match="expert id"):
+        buf.dispatch(x, bad, w, num_experts=case.E, allocate_on_comm_stream=True, previous_event=buf.capture(),
+                     async_with_compute_stream=True)
+    assert torch.cuda.current_stream() == before
+
+
+def test_previous_event_before_epilogue_orders_the_move_phase():
+    """`previous_event_before_epilogue` (csrc/elastic/buffer.hpp:528-586): the launches that write the outputs wait for
+    an event recorded behind work on another stream - here the producer of the tensor a cached dispatch moves."""
+    case = rc.small("before_epilogue", 2000, 2048, 32, 4, 4, seed=64)
+    buf = _buf(case)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    _, _, _, handle, _ = buf.dispatch(x, idx, w, num_experts=case.E)
+    ref = oracle.dispatch(case.x * 2, case.topk_idx, case.topk_weights, case.E, case.R, 0, case.M)
+    side = torch.cuda.Stream()
+    x2 = torch.empty_like(x)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        filler = torch.ones(1 << 24, device="cuda").cumsum(0)          # keeps the side stream busy first
+        torch.mul(x, 2, out=x2)
+        produced = buf.capture()
+    recv_x, _, _, _, event = buf.dispatch(x2, topk_weights=w, handle=handle, previous_event=buf.capture(),
+                                          previous_event_before_epilogue=produced, async_with_compute_stream=True,
+                                          allocate_on_comm_stream=True)
+    event.current_stream_wait()
+    assert_equal(recv_x, ref.recv_x, "recv_x moved after the producer finished")
+    out, _, ev2 = buf.combine(recv_x, handle, previous_event=buf.capture(), previous_event_before_epilogue=produced,
+                              async_with_compute_stream=True, allocate_on_comm_stream=True)
+    ev2.current_stream_wait()
+    ref_out, _ = oracle.combine(ref.recv_x, case.topk_idx, ref.recv_src_metadata, ref.dst_buffer_slot_idx,
+                                ref.psum_num_recv_tokens_per_scaleup_rank, case.E, case.R, 0, case.M)
+    assert_equal(out + 0.0, ref_out + 0.0, "combined_x")
+    assert float(filler[-1]) == float(1 << 24)

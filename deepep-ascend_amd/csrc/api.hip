@@ -683,6 +683,7 @@ int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* a, void* st
     REQUIRE(a->x != nullptr && a->topk_idx != nullptr && a->topk_weights != nullptr &&
             a->packed_recv_src_info != nullptr && a->packed_recv_layout_range != nullptr && a->combined_x != nullptr, "NULL tensor");
     REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
+    REQUIRE(!a->use_logfmt || a->hidden % 512 == 0, "use_logfmt needs hidden %% 512 == 0 (got %d)", a->hidden);
     LLCombineParams p{};
     p.S = a->num_src_ranks; p.src_rank_begin = a->src_rank_begin; p.src_token_stride = a->src_token_stride;
     p.num_tokens_per_src = a->num_tokens_per_src;
@@ -698,6 +699,7 @@ int deep_ep_hip_launch_ll_combine(const deep_ep_hip_ll_combine_args* a, void* st
     p.out = static_cast<uint8_t*>(a->combined_x);
     p.status = reinterpret_cast<int32_t*>(a->workspace);
     p.vecs = a->tuning.ll_combine_vecs;
+    p.use_logfmt = a->use_logfmt ? 1 : 0;
     hipError_t err = launch_ll_combine(p, static_cast<hipStream_t>(stream));
     if (err != hipSuccess) return hip_fail(err, "low-latency combine launch");
     return DEEP_EP_HIP_OK;

@@ -244,6 +244,7 @@ struct LLCombineParams {
     uint8_t* out;
     int32_t* status;
     int vecs;                    // forced column tile, 0 = choose
+    int use_logfmt;              // gathered rows pass through the LogFMT-10 codec
 };
 
 hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream);

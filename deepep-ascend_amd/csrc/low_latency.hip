@@ -357,8 +357,59 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
 }
 
-// Weighted reduce: one wavefront per (token, column tile of kVecs * 512 channels).
-template <int kVecs>
+// ---- LogFMT-10, the codec the reference puts the rows of a low-latency combine through on the wire
+// (csrc/kernels/legacy/internode_ll.cu:556-637 encode, :640-712 and :1048-1100 decode).  On one GPU nothing travels,
+// so the row is encoded and decoded in registers: what is accumulated is what the receiver would have decoded.
+//
+// Per group of 128 channels: amax and amin of |x|; log_amin = max(log2(amin), log_amax - 32).  A chunk of rows
+// (1024 channels, or 512 when hidden is not a multiple of 1024: what one warp of the reference's send loop stages)
+// is cast iff every one of its groups has log_amax < 0 and log_amin < log_amax.  A cast value becomes a sign and a
+// 9-bit code on a logarithmic grid with step = (log_amax - log_amin) / 510:
+//   code = floor(max(log2|x| / step + rounding - log_amin / step, 0)),  rounding = 2 - log2((1 + 2^step) / 2) / step
+//   decoded = code == 0 ? 0 : 2^((code - 1) * step + log_amin)
+// log2 / exp2 are the hardware's (v_log_f32 / v_exp_f32), as the reference uses its hardware's approximations.
+
+// One 16-byte vector (8 BF16 channels per lane, 64 lanes = 512 channels = 4 groups of 16 lanes) of a row.
+struct LogFmtGroup {
+    float log_amax, log_amin;
+    bool castable;
+};
+
+__device__ __forceinline__ LogFmtGroup logfmt_group_of(const float (&mag)[8]) {
+    float amax = 0.f, amin = __builtin_inff();
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        amax = fmaxf(amax, mag[c]);
+        amin = fminf(amin, mag[c]);
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {        // the 16 lanes of a 128-channel group
+        amax = fmaxf(amax, __shfl_xor(amax, off, kWaveSize));
+        amin = fminf(amin, __shfl_xor(amin, off, kWaveSize));
+    }
+    LogFmtGroup g;
+    g.log_amax = __builtin_amdgcn_logf(amax);
+    g.log_amin = amin == 0.f ? g.log_amax - 32.f : fmaxf(__builtin_amdgcn_logf(amin), g.log_amax - 32.f);
+    g.castable = g.log_amax < 0.f && g.log_amin < g.log_amax;
+    return g;
+}
+
+__device__ __forceinline__ void logfmt_round_trip(float (&val)[8], const float (&mag)[8], const LogFmtGroup& g) {
+    const float step = (g.log_amax - g.log_amin) / 510.f;
+    const float step_inv = 1.0f / step;
+    const float rounding = 2.0f - __builtin_amdgcn_logf((1.0f + __builtin_amdgcn_exp2f(step)) * 0.5f) * step_inv;
+    const float fused_rounding = rounding - g.log_amin * step_inv;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const uint32_t code = uint32_t(fmaxf(__builtin_amdgcn_logf(mag[c]) * step_inv + fused_rounding, 0.f));     // round down
+        const float decoded = code == 0u ? 0.f : __builtin_amdgcn_exp2f(float(code - 1u) * step + g.log_amin);
+        val[c] = val[c] < 0.f ? -decoded : decoded;       // a negative zero has magnitude 0: code 0 either way
+    }
+}
+
+// Weighted reduce: one wavefront per (token, column tile of kVecs * 512 channels).  kLogFmt: the tile is one chunk
+// of the codec (kVecs = 2 for hidden % 1024 == 0, else 1).
+template <int kVecs, bool kLogFmt = false>
 __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombineParams p, const int tiles) {
     const int lane = threadIdx.x & 63;
     const unsigned work = wave_work_index(blockIdx.x, kMoveWaves);
@@ -449,15 +500,39 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
         const int64_t row = int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j);
         const float wj = read_lane(w, j);
         const uint8_t* src = p.x + row * row_bytes;
+        if constexpr (kLogFmt) {
+            // hidden % (kVecs * 512) == 0: every lane of the tile holds channels of the row
+            float val[kVecs][8], mag[kVecs][8];
+            LogFmtGroup group[kVecs];
+            bool chunk_castable = true;
 #pragma unroll
-        for (int i = 0; i < kVecs; ++i) {
-            const int off = (tile * kVecs + i) * 1024 + lane * 16;
-            if (off < row_bytes) {
-                const vec16 v = load16_stream(src + off);
-                acc[i][0] += bf16_lo(v.x) * wj; acc[i][1] += bf16_hi(v.x) * wj;
-                acc[i][2] += bf16_lo(v.y) * wj; acc[i][3] += bf16_hi(v.y) * wj;
-                acc[i][4] += bf16_lo(v.z) * wj; acc[i][5] += bf16_hi(v.z) * wj;
-                acc[i][6] += bf16_lo(v.w) * wj; acc[i][7] += bf16_hi(v.w) * wj;
+            for (int i = 0; i < kVecs; ++i) {
+                const vec16 v = load16_stream(src + (tile * kVecs + i) * 1024 + lane * 16);
+                val[i][0] = bf16_lo(v.x); val[i][1] = bf16_hi(v.x); val[i][2] = bf16_lo(v.y); val[i][3] = bf16_hi(v.y);
+                val[i][4] = bf16_lo(v.z); val[i][5] = bf16_hi(v.z); val[i][6] = bf16_lo(v.w); val[i][7] = bf16_hi(v.w);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) mag[i][c] = fabsf(val[i][c]);
+                group[i] = logfmt_group_of(mag[i]);
+                chunk_castable = chunk_castable && group[i].castable;
+            }
+            chunk_castable = __ballot(!chunk_castable) == 0ull;          // every group of the chunk
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                if (chunk_castable) logfmt_round_trip(val[i], mag[i], group[i]);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) acc[i][c] += val[i][c] * wj;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                const int off = (tile * kVecs + i) * 1024 + lane * 16;
+                if (off < row_bytes) {
+                    const vec16 v = load16_stream(src + off);
+                    acc[i][0] += bf16_lo(v.x) * wj; acc[i][1] += bf16_hi(v.x) * wj;
+                    acc[i][2] += bf16_lo(v.y) * wj; acc[i][3] += bf16_hi(v.y) * wj;
+                    acc[i][4] += bf16_lo(v.z) * wj; acc[i][5] += bf16_hi(v.z) * wj;
+                    acc[i][6] += bf16_lo(v.w) * wj; acc[i][7] += bf16_hi(v.w) * wj;
+                }
             }
         }
     }
@@ -544,9 +619,15 @@ hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream) {
     int vecs = p.vecs;
     if (vecs != 1 && vecs != 2 && vecs != 4)
         vecs = (p.H * 2 <= 1024 || int64_t(p.S) * p.src_token_stride <= 4096) ? 1 : 4;   // decode sizes: many small wavefronts
+    if (p.use_logfmt) vecs = p.H % 1024 == 0 ? 2 : 1;                                     // one codec chunk per wavefront
     const int tiles = (p.H * 2 + vecs * 1024 - 1) / (vecs * 1024);
     const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
     const unsigned blocks = unsigned((waves + kMoveWaves - 1) / kMoveWaves);
+    if (p.use_logfmt) {
+        if (vecs == 2) hipLaunchKernelGGL((ll_combine_kernel<2, true>), dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+        else hipLaunchKernelGGL((ll_combine_kernel<1, true>), dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+        return hipGetLastError();
+    }
     if (vecs == 1) hipLaunchKernelGGL(ll_combine_kernel<1>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
     else if (vecs == 2) hipLaunchKernelGGL(ll_combine_kernel<2>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
     else hipLaunchKernelGGL(ll_combine_kernel<4>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);

@@ -205,6 +205,7 @@ class LLCombineArgs(Structure):
     _fields_ = [
         ("num_src_ranks", c_int32), ("src_rank_begin", c_int32),
         ("src_token_stride", c_int32),
+        ("use_logfmt", c_int32),
         ("num_tokens_per_src", c_void_p),
         ("hidden", c_int32), ("num_topk", c_int32), ("num_experts", c_int32),
         ("expert_begin", c_int32), ("num_local_experts", c_int32), ("num_ranks", c_int32),

@@ -301,12 +301,13 @@ class Buffer:
         order and in fp32, `weight * row` over its lanes whose expert lives on this rank, then rounds once to
         BF16.  Returns (combined_x, event, hook); `hook` is a no-op callable with `return_recv_hook`, else None.
         With `zero_copy` the rows are read from `get_next_low_latency_combine_buffer(handle)` instead of `x`.
-        `use_logfmt` is refused: LogFMT-10 is a wire format for rows in flight between GPUs
-        (csrc/kernels/legacy/internode_ll.cu:556-712); nothing is in flight here, and its encode/decode is built on
-        the approximate log2/exp2 instructions of another vendor's hardware, so its rounding cannot be reproduced.
+        `use_logfmt`: every row passes through the LogFMT-10 codec before it is accumulated (the reference compresses
+        the rows it sends this way, csrc/kernels/legacy/internode_ll.cu:556-712): chunks of 1024 channels (512 if hidden
+        is not a multiple of 1024) whose 128-channel groups all have amax < 1 come back as 9-bit logarithmic codes,
+        the others unchanged.  Needs hidden % 512 == 0 and excludes `zero_copy` (internode_ll.cu:1182).
         """
-        if use_logfmt:
-            raise NotImplementedError('LogFMT combine is a transport codec; the one-GPU HIP backend has no transport')
+        if use_logfmt and zero_copy:
+            raise RuntimeError('Assertion failed: not (zero_copy and use_logfmt)')
         assert not (return_recv_hook and async_finish), 'a receive hook and `async_finish` exclude each other'
         src_info, layout_range, M, H, num_experts = handle
         if zero_copy:
@@ -337,6 +338,7 @@ class Buffer:
                 args = _abi.LLCombineArgs()
                 args.tuning = _abi.tuning
                 args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
+                args.use_logfmt = int(use_logfmt)
                 args.num_tokens_per_src = 0
                 args.hidden, args.num_topk, args.num_experts = H, K, num_experts
                 args.expert_begin, args.num_local_experts, args.num_ranks = self.rank * E_l, E_l, R

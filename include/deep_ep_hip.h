@@ -29,7 +29,7 @@
  *   deep_ep_hip_launch_intranode_combine   csrc/kernels/legacy/intranode.cu:700-1095 (combine), called from
  *                                   csrc/legacy/buffer.hpp:719-860
  *   deep_ep_hip_launch_ll_dispatch  csrc/kernels/legacy/internode_ll.cu:464-554
- *   deep_ep_hip_launch_ll_combine   csrc/kernels/legacy/internode_ll.cu:1140-1238
+ *   deep_ep_hip_launch_ll_combine   csrc/kernels/legacy/internode_ll.cu:1140-1238 (LogFMT-10: :556-712, :1048-1100)
  *   deep_ep_hip_launch_cast_fp8     deep_ep/utils/math.py:30-39 (per_token_cast_to_fp8)
  */
 #ifndef DEEP_EP_HIP_H_
@@ -339,6 +339,12 @@ int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* args, voi
 typedef struct {
     int32_t num_src_ranks, src_rank_begin;  /* source ranks whose tokens are rebuilt in this launch */
     int32_t src_token_stride;           /* rows of topk_idx / topk_weights / combined_x per source rank */
+    int32_t use_logfmt;                 /* 1: every gathered row passes through the LogFMT-10 codec before it is
+                                           accumulated (what the reference's rows go through on the wire): per chunk
+                                           of 1024 channels (512 if hidden % 1024 != 0), if every 128-channel group has
+                                           amax < 1 and amin < amax, magnitudes become 9-bit codes on a logarithmic
+                                           grid between the group's amin (at most 2^32 below amax) and amax, and are
+                                           decoded again; other chunks stay BF16.  Needs hidden % 512 == 0. */
     const int32_t* num_tokens_per_src;  /* [num_src_ranks] device, or NULL = src_token_stride each */
     int32_t hidden, num_topk, num_experts;
     int32_t expert_begin, num_local_experts, num_ranks;

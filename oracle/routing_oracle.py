@@ -34,6 +34,9 @@ Each function names the reference source it restates (paths relative to the refe
                             rank order, fp32, one rounding; top-k weights summed over the same rows)
   ll_dispatch()             csrc/legacy/buffer.hpp:1515-1541 + csrc/kernels/legacy/internode_ll.cu:361-461
   ll_combine()              csrc/kernels/legacy/internode_ll.cu:1072-1135 (BF16 branch :704-711)
+  logfmt10_round_trip()     csrc/kernels/legacy/internode_ll.cu:556-637 (encode), :640-712 (decode): pinned in
+                            tests/test_oracle_logfmt.py by what the grid construction fixes (a cast value decodes to
+                            the nearest grid point, amax and amin survive, error bound, chunk rules, special cases)
 
 Pinning status (which independent evidence fixes each function) is listed in tests/test_oracle_*.py:
 layout -> brute force + literal cases; FP8 cast -> C software e4m3 encoder (oracle/fp8_ref.c) +
@@ -483,14 +486,51 @@ def ll_dispatch(xs: Sequence[torch.Tensor], topk_idxs: Sequence[torch.Tensor],
     return px, ps, cnt, src_info, layout_range
 
 
+def logfmt10_round_trip(x: torch.Tensor) -> torch.Tensor:
+    """What a receiver decodes from rows sent through the LogFMT-10 codec of the reference's low-latency combine
+    (csrc/kernels/legacy/internode_ll.cu:556-637 encode, :640-712 decode, chunking :754-756 and :876-885), with exact
+    log2 / exp2 in fp64 where the reference uses its hardware's approximations.
+
+    x: bf16 [..., H], H % 512 == 0.  Returns fp32 of the same shape.  Per group of 128 channels: amax, amin of |x|;
+    log_amin = max(log2(amin), log_amax - 32) (amin == 0: log_amax - 32).  A chunk (1024 channels when H % 1024 == 0,
+    else 512: what one warp of the send loop stages) is cast iff every group in it has log_amax < 0 and
+    log_amin < log_amax; other chunks pass unchanged.  Cast value: sign and
+    code = floor(max(log2|x| / step + rounding - log_amin / step, 0)) with step = (log_amax - log_amin) / 510 and
+    rounding = 2 - log2((1 + 2^step) / 2) / step; decoded = 0 for code 0, else 2^((code - 1) * step + log_amin).
+    """
+    import numpy as np
+    assert x.dtype == torch.bfloat16 and x.shape[-1] % 512 == 0
+    H = x.shape[-1]
+    chunk_groups = (1024 if H % 1024 == 0 else 512) // 128
+    v = x.to(torch.float64).numpy().reshape(-1, H // 128, 128)
+    mag = np.abs(v)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        amax, amin = mag.max(axis=2), mag.min(axis=2)
+        log_amax = np.log2(amax)
+        log_amin = np.where(amin == 0, log_amax - 32.0, np.maximum(np.log2(amin), log_amax - 32.0))
+        castable = (log_amax < 0) & (log_amin < log_amax)
+        chunk_ok = castable.reshape(castable.shape[0], -1, chunk_groups).all(axis=2, keepdims=True)
+        chunk_ok = np.broadcast_to(chunk_ok, (castable.shape[0], castable.shape[1] // chunk_groups, chunk_groups)).reshape(castable.shape)
+        step = ((log_amax - log_amin) / 510.0)[:, :, None]
+        step_inv = 1.0 / step
+        rounding = 2.0 - np.log2((1.0 + np.exp2(step)) * 0.5) * step_inv
+        fused = rounding - log_amin[:, :, None] * step_inv
+        code = np.floor(np.maximum(np.log2(mag) * step_inv + fused, 0.0))
+        decoded = np.where(code == 0, 0.0, np.exp2((code - 1.0) * step + log_amin[:, :, None]))
+    decoded = np.where(np.signbit(v), -decoded, decoded)
+    out = np.where(chunk_ok[:, :, None], decoded, v)
+    return torch.from_numpy(out.reshape(x.shape).astype(np.float32))
+
+
 def ll_combine(x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
                src_info: torch.Tensor, layout_range: torch.Tensor, src_rank: int,
-               num_experts: int, num_ranks: int, dst_rank: int) -> torch.Tensor:
+               num_experts: int, num_ranks: int, dst_rank: int, use_logfmt: bool = False) -> torch.Tensor:
     """Weighted reduce back to source rank `src_rank`'s token order.
 
     x is [E_l, R*M, H] bf16 held by `dst_rank`.  out[t] = bf16( sum over lanes k in order with
     topk_idx[t,k] on dst_rank of  w[t,k] * float(x[e_local, row(t,k)]) ), accumulated with
     separate fp32 multiply and add.  Lanes routed to other ranks contribute nothing here.
+    With use_logfmt every row first passes through logfmt10_round_trip.
     """
     T, K = topk_idx.shape
     E_l = num_experts // num_ranks
@@ -510,7 +550,8 @@ def ll_combine(x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tens
                 continue
             le = e - dst_rank * E_l
             r = row_of[(le, t)]
-            out[t] = out[t] + x[le, r].to(torch.float32) * topk_weights[t, k]
+            row = logfmt10_round_trip(x[le, r]) if use_logfmt else x[le, r].to(torch.float32)
+            out[t] = out[t] + row * topk_weights[t, k]
     return out.to(torch.bfloat16)
 
 

@@ -123,8 +123,8 @@ def test_ll_power_of_two_scales_hooks_and_zero_copy(R, T, H, E, K, M, use_ue8m0)
     out_b, _, hook_b = buf.low_latency_combine(torch.empty_like(y), idx.cuda(), w.cuda(), handle, zero_copy=True)
     assert hook_b is None
     assert_equal(out_a, out_b, "zero-copy combine")
-    with pytest.raises(NotImplementedError):
-        buf.low_latency_combine(y, idx.cuda(), w.cuda(), handle, use_logfmt=True)
+    with pytest.raises(RuntimeError):           # the codec and zero-copy exclude each other (internode_ll.cu:1182)
+        buf.low_latency_combine(y, idx.cuda(), w.cuda(), handle, use_logfmt=True, zero_copy=True)
 
 
 def test_ll_empty_and_unrouted_tokens():
@@ -143,3 +143,52 @@ def test_ll_empty_and_unrouted_tokens():
         y = torch.ones((E // R, R * M, H), dtype=torch.bfloat16, device="cuda")
         out, _, _ = buf.low_latency_combine(y, idx, w, handle)
         assert out.shape == (T, H) and bool((out == 0).all())
+
+
+def _calc_diff(a, b):
+    a, b = a.double(), b.double()
+    return float(1 - 2 * (a * b).sum() / ((a * a).sum() + (b * b).sum()))
+
+
+@pytest.mark.parametrize("hidden", [7168, 1536])           # chunks of 1024 channels / of 512 channels
+def test_low_latency_combine_with_logfmt(hidden):
+    """`use_logfmt=True` (csrc/kernels/legacy/internode_ll.cu:556-712): rows pass through the LogFMT-10 codec before the
+    weighted reduce.  Against the oracle's codec (exact log2 / exp2 in fp64; the kernel uses the hardware's, as the
+    reference uses its hardware's): the reference's own bar calc_diff < 9e-4 against the exact result
+    (tests/legacy/test_low_latency.py:178-181), near bit-equality with the oracle, and bit-equality where the codec
+    must leave rows alone."""
+    import deep_ep
+    R, T, E, K, M = 4, 96, 32, 6, 128
+    x, idx, w = rc.c5_sources(seed=91, R=R, T=T, H=hidden, E=E, K=K)
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(1, R), low_latency_mode=True)
+    _, count, handle, _, _ = buf.low_latency_dispatch(x.cuda(), idx.cuda(), M, E, use_fp8=False)
+    _, _, ref_cnt, ref_info, ref_range = oracle.ll_dispatch(list(x), list(idx), M, E, R, 1, False)
+    g = torch.Generator().manual_seed(92)
+    y = (torch.randn((E // R, R * M, hidden), generator=g) * 0.1).to(torch.bfloat16)      # expert outputs: mostly below 1
+    y[0, :, :1024] = (torch.randn((R * M, 1024), generator=g) * 3).to(torch.bfloat16)      # a chunk the codec leaves alone
+    y[1, :, 0:128] = 0.25                                                                  # a single-magnitude group
+    out_q, _, _ = buf.low_latency_combine(y.cuda(), idx.cuda(), w.cuda(), handle, use_logfmt=True)
+    out_x, _, _ = buf.low_latency_combine(y.cuda(), idx.cuda(), w.cuda(), handle, use_logfmt=False)
+    assert not torch.isnan(out_q).any()
+    total, same = 0, 0
+    for s in range(R):
+        ref_q = oracle.ll_combine(y, idx[s], w[s], ref_info, ref_range, s, E, R, 1, use_logfmt=True)
+        ref_x = oracle.ll_combine(y, idx[s], w[s], ref_info, ref_range, s, E, R, 1)
+        assert_equal(out_x[s] + 0.0, ref_x + 0.0, f"plain combine of source {s}")
+        got = out_q[s].cpu()
+        assert _calc_diff(got, ref_x) < 9e-4, "the reference's acceptance bar"
+        assert _calc_diff(got, ref_q) < 1e-7, "against the oracle's codec"
+        same += int((got.view(torch.int16) == ref_q.view(torch.int16)).sum())
+        total += got.numel()
+        # tokens whose only rows on this rank (experts [E/R, 2E/R)) come from its first expert read, in their first
+        # chunk, values of magnitude >= 1: there the codec must hand the rows through unchanged
+        first = E // R
+        elsewhere = (idx[s] < first) | (idx[s] >= 2 * first)
+        tokens = ((idx[s] == first) | elsewhere).all(dim=1)
+        chunk = 1024 if hidden % 1024 == 0 else 512
+        assert_equal(out_q[s].cpu()[tokens][:, :chunk] + 0.0, out_x[s].cpu()[tokens][:, :chunk] + 0.0,
+                     "chunks the codec must not touch")
+    assert same / total > 0.999, f"only {same / total:.5f} of the outputs equal the oracle's bit for bit"
+    assert _calc_diff(out_q.cpu(), out_x.cpu()) > 1e-9, "the codec did nothing"
+    with pytest.raises(RuntimeError):
+        buf.low_latency_combine(y.cuda(), idx.cuda(), w.cuda(), handle, use_logfmt=True, zero_copy=True)

@@ -200,7 +200,8 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
         REQUIRE((int64_t(H) * elem_in) % 16 == 0, "a row of x must be a multiple of 16 bytes (hidden %d, %d-byte elements)", H, elem_in);
         REQUIRE(int64_t(H) * elem_in < (int64_t(1) << 30), "row too large");
         REQUIRE(T == 0 || a->x != nullptr, "x is NULL");
-        REQUIRE(a->recv_x != nullptr || (a->recv_capacity == 0 && a->expanded_capacity == 0), "recv_x is NULL");
+        const bool no_rows = a->recv_capacity == 0 && a->expanded_capacity == 0;     // empty outputs have no storage
+        REQUIRE(a->recv_x != nullptr || no_rows, "recv_x is NULL");
         REQUIRE(a->recv_src_metadata != nullptr || a->recv_capacity == 0, "recv_src_metadata is NULL");
         REQUIRE(a->dst_buffer_slot_idx != nullptr || T == 0, "dst_buffer_slot_idx is NULL");
         REQUIRE(a->recv_capacity >= 0 && a->expanded_capacity >= 0, "negative capacity");
@@ -209,12 +210,13 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
             REQUIRE(a->num_sf_packs == 0 && a->sf == nullptr && a->recv_sf == nullptr, "a BF16 payload carries no scale factors");
         if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8) {
             REQUIRE(a->num_sf_packs >= 0, "num_sf_packs must be >= 0");
-            REQUIRE(a->num_sf_packs == 0 || (a->sf != nullptr && a->recv_sf != nullptr) || T == 0, "sf / recv_sf is NULL");
+            REQUIRE(a->num_sf_packs == 0 || a->sf != nullptr || T == 0, "sf is NULL");
+            REQUIRE(a->num_sf_packs == 0 || a->recv_sf != nullptr || no_rows, "recv_sf is NULL");
         }
         if (a->payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
             REQUIRE(H % 128 == 0, "the fused FP8 cast needs hidden %% 128 == 0 (got %d)", H);
             REQUIRE(a->num_sf_packs == H / 128, "num_sf_packs must be hidden / 128 for the fused cast");
-            REQUIRE(a->recv_sf != nullptr || T == 0, "recv_sf is NULL");
+            REQUIRE(a->recv_sf != nullptr || no_rows, "recv_sf is NULL");
         }
         REQUIRE(!(a->do_expand == 0 && a->recv_topk_idx == nullptr && a->recv_capacity > 0), "recv_topk_idx is NULL");
     }

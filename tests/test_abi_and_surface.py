@@ -92,6 +92,18 @@ def _dispatch_args(**kw):
     (dict(phases=_abi.PHASE_MOVE, hidden=100, payload=_abi.PAYLOAD_FP8), "16 bytes"),
     (dict(phases=_abi.PHASE_MOVE, hidden=192, payload=_abi.PAYLOAD_CAST_FP8, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000,
           dst_buffer_slot_idx=0x1000), "128"),
+    # a BF16 payload carries no scale factors: neither tensor nor pack count may be set
+    (dict(phases=_abi.PHASE_MOVE, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000, dst_buffer_slot_idx=0x1000, sf=0x1000),
+     "no scale factors"),
+    (dict(phases=_abi.PHASE_MOVE, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000, dst_buffer_slot_idx=0x1000, recv_sf=0x1000),
+     "no scale factors"),
+    (dict(phases=_abi.PHASE_MOVE, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000, dst_buffer_slot_idx=0x1000, num_sf_packs=2),
+     "no scale factors"),
+    # FP8 rows with scale-factor packs need both scale-factor tensors, unless the outputs are empty
+    (dict(phases=_abi.PHASE_MOVE, payload=_abi.PAYLOAD_FP8, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000,
+          dst_buffer_slot_idx=0x1000, num_sf_packs=2, recv_sf=0x1000, recv_capacity=4), "sf is NULL"),
+    (dict(phases=_abi.PHASE_MOVE, payload=_abi.PAYLOAD_FP8, x=0x1000, recv_x=0x1000, recv_src_metadata=0x1000,
+          dst_buffer_slot_idx=0x1000, num_sf_packs=2, sf=0x1000, recv_capacity=4), "recv_sf is NULL"),
 ])
 def test_dispatch_rejects_bad_arguments_before_launch(kw, fragment):
     rc = _abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(_dispatch_args(**kw)), None)

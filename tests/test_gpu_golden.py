@@ -119,3 +119,37 @@ def test_combine_known_answers():
     y = torch.tensor(fx["contributions"]).to(torch.bfloat16).view(2, 1).expand(2, 8).contiguous()
     out, _, _ = buf.combine(y.cuda(), handle)
     assert out.cpu().float()[0].tolist() == [fx["expected"]] * 8
+
+
+@pytest.mark.parametrize("name", list(G["cached_cases"]))
+def test_cached_handle_moves_a_changed_payload(name):
+    """The reference's cached cases: a second dispatch through the first call's handle, with every payload value
+    raised by 300 and every weight negated, must route the new values exactly as the first call routed the old."""
+    case = G["cached_cases"][name]
+    K = len(case["routes"][0][0])
+    do_expand, A = case.get("do_expand", False), case.get("expert_alignment", 1)
+    zero_pad = case.get("do_zero_padding", False)
+    buf = _buffer()
+
+    def stacked(payloads, weights):
+        x4, idx, w = world.stack_world(payloads, case["routes"], weights, M, H, K)
+        return torch.cat([x4, x4], dim=1).contiguous(), idx, w
+
+    x1, idx, w1 = stacked(case["payloads"], case["weights"])
+    x2, _, w2 = stacked(case["second_payloads"], case["second_weights"])
+    first_x, _, first_w, handle, _ = buf.dispatch(x1.cuda(), idx.cuda(), w1.cuda(), num_experts=E, expert_alignment=A,
+                                                  do_expand=do_expand, do_zero_padding=zero_pad)
+    recv_x, recv_idx, recv_w, same, _ = buf.dispatch(x2.cuda(), topk_weights=w2.cuda(), handle=handle, do_expand=do_expand,
+                                                     do_zero_padding=zero_pad)
+    assert same is handle, "the cached dispatch replaced its handle"
+    for x, w, got_x, got_w in ((x1, w1, first_x, first_w), (x2, w2, recv_x, recv_w)):
+        ref = oracle.dispatch(x, idx, w, E, R, 0, R * M, expert_alignment=A, do_expand=do_expand)
+        n = ref.num_expanded_tokens if do_expand else ref.num_recv_tokens
+        assert_equal(got_x[:n], ref.recv_x, "recv_x")                       # zero padding: padding rows are zero in both
+        assert_equal(got_w[:n], ref.recv_topk_weights, "recv_topk_weights")
+    assert not torch.equal(first_x.cpu(), recv_x.cpu()[:first_x.shape[0]]), "the cached dispatch ignored the new payload"
+    assert not torch.equal(first_w.cpu(), recv_w.cpu()[:first_w.shape[0]]), "the cached dispatch ignored the new weights"
+    if do_expand:
+        # rank 0 hosts experts 0 and 1: 5 + 1 rows padded to 8 + 4; rank 1 hosts 2 and 3: 1 + 1 rows padded to 4 + 4
+        assert handle.num_recv_tokens_per_expert_list == [8, 4, 4, 4]
+    buf.check_device_status()

@@ -259,3 +259,22 @@ def test_dispatch_without_cpu_sync(name, cast):
                                 ref.psum_num_recv_tokens_per_scaleup_rank, case.E, case.R, case.R - 1, case.M)
     assert_equal(out + 0.0, ref_out + 0.0, "combined_x")
     buf.check_device_status()
+
+
+@pytest.mark.parametrize("hidden", [192, 7232, 128, 8, 1000])
+@pytest.mark.parametrize("tokens", [1, 77])
+def test_standalone_cast_with_a_ragged_last_group(hidden, tokens):
+    """per_token_cast_to_fp8 when hidden is not a multiple of 128 (192 = 1.5 groups, 7232 = 56.5 groups): the last
+    group takes its amax over the channels that exist, and the round trip restores BF16 within FP8's resolution."""
+    from deep_ep.utils.math import per_token_cast_back, per_token_cast_to_fp8
+    g = torch.Generator().manual_seed(hidden + tokens)
+    x = (torch.randn((tokens, hidden), generator=g) * torch.rand((tokens, 1), generator=g) * 8).to(torch.bfloat16)
+    x[0, -1] = 300.0          # the largest value of its row sits in the ragged tail
+    q, s = per_token_cast_to_fp8(x.cuda())
+    q_ref, s_ref = oracle.per_token_cast_to_fp8(x)
+    assert q.shape == (tokens, hidden) and s.shape == (tokens, (hidden + 127) // 128)
+    assert_equal(q, q_ref, "fp8 payload")
+    assert_equal(s, s_ref, "scales")
+    back = per_token_cast_back(q, s)
+    assert_equal(back, oracle.per_token_cast_back(q_ref, s_ref), "cast back")
+    assert float((back.float().cpu() - x.float()).abs().max()) <= 300.0 / 16      # e4m3: 3 mantissa bits

@@ -59,7 +59,7 @@ def main():
     ap.add_argument("--launches", type=int, default=0, choices=[0, 1, 2],
                     help="dispatch: 0 library's choice (single launch), 1 single launch even where it does not pay, 2 layout kernel + move kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="tokens the CPU baseline runs over (0: all of the workload)")
     ap.add_argument("--routing", default="case", choices=["case", "sequential"],
                     help="sequential: every token goes to ranks 0..4 (dest rows of consecutive tokens are adjacent)")
     ap.add_argument("--stream-yardsticks", action="store_true",
@@ -281,12 +281,7 @@ def main():
     }
 
     if args.calibration_copy:
-        a = torch.ones(256 * 1024 * 1024, dtype=torch.float32, device=dev)
-        b = torch.empty_like(a)
-        for _ in range(3):
-            torch.mul(a, 1.0, out=b)      # reads 2^30 bytes, writes 2^30 bytes
-        torch.cuda.synchronize()
-        del a, b
+        calibration_copy(torch, dev)
 
     if args.stream_yardsticks:
         result["stream_yardsticks_gbs"] = stream_yardsticks(torch, dev)
@@ -294,6 +289,16 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens, fp8, expanded)
     print(json.dumps(result))
+
+
+def calibration_copy(torch, dev):
+    """A plain elementwise kernel of known size (reads 2^30 bytes, writes 2^30 bytes): what a byte counter reads for
+    it fixes the counter's scale."""
+    a = torch.ones(256 * 1024 * 1024, dtype=torch.float32, device=dev)
+    b = torch.empty_like(a)
+    for _ in range(3):
+        torch.mul(a, 1.0, out=b)
+    torch.cuda.synchronize()
 
 
 def stream_yardsticks(torch, dev, iters=10):
@@ -388,14 +393,56 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     d_us, c_us = timed(dispatch, max(args.steps, 20)), timed(combine, max(args.steps, 20))
     d_bytes = R * T * H * 2 + R * T * K * 8 + n_e * (H + (H // 128) * 4 + 4) + E_l * (4 + R * 8)
     c_bytes = n_e * H * 2 + R * T * K * 12 + R * T * H * 2
-    return {"metric": "low-latency dispatch+combine us/call, 8 sources x 128 tokens x 7168, top-8 of 256, destination rank 0",
+    if args.calibration_copy:
+        calibration_copy(torch, dev)
+    result = {"metric": "low-latency dispatch+combine us/call, 8 sources x 128 tokens x 7168, top-8 of 256, destination rank 0",
             "value": round(step_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(step_us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
             "dtype": "fp8_e4m3 dispatch / bf16 weighted combine", "data": "synthetic",
             "config": {"workload": f"C5: R={R} T={T} H={H} E={E} K={K} M={M}, rows on rank 0: {n_e}"},
             "us_per_call": {"ll_dispatch": round(d_us, 2), "ll_combine": round(c_us, 2)},
             "achieved_gbs": {"ll_dispatch": round(d_bytes / d_us * 1e-3, 1), "ll_combine": round(c_bytes / c_us * 1e-3, 1)},
-            "algorithmic_bytes": {"ll_dispatch": d_bytes, "ll_combine": c_bytes}}
+            "algorithmic_bytes": {"ll_dispatch": d_bytes, "ll_combine": c_bytes},
+            "roofline": {"kernel": "ll_fused_kernel", "bound": "hbm", "achieved": round(d_bytes / d_us * 1e-3, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(d_bytes / d_us * 1e-3 / HBM_PEAK_GBS, 4),
+                         "traffic": MEASURED_TRAFFIC_BYTES.get(("C5", "packed", "fp8", "ll_dispatch"))},
+            "roofline_combine": {"kernel": "ll_combine_kernel", "bound": "hbm", "achieved": round(c_bytes / c_us * 1e-3, 1),
+                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(c_bytes / c_us * 1e-3 / HBM_PEAK_GBS, 4),
+                                 "traffic": MEASURED_TRAFFIC_BYTES.get(("C5", "packed", "fp8", "ll_combine"))}}
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_low_latency(x_cpu, idx_cpu, w_cpu, R, M, E)
+    return result
+
+
+def cpu_baseline_low_latency(x, idx, w, R, M, E):
+    """The CPU oracle on the whole low-latency workload: what destination rank 0 receives from the R source ranks
+    (FP8 cast + packed scatter), then the weighted combine back to every source rank."""
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import routing_oracle as oracle
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    E_l, H = E // R, x.shape[2]
+    y = torch.zeros((E_l, R * M, H), dtype=torch.bfloat16)
+
+    def one_pass():
+        _, _, _, info, ranges = oracle.ll_dispatch(list(x), list(idx), M, E, R, 0)
+        for s in range(R):
+            oracle.ll_combine(y, idx[s], w[s], info, ranges, s, E, R, 0)
+
+    one_pass()   # warm-up
+    iters, t0 = 0, time.perf_counter()
+    while True:
+        one_pass()
+        iters += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed > 10.0 or iters >= 10:
+            break
+    per_pass = elapsed / iters
+    return {"value": round(per_pass * 1e6, 1), "unit": "us", "cores": cores, "kind": "port",
+            "sample": f"the whole workload ({R} sources x {x.shape[1]} tokens), 1 warm-up + {iters} timed passes of "
+                      f"ll_dispatch + ll_combine for every source (torch CPU, eager)"}
 
 
 def cpu_baseline(case, sample_tokens, fp8, expanded):
@@ -407,7 +454,7 @@ def cpu_baseline(case, sample_tokens, fp8, expanded):
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    n = min(sample_tokens, case.T)
+    n = case.T if sample_tokens <= 0 else min(sample_tokens, case.T)
     x, idx, w = case.x[:n].contiguous(), case.topk_idx[:n].contiguous(), case.topk_weights[:n].contiguous()
     T, H, K, E, R = n, case.H, case.K, case.E, case.R
 
@@ -427,7 +474,7 @@ def cpu_baseline(case, sample_tokens, fp8, expanded):
         one_pass()
         iters += 1
         elapsed = time.perf_counter() - t0
-        if elapsed > 10.0 or iters >= 5:
+        if elapsed > 10.0 or iters >= 2:
             break
     per_pass = elapsed / iters
     valid = idx >= 0
@@ -436,7 +483,7 @@ def cpu_baseline(case, sample_tokens, fp8, expanded):
     ab = algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=fp8, expanded=expanded)
     total = ab["layout"] + ab["dispatch"] + ab["combine"]
     return {"value": round(total / per_pass * 1e-9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"first {n} of {case.T} tokens of the same workload, 1 warm-up + {iters} timed passes of "
+            "sample": f"{'all' if n == case.T else 'first ' + str(n) + ' of'} {case.T} tokens of the same workload, 1 warm-up + {iters} timed passes of "
                       f"layout+dispatch+combine (torch CPU, eager), {per_pass * 1e3:.1f} ms/pass",
             "ms_per_pass": round(per_pass * 1e3, 2)}
 

@@ -140,6 +140,22 @@ __global__ void clear_words_kernel(uint32_t* words, size_t n) {
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) words[i] = 0u;
 }
 
+// The status word as memory has it (past every cache between the kernels that OR into it and this read), stored so
+// that a host polling pinned memory sees it.  A clearing read swaps the word with zero and, if a single-launch dispatch
+// had given up, zeroes the bookkeeping words that launch left mid-protocol.
+__global__ void read_status_kernel(int32_t* status, int32_t* out, int clear, uint32_t* control, int control_words) {
+    __shared__ int32_t seen;
+    if (threadIdx.x == 0) {
+        const int32_t v = clear ? __hip_atomic_exchange(status, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                : __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(out, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        seen = v;
+    }
+    __syncthreads();
+    if (clear && (seen & DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT))
+        for (int i = threadIdx.x; i < control_words; i += blockDim.x) store_agent(reinterpret_cast<int*>(control) + i, 0);
+}
+
 // Device address of `scratch` on the current device.  First use on a device resolves the address and clears the
 // bookkeeping words with a small kernel on `stream` (no memset: the call may be under graph capture).
 int static_workspace(hipStream_t stream, void** out) {
@@ -326,6 +342,20 @@ size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_exp
 size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
 
 size_t deep_ep_hip_workspace_control_bytes(void) { return make_workspace_layout(1, 1, 1, 1).expert_start; }
+
+int deep_ep_hip_read_status(void* workspace, int32_t* status_out, int clear, void* stream) {
+    REQUIRE(status_out != nullptr, "status_out is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (workspace == nullptr)
+        if (int rc = static_workspace(s, &workspace)) return rc;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const WorkspaceLayout w = make_workspace_layout(1, 1, 1, 1);
+    hipLaunchKernelGGL(read_status_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<int32_t*>(ws + w.status), status_out,
+                       clear, reinterpret_cast<uint32_t*>(ws), static_cast<int>(w.expert_start / 4));
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return hip_fail(err, "launching the status read");
+    return DEEP_EP_HIP_OK;
+}
 
 int deep_ep_hip_launch_layout(const deep_ep_hip_layout_args* a, void* stream) {
     REQUIRE(a != nullptr, "args is NULL");

@@ -64,6 +64,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     cls.def("is_destroyed", &deep_ep::hip::ElasticBuffer::is_destroyed)
         .def("get_dispatch_layout", &deep_ep::hip::ElasticBuffer::get_dispatch_layout)
         .def("check_device_status", &deep_ep::hip::ElasticBuffer::check_device_status, py::arg("what") = "routing")
+        .def("queue_status_read", &deep_ep::hip::ElasticBuffer::queue_status_read, py::arg("out"), py::arg("clear") = true)
+        .def("poll_device_status", &deep_ep::hip::ElasticBuffer::poll_device_status, py::arg("what") = "routing")
         .def("device_status", &deep_ep::hip::ElasticBuffer::device_status)
         .def("workspace_control_words", &deep_ep::hip::ElasticBuffer::workspace_control_words);
     m.def("get_elastic_buffer_alignment", []() { return deep_ep::hip::kBufferAlignmentBytes; });

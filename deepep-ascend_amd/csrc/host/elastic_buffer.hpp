@@ -120,6 +120,7 @@ public:
         EP_HIP_HOST_ASSERT(not destroyed_);
         c10::hip::device_synchronize();
         workspace_.reset();
+        status_read_.reset();
         destroyed_ = true;
     }
 
@@ -503,6 +504,38 @@ public:
         if (workspace_.has_value()) read_and_clear_status(*workspace_, what.c_str());
     }
 
+    // Queues, on the current stream, a copy of the status word into `out` (one int32 in pinned host memory or on the
+    // device), clearing it on the way if asked.  Capturable: a graph that holds it refreshes `out` on every replay.
+    void queue_status_read(const torch::Tensor& out, bool clear) {
+        EP_HIP_HOST_ASSERT(out.scalar_type() == torch::kInt32 and out.numel() >= 1 and (out.is_cuda() or out.is_pinned()));
+        EP_HIP_HOST_ASSERT(workspace_.has_value());                    // a dispatch or combine has run on this buffer
+        const Stream stream = current_stream();
+        if (last_stream_ != stream) stream_wait(stream, last_stream_);
+        check_abi(deep_ep_hip_read_status(workspace_->data_ptr(), out.data_ptr<int32_t>(), clear ? 1 : 0, stream.stream()),
+                  "status read");
+    }
+
+    // The status check of a loop that never waits for the GPU.  A call that finds no read in flight queues one on the
+    // current stream (deep_ep_hip_read_status in its clearing form: a small kernel moves the status word into pinned
+    // host memory and leaves the workspace ready for the next launch) and returns false.  A later call returns false
+    // while that read is still running; once it has finished, the call throws like check_device_status if a kernel had
+    // flagged something since the previous read, and returns true if nothing was flagged.
+    bool poll_device_status(const std::string& what) {
+        if (not workspace_.has_value()) return true;
+        if (not status_read_.has_value()) {
+            if (not status_host_.has_value())
+                status_host_ = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
+            queue_status_read(*status_host_, true);
+            status_read_.emplace(current_stream());
+            return false;
+        }
+        if (not status_read_->event->query()) return false;
+        status_read_.reset();
+        const int status = *status_host_->data_ptr<int32_t>();
+        if (status != 0) throw_status(status, what.c_str());
+        return true;
+    }
+
     // The status word as the GPU has it now (every launch queued so far has finished): 0 = nothing flagged.
     int device_status() {
         c10::hip::device_synchronize();
@@ -600,6 +633,10 @@ private:
         if (status == 0) return;
         // also the launch bookkeeping words that follow: a dispatch that gave up has left them mid-protocol
         workspace.slice(0, 0, static_cast<int64_t>(deep_ep_hip_workspace_control_bytes())).zero_();
+        throw_status(status, what);
+    }
+
+    [[noreturn]] static void throw_status(int status, const char* what) {
         std::string reasons;
         auto add = [&](int bit, const char* text) {
             if (status & bit) reasons += (reasons.empty() ? "" : "; ") + std::string(text);
@@ -621,6 +658,8 @@ private:
     Stream last_stream_;                     // stream of the last launch that used the workspace
     torch::Device device_ = torch::Device(torch::kCUDA, 0);
     std::optional<torch::Tensor> workspace_;
+    std::optional<torch::Tensor> status_host_;        // one pinned int32: where poll_device_status has the status copied
+    std::optional<EventHandle> status_read_;          // recorded after the read in flight
 };
 
 }  // namespace deep_ep::hip

@@ -125,6 +125,8 @@ class ElasticBuffer:
         self.comm_stream = torch.cuda.Stream(device=self.device)
         self._workspace: Optional[torch.Tensor] = None
         self._last_stream: Optional[torch.cuda.Stream] = None      # stream of the last launch that used the workspace
+        self._status_host: Optional[torch.Tensor] = None           # one pinned int32: where poll_device_status has the status copied
+        self._status_read: Optional[torch.cuda.Event] = None       # recorded after the status read in flight
         self._destroyed = False
 
     # ---- lifetime ----
@@ -133,6 +135,7 @@ class ElasticBuffer:
         _host_assert(not self._destroyed, "not destroyed")
         torch.cuda.synchronize(self.device)
         self._workspace = None
+        self._status_read = None
         self._destroyed = True
 
     def is_destroyed(self) -> bool:
@@ -182,6 +185,42 @@ class ElasticBuffer:
         if self._workspace is not None:
             self._read_and_clear_status(what)
 
+    def queue_status_read(self, out: torch.Tensor, clear: bool = True) -> None:
+        """Queues, on the current stream, a copy of the status word into `out` (one int32 in pinned host memory or on
+        the device), clearing it on the way if asked.  Capturable: a graph that holds it refreshes `out` on every
+        replay."""
+        _host_assert(out.dtype == torch.int32 and out.numel() >= 1 and (out.is_cuda or out.is_pinned()), "out: int32, pinned or on the device")
+        _host_assert(self._workspace is not None, "a dispatch or combine has run on this buffer")
+        stream = torch.cuda.current_stream()
+        if self._last_stream is not None and self._last_stream != stream:
+            stream.wait_stream(self._last_stream)
+        _abi.check(_abi.lib.deep_ep_hip_read_status(self._workspace.data_ptr(), out.data_ptr(), int(clear), stream.cuda_stream),
+                   "status read")
+
+    def poll_device_status(self, what: str = "routing") -> bool:
+        """The status check of a loop that never waits for the GPU.  A call that finds no read in flight queues one on
+        the current stream (deep_ep_hip_read_status in its clearing form: a small kernel moves the status word into
+        pinned host memory and leaves the workspace ready for the next launch) and returns False.  A later call
+        returns False while that read is still running; once it has finished, the call raises like
+        check_device_status if a kernel had flagged something since the previous read, and returns True if nothing
+        was flagged."""
+        if self._workspace is None:
+            return True
+        if self._status_read is None:
+            if self._status_host is None:
+                self._status_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+            self.queue_status_read(self._status_host, True)
+            self._status_read = torch.cuda.Event()
+            self._status_read.record(torch.cuda.current_stream())
+            return False
+        if not self._status_read.query():
+            return False
+        self._status_read = None
+        status = int(self._status_host[0])
+        if status != 0:
+            self._raise_status(status, what)
+        return True
+
     def workspace_control_words(self) -> torch.Tensor:
         """The bookkeeping words at the head of the workspace (status, launch protocol), copied to the host after a full
         synchronisation: between launches everything but the status word and the two row totals reads zero."""
@@ -196,21 +235,24 @@ class ElasticBuffer:
         return 0 if self._workspace is None else int(self._workspace[:4].view(torch.int32).item())
 
     def _read_and_clear_status(self, what: str) -> None:
-        ws = self._workspace
-        status = int(ws[:4].view(torch.int32).item())
+        status = int(self._workspace[:4].view(torch.int32).item())
         if status != 0:
             # also the launch bookkeeping words that follow: a dispatch that gave up has left them mid-protocol
-            ws[:_abi.lib.deep_ep_hip_workspace_control_bytes()].zero_()
-            reasons = []
-            if status & _abi.STATUS_EXPERT_OUT_OF_RANGE:
-                reasons.append("topk_idx holds an expert id >= num_experts")
-            if status & _abi.STATUS_DUPLICATE_EXPERT:
-                reasons.append("a token selects the same expert twice")
-            if status & _abi.STATUS_ROW_OVERFLOW:
-                reasons.append("a received row did not fit the output tensors")
-            if status & _abi.STATUS_LAYOUT_TIMEOUT:
-                reasons.append("a single-launch dispatch gave up waiting for its counting workgroups (outputs invalid)")
-            raise RuntimeError(f"DeepEP HIP backend: {what}: " + "; ".join(reasons))
+            self._workspace[:_abi.lib.deep_ep_hip_workspace_control_bytes()].zero_()
+            self._raise_status(status, what)
+
+    @staticmethod
+    def _raise_status(status: int, what: str) -> None:
+        reasons = []
+        if status & _abi.STATUS_EXPERT_OUT_OF_RANGE:
+            reasons.append("topk_idx holds an expert id >= num_experts")
+        if status & _abi.STATUS_DUPLICATE_EXPERT:
+            reasons.append("a token selects the same expert twice")
+        if status & _abi.STATUS_ROW_OVERFLOW:
+            reasons.append("a received row did not fit the output tensors")
+        if status & _abi.STATUS_LAYOUT_TIMEOUT:
+            reasons.append("a single-launch dispatch gave up waiting for its counting workgroups (outputs invalid)")
+        raise RuntimeError(f"DeepEP HIP backend: {what}: " + "; ".join(reasons))
 
     def _prologue(self, previous_event, allocate_on_comm_stream: bool, async_with_compute_stream: bool,
                   v1_rules: bool = False):

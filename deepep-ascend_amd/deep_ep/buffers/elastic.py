@@ -315,3 +315,17 @@ class ElasticBuffer:
         [0, num_experts), one expert named twice by a token) or a row that did not fit the outputs.
         Calls with `do_cpu_sync=True` check this themselves."""
         self.runtime.check_device_status("routing")
+
+    def poll_device_status(self) -> bool:
+        """The same check without waiting for the GPU, for loops that run without host synchronisation (for example
+        `do_cpu_sync=False` dispatches replayed from a graph).  The first call queues a read of the status word on the
+        current stream and returns False; later calls return False until that read has finished, then raise as
+        `check_device_status` does if something was flagged, or return True (the next call queues a new read)."""
+        return self.runtime.poll_device_status("routing")
+
+    def queue_status_read(self, out: torch.Tensor, clear: bool = True) -> None:
+        """Queues, on the current stream, a copy of the device status word into `out` (one int32, pinned host memory or
+        device memory) without any host wait; with `clear` the word is reset on the way, so `out` holds what was
+        flagged since the previous clearing read (0 = nothing; bits as in `deep_ep_hip.h`).  May be captured into a
+        graph together with `do_cpu_sync=False` dispatches: every replay then refreshes `out`."""
+        self.runtime.queue_status_read(out, clear)

@@ -95,6 +95,17 @@ size_t deep_ep_hip_workspace_status_offset(void);
  * zero at the start of a launch (and leave zero at its end).  After DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT, zero these
  * bytes before the workspace is used again. */
 size_t deep_ep_hip_workspace_control_bytes(void);
+/* A status read that does not synchronise the device, for loops that run without host waits (graph replays, serving
+ * loops).  Enqueues on `stream` one small kernel that copies the status word of `workspace` (NULL: the built-in
+ * workspace deep_ep_hip_launch_dispatch_static uses on the current device) to *status_out.  status_out must be memory
+ * the GPU can write: pinned host memory from hipHostMalloc, which the host may read once an event recorded on `stream`
+ * after this call has completed, or device memory.  Kernels only ever OR bits into the status word, so one read after N
+ * launches reports what any of them flagged (DEEP_EP_HIP_STATUS_*).  With clear != 0 the read also puts the word back
+ * to zero, and after DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT zeroes the launch bookkeeping behind it, so that the workspace is
+ * ready for the next launch: *status_out then holds what was flagged since the previous clearing read.  Nothing is
+ * allocated; the launch is an ordinary kernel node and may be captured into a HIP graph, every replay refreshing
+ * *status_out. */
+int deep_ep_hip_read_status(void* workspace, int32_t* status_out, int clear, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Dispatch layout (V1 `Buffer.get_dispatch_layout`): counts only.

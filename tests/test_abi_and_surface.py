@@ -208,7 +208,8 @@ COMMON_MODULE_NAMES = {"get_platform", "topk_idx_t", "EventHandle", "ElasticBuff
 COMMON_BUFFER_METHODS = {"destroy", "get_comm_stream", "get_physical_domain_size", "get_logical_domain_size", "barrier",
                          "dispatch", "combine"}
 HIP_ONLY_MODULE_NAMES = {"EPException", "get_elastic_buffer_alignment", "set_tuning", "get_tuning", "abi_version"}
-HIP_ONLY_BUFFER_METHODS = {"is_destroyed", "get_dispatch_layout", "check_device_status", "device_status",
+HIP_ONLY_BUFFER_METHODS = {"is_destroyed", "get_dispatch_layout", "check_device_status", "poll_device_status", "queue_status_read",
+                           "device_status",
                            "workspace_control_words"}
 
 

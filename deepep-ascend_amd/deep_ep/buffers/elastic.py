@@ -10,6 +10,7 @@ have `num_experts` entries.  With R = 1 every shape and value equals the referen
 size 1.  Placement is scan based, hence already deterministic: `deterministic=True` changes nothing.
 """
 import os
+from dataclasses import dataclass, field
 from typing import List, Optional, Tuple, Union
 
 import torch
@@ -39,54 +40,56 @@ class LogicalGroup:
         pass
 
 
+@dataclass(eq=False)
 class EPHandle:
-    """What `dispatch` returns for `combine` and for cached re-dispatch.
+    """What `dispatch` returns for `combine` and for cached re-dispatch.  Constructor arguments, in order, are the
+    fields up to `channel_linked_list` (reference deep_ep/buffers/elastic.py:40-113).
 
-    Attributes:
+    Fields:
         do_expand: whether the expanded (one row per (token, expert)) layout is used.
         num_experts, expert_alignment, num_max_tokens_per_rank, num_sms: the dispatch settings.
         topk_idx: the routing the handle was built from, `[num_tokens, num_topk]`.
+        num_recv_tokens, num_expanded_tokens: row counts (upper bounds without CPU sync).
+        num_recv_tokens_per_expert_list: aligned rows per expert as a Python list (empty without CPU sync).
         psum_num_recv_tokens_per_scaleup_rank: inclusive prefix of rows per destination rank, `[num_ranks]`.
         psum_num_recv_tokens_per_expert: per expert, inclusive prefix of aligned counts (compact) or
             region start + actual count (expanded), `[num_experts]`.
         num_unaligned_recv_tokens_per_expert: actual rows per expert, `[num_experts]`.
-        num_recv_tokens_per_expert_list: aligned rows per expert as a Python list (empty without CPU sync).
         recv_src_metadata: `[num_recv_tokens, num_topk + 2]`: source token, source rank * num_topk + master
             lane, then the expanded row of each lane (-1 if none).
         dst_buffer_slot_idx: `[num_tokens, num_topk]`: rank_idx * num_max_tokens_per_rank + slot inside the
             destination bucket on each destination's master (highest) lane, -1 elsewhere.
         token_metadata_at_forward, channel_linked_list: hybrid-mode fields, always None here.
-        num_recv_tokens, num_expanded_tokens: row counts (upper bounds without CPU sync).
+        cached_recv_src_metadata_before_sort: deterministic-mode scratch of the reference, always None here.
     """
+    do_expand: bool
+    num_experts: int
+    expert_alignment: int
+    num_max_tokens_per_rank: int
+    num_sms: int
+    topk_idx: torch.Tensor
+    num_recv_tokens: int
+    num_expanded_tokens: int
+    num_recv_tokens_per_expert_list: list
+    psum_num_recv_tokens_per_scaleup_rank: torch.Tensor
+    psum_num_recv_tokens_per_expert: torch.Tensor
+    num_unaligned_recv_tokens_per_expert: torch.Tensor
+    recv_src_metadata: torch.Tensor
+    dst_buffer_slot_idx: torch.Tensor
+    token_metadata_at_forward: Optional[torch.Tensor]
+    channel_linked_list: Optional[torch.Tensor]
+    cached_recv_src_metadata_before_sort: Optional[torch.Tensor] = field(default=None, init=False)
 
-    def __init__(self, do_expand: bool, num_experts: int, expert_alignment: int,
-                 num_max_tokens_per_rank: int, num_sms: int, topk_idx: torch.Tensor,
-                 num_recv_tokens: int, num_expanded_tokens: int,
-                 num_recv_tokens_per_expert_list: list,
-                 psum_num_recv_tokens_per_scaleup_rank: torch.Tensor,
-                 psum_num_recv_tokens_per_expert: torch.Tensor,
-                 num_unaligned_recv_tokens_per_expert: torch.Tensor,
-                 recv_src_metadata: torch.Tensor, dst_buffer_slot_idx: torch.Tensor,
-                 token_metadata_at_forward: Optional[torch.Tensor],
-                 channel_linked_list: Optional[torch.Tensor]):
-        assert topk_idx is not None
-        self.do_expand = do_expand
-        self.num_experts = num_experts
-        self.expert_alignment = expert_alignment
-        self.num_max_tokens_per_rank = num_max_tokens_per_rank
-        self.num_sms = num_sms
-        self.topk_idx = topk_idx
-        self.psum_num_recv_tokens_per_scaleup_rank = psum_num_recv_tokens_per_scaleup_rank
-        self.psum_num_recv_tokens_per_expert = psum_num_recv_tokens_per_expert
-        self.num_unaligned_recv_tokens_per_expert = num_unaligned_recv_tokens_per_expert
-        self.num_recv_tokens_per_expert_list = num_recv_tokens_per_expert_list
-        self.recv_src_metadata = recv_src_metadata
-        self.dst_buffer_slot_idx = dst_buffer_slot_idx
-        self.token_metadata_at_forward = token_metadata_at_forward
-        self.channel_linked_list = channel_linked_list
-        self.num_recv_tokens = num_recv_tokens
-        self.num_expanded_tokens = num_expanded_tokens
-        self.cached_recv_src_metadata_before_sort = None
+    def __post_init__(self):
+        assert self.topk_idx is not None, "a handle always carries the routing it was built from"
+        self.cached_recv_src_metadata_before_sort = None        # an instance attribute, as in the reference
+
+    def layout_fields(self) -> tuple:
+        """The ten values a cached dispatch hands back to the runtime, in the runtime's argument order."""
+        return (self.num_recv_tokens, self.num_expanded_tokens, self.num_recv_tokens_per_expert_list,
+                self.psum_num_recv_tokens_per_scaleup_rank, self.psum_num_recv_tokens_per_expert,
+                self.num_unaligned_recv_tokens_per_expert, self.dst_buffer_slot_idx,
+                self.token_metadata_at_forward, self.recv_src_metadata, self.channel_linked_list)
 
 
 class ElasticBuffer:
@@ -109,41 +112,36 @@ class ElasticBuffer:
                  prefer_overlap_with_compute: bool = True, sl_idx: int = 3, num_allocated_qps: int = 0,
                  num_cpu_timeout_secs: int = 300, num_gpu_timeout_secs: int = 100,
                  explicitly_destroy: bool = False):
-        self.group = group
-        self.rank_idx = group.rank()
-        self.num_ranks = group.size()
-        self.allow_hybrid_mode = allow_hybrid_mode
-        self.allow_multiple_reduction = allow_multiple_reduction
-        self.prefer_overlap_with_compute = prefer_overlap_with_compute
+        self.group, self.rank_idx, self.num_ranks = group, group.rank(), group.size()
+        self.comm_handle = None                     # the reference's communicator handle: there is none
         self.deterministic = deterministic
-        self.comm_handle = None
-
-        if num_bytes is None:
-            num_bytes = _C.calculate_elastic_buffer_size(
-                self.num_ranks, num_max_tokens_per_rank, hidden, num_topk, use_fp8_dispatch,
-                allow_hybrid_mode, allow_multiple_reduction)
-        if os.environ.get('EP_BUFFER_DEBUG', 0):
-            print(f'Initializing EP elastic buffer with {num_bytes} bytes '
-                  f'(cpu: {num_cpu_bytes}) at rank EP {self.rank_idx}/{self.num_ranks}')
-        self.num_bytes = num_bytes
-        self.num_max_tokens_per_rank = num_max_tokens_per_rank
-        self.num_allocated_qps = num_allocated_qps
+        self.allow_hybrid_mode, self.allow_multiple_reduction = allow_hybrid_mode, allow_multiple_reduction
+        self.prefer_overlap_with_compute = prefer_overlap_with_compute
+        self.num_max_tokens_per_rank, self.num_allocated_qps = num_max_tokens_per_rank, num_allocated_qps
         self.explicitly_destroy = explicitly_destroy
-        self.runtime = _C.ElasticBuffer(self.rank_idx, self.num_ranks, 0, None, num_bytes, num_cpu_bytes,
+
+        # Sizing is kept for compatibility: the rows land in the tensors dispatch returns, not in a staging buffer.
+        self.num_bytes = num_bytes if num_bytes is not None else self.get_buffer_size_hint(
+            group, num_max_tokens_per_rank, hidden, num_topk, use_fp8_dispatch, allow_hybrid_mode, allow_multiple_reduction)
+        if os.environ.get('EP_BUFFER_DEBUG'):
+            print(f'EP elastic buffer, logical rank {self.rank_idx} of {self.num_ranks}: {self.num_bytes} bytes '
+                  f'(+ {num_cpu_bytes} on the host)')
+        self.runtime = _C.ElasticBuffer(self.rank_idx, self.num_ranks, 0, None, self.num_bytes, num_cpu_bytes,
                                         allow_hybrid_mode, allow_multiple_reduction, prefer_overlap_with_compute,
                                         sl_idx, num_allocated_qps, num_cpu_timeout_secs, num_gpu_timeout_secs,
                                         explicitly_destroy)
+
+        # One scale-up domain holds every logical rank.
         self.num_scaleout_ranks, self.num_scaleup_ranks = self.get_logical_domain_size()
-        self.scaleout_rank_idx = self.rank_idx // self.num_scaleup_ranks
-        self.scaleup_rank_idx = self.rank_idx % self.num_scaleup_ranks
+        self.scaleout_rank_idx, self.scaleup_rank_idx = divmod(self.rank_idx, self.num_scaleup_ranks)
         self.num_rdma_ranks, self.num_nvlink_ranks = self.get_physical_domain_size()
 
     def destroy(self) -> None:
         """Release the runtime. Requires `explicitly_destroy=True` at construction."""
-        assert self.explicitly_destroy
-        if self.runtime is not None:
-            self.runtime.destroy()
-            self.runtime = None
+        assert self.explicitly_destroy, 'construct with explicitly_destroy=True to release by hand'
+        runtime, self.runtime = self.runtime, None
+        if runtime is not None:
+            runtime.destroy()
 
     @staticmethod
     def get_buffer_size_hint(group, num_max_tokens_per_rank: int, hidden: int, num_topk: int = 0,
@@ -155,15 +153,6 @@ class ElasticBuffer:
 
     def barrier(self, use_comm_stream: bool = True, with_cpu_sync: bool = False, sequential: bool = True) -> None:
         self.runtime.barrier(use_comm_stream, with_cpu_sync, sequential)
-
-    @staticmethod
-    def _unpack_handle(handle: Optional[EPHandle] = None):
-        if handle is None:
-            return (None,) * 10
-        return (handle.num_recv_tokens, handle.num_expanded_tokens, handle.num_recv_tokens_per_expert_list,
-                handle.psum_num_recv_tokens_per_scaleup_rank, handle.psum_num_recv_tokens_per_expert,
-                handle.num_unaligned_recv_tokens_per_expert, handle.dst_buffer_slot_idx,
-                handle.token_metadata_at_forward, handle.recv_src_metadata, handle.channel_linked_list)
 
     @staticmethod
     def capture() -> EventHandle:
@@ -228,33 +217,32 @@ class ElasticBuffer:
 
         Returns (recv_x or (recv_x, recv_sf), recv_topk_idx, recv_topk_weights, handle, event).
         """
-        x, sf = x if isinstance(x, tuple) else (x, None)
+        payload, scale_factors = x if isinstance(x, tuple) else (x, None)
 
+        cached = (None,) * 10
         if handle is not None:
-            assert topk_idx is None
-            assert do_cpu_sync is None or not do_cpu_sync, 'Cannot do CPU sync with cached handle'
-            topk_idx = handle.topk_idx
-            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, handle.num_max_tokens_per_rank)
-            num_experts = value_or(num_experts, handle.num_experts)
-            expert_alignment = value_or(expert_alignment, handle.expert_alignment)
-            do_cpu_sync = False
-            assert (num_experts, expert_alignment, num_max_tokens_per_rank) == \
-                   (handle.num_experts, handle.expert_alignment, handle.num_max_tokens_per_rank)
+            # A cached dispatch replays the handle's routing: its settings may be repeated but not changed.
+            assert topk_idx is None, 'A cached dispatch takes its routing from the handle'
+            assert not do_cpu_sync, 'Cannot do CPU sync with cached handle'
             assert do_expand == handle.do_expand, 'The cached handle was built for the other layout'
-        cached = self._unpack_handle(handle)
-
-        num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
-        expert_alignment = value_or(expert_alignment, 1)
-        do_cpu_sync = value_or(do_cpu_sync, True)
-        assert num_experts is not None, '`num_experts` is required'
-        num_sms = self.get_theoretical_num_sms(num_experts, 0) if num_sms == 0 else num_sms
+            settings = (value_or(num_experts, handle.num_experts), value_or(expert_alignment, handle.expert_alignment),
+                        value_or(num_max_tokens_per_rank, handle.num_max_tokens_per_rank))
+            assert settings == (handle.num_experts, handle.expert_alignment, handle.num_max_tokens_per_rank), \
+                'A cached dispatch cannot change num_experts, expert_alignment or num_max_tokens_per_rank'
+            num_experts, expert_alignment, num_max_tokens_per_rank = settings
+            topk_idx, do_cpu_sync, cached = handle.topk_idx, False, handle.layout_fields()
+        else:
+            assert num_experts is not None, '`num_experts` is required'
+            num_max_tokens_per_rank = value_or(num_max_tokens_per_rank, self.num_max_tokens_per_rank)
+            expert_alignment, do_cpu_sync = value_or(expert_alignment, 1), value_or(do_cpu_sync, True)
+        num_sms = num_sms or self.get_theoretical_num_sms(num_experts, 0)
 
         (recv_x, recv_sf, recv_topk_idx, recv_topk_weights, cloned_topk_idx,
          num_recv_tokens, num_expanded_tokens, num_recv_tokens_per_expert_list,
          psum_num_recv_tokens_per_scaleup_rank, psum_num_recv_tokens_per_expert,
          num_unaligned_recv_tokens_per_expert, recv_src_metadata, dst_buffer_slot_idx,
          token_metadata_at_forward, channel_linked_list, event) = self.runtime.dispatch(
-            x, sf, topk_idx, topk_weights, cumulative_local_expert_recv_stats,
+            payload, scale_factors, topk_idx, topk_weights, cumulative_local_expert_recv_stats,
             *cached,
             num_max_tokens_per_rank, num_experts, expert_alignment, num_sms, num_qps,
             unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
@@ -263,24 +251,22 @@ class ElasticBuffer:
             cast_to_fp8)
 
         if handle is None:
-            handle = EPHandle(do_expand, num_experts, expert_alignment, num_max_tokens_per_rank, num_sms,
-                              cloned_topk_idx if do_handle_copy else topk_idx,
+            kept_topk_idx = cloned_topk_idx if do_handle_copy else topk_idx      # without a copy the handle aliases the caller's tensor
+            handle = EPHandle(do_expand, num_experts, expert_alignment, num_max_tokens_per_rank, num_sms, kept_topk_idx,
                               num_recv_tokens, num_expanded_tokens, num_recv_tokens_per_expert_list,
                               psum_num_recv_tokens_per_scaleup_rank, psum_num_recv_tokens_per_expert,
                               num_unaligned_recv_tokens_per_expert, recv_src_metadata, dst_buffer_slot_idx,
                               token_metadata_at_forward, channel_linked_list)
-        recv_x = (recv_x, recv_sf) if recv_sf is not None else recv_x
-        return recv_x, recv_topk_idx, recv_topk_weights, handle, EventOverlap(event)
+        received = recv_x if recv_sf is None else (recv_x, recv_sf)
+        return received, recv_topk_idx, recv_topk_weights, handle, EventOverlap(event)
 
     @staticmethod
     def _unpack_bias(bias) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-        bias_0, bias_1 = None, None
-        if isinstance(bias, torch.Tensor):
-            bias_0 = bias
-        elif isinstance(bias, tuple):
-            assert len(bias) == 2
-            bias_0, bias_1 = bias
-        return bias_0, bias_1
+        """None, one tensor or a pair of tensors -> always a pair."""
+        if bias is None or isinstance(bias, torch.Tensor):
+            return bias, None
+        first, second = bias            # anything else must be exactly two tensors
+        return first, second
 
     def combine(self, x: torch.Tensor, handle: EPHandle, topk_weights: Optional[torch.Tensor] = None,
                 bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]] = None,
@@ -299,13 +285,12 @@ class ElasticBuffer:
         Returns (combined_x BF16 `[num_tokens, hidden]`, combined_topk_weights float `[num_tokens, num_topk]`
         or None, event).  Accumulation is fp32 with one round-to-nearest-even BF16 store.
         """
-        num_sms = handle.num_sms if num_sms == 0 else num_sms
-        bias_0, bias_1 = ElasticBuffer._unpack_bias(bias)
+        first_bias, second_bias = self._unpack_bias(bias)
         combined_x, combined_topk_weights, event = self.runtime.combine(
-            x, topk_weights, bias_0, bias_1, handle.recv_src_metadata, handle.topk_idx,
+            x, topk_weights, first_bias, second_bias, handle.recv_src_metadata, handle.topk_idx,
             handle.psum_num_recv_tokens_per_scaleup_rank, handle.token_metadata_at_forward,
             handle.channel_linked_list, handle.num_experts, handle.num_max_tokens_per_rank,
-            num_sms, num_qps, unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
+            num_sms or handle.num_sms, num_qps, unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
             async_with_compute_stream, allocate_on_comm_stream, handle.do_expand,
             handle.dst_buffer_slot_idx)
         return combined_x, combined_topk_weights, EventOverlap(event)

@@ -35,12 +35,9 @@ class Buffer:
                  num_qps_per_rank: int = 24, allow_nvlink_for_low_latency_mode: bool = True,
                  allow_mnnvl: bool = False, explicitly_destroy: bool = False, enable_shrink: bool = False,
                  comm=None) -> None:
-        self.group = group
-        self.rank = group.rank()
-        self.group_size = group.size()
-        self.num_nvl_bytes = num_nvl_bytes
-        self.num_rdma_bytes = num_rdma_bytes
-        self.low_latency_mode = low_latency_mode
+        self.group, self.rank, self.group_size = group, group.rank(), group.size()
+        # sizes and mode are recorded as given; the rows land in the tensors the calls return, not in these buffers
+        self.num_nvl_bytes, self.num_rdma_bytes, self.low_latency_mode = num_nvl_bytes, num_rdma_bytes, low_latency_mode
         self.explicitly_destroy = explicitly_destroy
         self.runtime = _C.ElasticBuffer(self.rank, self.group_size, 0, [], _C.get_elastic_buffer_alignment(), 0,
                                         False, True, True, 0, 0, 300, 100, explicitly_destroy)
@@ -49,9 +46,9 @@ class Buffer:
         self._ll_lane_rows = None
 
     def destroy(self) -> None:
-        assert self.explicitly_destroy, '`explicitly_destroy` flag must be set'
-        self.runtime.destroy()
-        self.runtime = None
+        assert self.explicitly_destroy, 'construct with explicitly_destroy=True to release by hand'
+        runtime, self.runtime = self.runtime, None
+        runtime.destroy()
 
     @staticmethod
     def capture() -> EventOverlap:
@@ -121,13 +118,11 @@ class Buffer:
 
     @staticmethod
     def _unpack_bias(bias):
-        bias_0, bias_1 = None, None
-        if isinstance(bias, torch.Tensor):
-            bias_0 = bias
-        elif isinstance(bias, tuple):
-            assert len(bias) == 2
-            bias_0, bias_1 = bias
-        return bias_0, bias_1
+        """None, one tensor or a pair of tensors -> always a pair."""
+        if bias is None or isinstance(bias, torch.Tensor):
+            return bias, None
+        first, second = bias            # anything else must be exactly two tensors
+        return first, second
 
     def dispatch(self, x: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]],
                  handle: Optional[Tuple] = None,
@@ -148,26 +143,28 @@ class Buffer:
         expert of every destination rank (empty with `num_worst_tokens`).  With `handle=` the layout is reused
         and only `recv_x` is returned.
         """
-        config = self.get_dispatch_config(self.group_size) if config is None else config
-        x, x_scales = x if isinstance(x, tuple) else (x, None)
+        config = config or self.get_dispatch_config(self.group_size)
+        payload, scales = x if isinstance(x, tuple) else (x, None)
+        streams = (unwrap_event(previous_event), async_finish, allocate_on_comm_stream)
+        pack = (lambda rows, row_scales: rows) if scales is None else (lambda rows, row_scales: (rows, row_scales))
+
         if handle is not None:
-            assert topk_idx is None and topk_weights is None
-            rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, is_token_in_rank, send_head = handle
-            num_recv_tokens = recv_src_idx.size(0)
-            recv_x, recv_x_scales, _, _, _, _, _, _, _, _, event = self.runtime.intranode_dispatch(
-                x, x_scales, None, None, None, is_token_in_rank, None, num_recv_tokens, rank_prefix_matrix,
-                channel_prefix_matrix, expert_alignment, num_worst_tokens, config, unwrap_event(previous_event),
-                async_finish, allocate_on_comm_stream, cached_send_head=send_head)
-            return (recv_x, recv_x_scales) if x_scales is not None else recv_x, None, None, None, None, EventOverlap(event)
-        assert num_tokens_per_rank is not None and is_token_in_rank is not None and num_tokens_per_expert is not None
-        (recv_x, recv_x_scales, recv_topk_idx, recv_topk_weights, num_recv_tokens_per_expert_list, rank_prefix_matrix,
-         channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, send_head, event) = \
-            self.runtime.intranode_dispatch(x, x_scales, topk_idx, topk_weights, num_tokens_per_rank, is_token_in_rank,
-                                            num_tokens_per_expert, 0, None, None, expert_alignment, num_worst_tokens,
-                                            config, unwrap_event(previous_event), async_finish, allocate_on_comm_stream)
-        handle = (rank_prefix_matrix, channel_prefix_matrix, recv_channel_prefix_matrix, recv_src_idx, is_token_in_rank, send_head)
-        return ((recv_x, recv_x_scales) if x_scales is not None else recv_x, recv_topk_idx, recv_topk_weights,
-                num_recv_tokens_per_expert_list, handle, EventOverlap(event))
+            # cached: the six handle tensors stand in for the layout; only the payload moves
+            assert topk_idx is None and topk_weights is None, 'A cached dispatch takes its routing from the handle'
+            rank_prefix, channel_prefix, _, recv_src_idx, in_rank, send_head = handle
+            out = self.runtime.intranode_dispatch(payload, scales, None, None, None, in_rank, None, recv_src_idx.size(0),
+                                                  rank_prefix, channel_prefix, expert_alignment, num_worst_tokens, config,
+                                                  *streams, cached_send_head=send_head)
+            return pack(out[0], out[1]), None, None, None, None, EventOverlap(out[-1])
+
+        assert all(t is not None for t in (num_tokens_per_rank, is_token_in_rank, num_tokens_per_expert)), \
+            'A fresh dispatch needs the three outputs of get_dispatch_layout'
+        (rows, row_scales, recv_topk_idx, recv_topk_weights, per_expert_list, rank_prefix, channel_prefix,
+         recv_channel_prefix, recv_src_idx, send_head, event) = self.runtime.intranode_dispatch(
+            payload, scales, topk_idx, topk_weights, num_tokens_per_rank, is_token_in_rank, num_tokens_per_expert, 0,
+            None, None, expert_alignment, num_worst_tokens, config, *streams)
+        handle = (rank_prefix, channel_prefix, recv_channel_prefix, recv_src_idx, is_token_in_rank, send_head)
+        return pack(rows, row_scales), recv_topk_idx, recv_topk_weights, per_expert_list, handle, EventOverlap(event)
 
     def combine(self, x: torch.Tensor, handle: Tuple, topk_weights: Optional[torch.Tensor] = None,
                 bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor], None] = None, config=None,
@@ -177,13 +174,13 @@ class Buffer:
         (deep_ep/buffers/legacy.py:407-455): fp32 sum of the biases and of the token's rows in ascending rank
         order, one rounding to BF16; `topk_weights` rows are summed the same way.
         Returns (combined_x, combined_topk_weights, event)."""
-        config = self.get_combine_config(self.group_size) if config is None else config
-        rank_prefix_matrix, _, channel_prefix_matrix, src_idx, is_recv_token_in_rank, send_head = handle
-        bias_0, bias_1 = Buffer._unpack_bias(bias)
-        recv_x, recv_topk_weights, event = self.runtime.intranode_combine(
-            x, topk_weights, bias_0, bias_1, src_idx, rank_prefix_matrix, channel_prefix_matrix, send_head, config,
+        config = config or self.get_combine_config(self.group_size)
+        rank_prefix, _, channel_prefix, src_idx, _, send_head = handle
+        first_bias, second_bias = self._unpack_bias(bias)
+        combined_x, combined_topk_weights, event = self.runtime.intranode_combine(
+            x, topk_weights, first_bias, second_bias, src_idx, rank_prefix, channel_prefix, send_head, config,
             unwrap_event(previous_event), async_finish, allocate_on_comm_stream)
-        return recv_x, recv_topk_weights, EventOverlap(event)
+        return combined_x, combined_topk_weights, EventOverlap(event)
 
     def _workspace(self, num_bytes: int) -> torch.Tensor:
         if self._ll_workspace is None or self._ll_workspace.numel() < num_bytes:

@@ -13,11 +13,13 @@
 // is stored to each destination with 16-byte stores.
 //
 // Single-launch mode ("fused"): the first workgroups of the grid are counting workgroups (one 256-token
-// chunk each, the code of the layout kernel); the last of them to finish publishes the handle tensors.
+// chunk each, the code of the layout kernel) and one publishing workgroup that writes the handle tensors.
 // Mover workgroups issue their payload loads, then wait (first wavefront polls an agent-scope word, the
-// others sit at a workgroup barrier) until the counts are complete, and read what the counting
-// workgroups wrote with agent-scope loads.  Counting workgroups have the lowest workgroup ids, wait for
-// nothing and are therefore resident before any mover can wait for them; every wait is bounded.
+// others sit at a workgroup barrier) until every counting workgroup has stored its chunk totals and
+// positions, and work their row numbers out from those.  Counting workgroups have the lowest workgroup
+// ids, wait for nothing and are therefore resident before any mover can wait for them; every wait is bounded.
+#include <algorithm>
+
 #include "device_utils.h"
 #include "fp8_cast.h"
 #include "kernels.h"
@@ -73,24 +75,28 @@ __device__ __forceinline__ RouteInputs load_route_inputs(const MoveParams& p, in
     return in;
 }
 
+// The word of the layout pass for (token, lane): the cached handle's slot, or the packed chunk-relative positions.
 template <bool kFused>
-__device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteInputs& in, int t, int lane, bool first_tile) {
+__device__ __forceinline__ uint32_t load_position_word(const MoveParams& p, int t, int lane) {
+    if (lane >= p.K) return 0xffffffffu;
+    const int32_t* words = p.cached ? p.cached_slot : reinterpret_cast<const int32_t*>(p.pos);
+    return uint32_t(layout_word<kFused>(words + int64_t(t) * p.K + lane));
+}
+
+// flat_bases (single-launch dispatch): this workgroup's LDS copy of the exclusive prefix over rank_counts.
+template <bool kFused>
+__device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteInputs& in, uint32_t word, const int* flat_bases,
+                                               int t, int lane, bool first_tile) {
     Route r{-1, -1, -1, -1, -1, in.w};
     const int chunk = t / kLayoutChunk;
 
     // ---- issue every load that does not depend on another one, then consume: one memory round trip ----
     int64_t raw = in.raw;
     const uint8_t mask_byte = in.mask_byte;
-    uint32_t word = 0xffffffffu;     // cached: handle slot (-1 = none); otherwise the packed positions of the layout pass
     const bool rank_lanes_cached = p.cached && p.rank_lanes;
-    if (lane < p.K) {
-        const int64_t at = int64_t(t) * p.K + lane;
-        const int32_t* words = p.cached ? p.cached_slot : reinterpret_cast<const int32_t*>(p.pos);
-        word = uint32_t(layout_word<kFused>(words + at));
-    }
     // Wave lane q < R fetches the base row of (rank q, this token's chunk) and the start of rank q's bucket; the
     // routing lanes pick theirs up by shuffle.  (More than 64 ranks: each master lane fetches its own pair below.)
-    const bool bases_by_lane = !p.cached && p.R <= kWaveSize;
+    const bool bases_by_lane = !kFused && !p.cached && p.R <= kWaveSize;
     int base_of_rank = 0, start_of_rank = 0;
     if (bases_by_lane && lane < p.R) {
         base_of_rank = layout_word<kFused>(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded + chunk);
@@ -120,7 +126,11 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteI
     else slot = -1;
     if (!p.cached) {
         int base, start;
-        if (bases_by_lane) {
+        if constexpr (kFused) {
+            const int row = (r.d >= 0 && slot >= 0 ? r.d : 0) * p.tab.chunks_padded;
+            base = flat_bases[row + chunk];
+            start = flat_bases[row];
+        } else if (bases_by_lane) {
             const int from = r.d >= 0 ? r.d : 0;
             base = __shfl(base_of_rank, from, kWaveSize);
             start = __shfl(start_of_rank, from, kWaveSize);
@@ -256,36 +266,45 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
 
 // ---- single-launch dispatch ----
 //
-// Grid: C counting workgroups (one 256-token chunk each), one publishing workgroup, then the movers.  Hand-offs
-// between workgroups of one launch cost a trip to the memory side each (about 0.4 us on an idle GPU), so the
-// protocol keeps them few, and none of its words is touched by more than a few dozen workgroups (agent-scope
-// atomics on one address serialise at about 11 ns each):
-//   - counting workgroup c stores its chunk totals and sets counts_done[c]; then it works out and stores the
-//     positions of its tokens and sets positions_done[c];
-//   - the publisher waits for all counts_done flags, writes the rank rows of the base table and the per-rank
-//     outputs (while the counting workgroups are still busy with their positions), waits for all positions_done
-//     flags, clears both sets of flags and opens every gate (stage 1); then it publishes the per-expert outputs
-//     (and, for the expanded layout, the expert base table) and opens every gate a second time (stage 2);
-//   - mover workgroup m watches gate m % kDispatchGates (each gate a cache line of its own) until it shows the
-//     stage the launch needs (compact layout: 1; expanded layout, whose rows are placed through the published
-//     expert regions: 2), then passes it.
+// Grid: C counting workgroups (one 256-token chunk each), one publishing workgroup, then the movers.  A mover cannot
+// store a row before the layout is known, and the kernel is bound by its stores, so every microsecond before the
+// first store is a microsecond of the launch: the path from the counting workgroups to the movers is kept as short
+// as the hardware allows.  Hand-offs between workgroups of one launch cost a trip to the memory side each (about
+// 0.4 us on an idle GPU, more under load), and agent-scope atomics on one address serialise at about 11 ns each, so
+// no word of the protocol is touched by more than a few dozen workgroups:
+//   - counting workgroup c stores its chunk totals and the positions of its tokens (written through), waits for its
+//     own stores, raises counts_done[c] for the publisher and advances every gate once;
+//   - mover workgroup m watches gate m % kDispatchGates (each gate a cache line of its own) until it shows that all C
+//     counting workgroups have been there; it then works the rank bases out for itself (an exclusive prefix sum over
+//     the R x C chunk totals, into LDS: nobody sits between the counting workgroups and the movers), and passes the
+//     gate (advances it once more);
+//   - the publisher waits for all counts_done flags, clears them, and writes the per-rank and per-expert outputs of
+//     the call while the movers are already moving.  For the expanded layout, whose rows are placed through the
+//     expert regions, it also writes the expert base table and then advances every gate once: the movers of an
+//     expanded dispatch wait for C + 1.
 // Everything handed over is stored at agent scope (written through), so a workgroup only waits for its own
 // stores before it raises a flag: no cache-wide write-back or invalidate runs while the movers stream through
 // the same L2.
 // A gate is only ever advanced with a wrapping increment (0, 1, ..., limit, 0).  Gate g is passed by n_g movers,
-// limit = 1 + n_g, and receives exactly 2 + n_g increments per launch, so it is back at 0 when the launch ends and
-// nobody has to know who was last.  No mover increments a gate before it has seen the stage it needs, hence a gate
-// value >= stage means what it says, and the wrap to 0 happens only after all of the gate's movers have passed.
-// Counting and publishing workgroups have the lowest workgroup ids and wait for nothing that is dispatched after
-// them, so every wait ends; each is bounded anyway and reports DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT.
+// limit = target + n_g - 1 with target = C (+ 1), and receives exactly target + n_g increments per launch, so it is
+// back at 0 when the launch ends and nobody has to know who was last.  No mover increments a gate before it has seen
+// the target, hence a gate value >= target means what it says, and the wrap to 0 happens only after all of the gate's
+// movers have passed.  Counting and publishing workgroups have the lowest workgroup ids and wait for nothing that is
+// dispatched after them, so every wait ends; each is bounded anyway and reports DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT.
 constexpr unsigned kLayoutSpinLimit = 1u << 22;      // polls (each with a short sleep) before giving up: seconds
+
+// Value of a gate at which its movers may pass: every counting workgroup has advanced it once, and for the expanded
+// layout the publisher too.
+__device__ __forceinline__ unsigned gate_target(const MoveParams& p) {
+    return unsigned(p.count_blocks) + (p.do_expand ? 1u : 0u);
+}
 
 __device__ __forceinline__ unsigned movers_of_gate(const MoveParams& p, unsigned gate) {
     return (p.num_movers + unsigned(kDispatchGates) - 1u - gate) / unsigned(kDispatchGates);
 }
 
 __device__ __forceinline__ void advance_gate(const MoveParams& p, unsigned gate) {
-    atomicInc(p.gates + gate * kDispatchGateStride, 1u + movers_of_gate(p, gate));
+    atomicInc(p.gates + gate * kDispatchGateStride, gate_target(p) + movers_of_gate(p, gate) - 1u);
 }
 
 __device__ __forceinline__ void open_all_gates(const MoveParams& p) {
@@ -295,16 +314,11 @@ __device__ __forceinline__ void open_all_gates(const MoveParams& p) {
 __device__ __forceinline__ void fused_count_block(const MoveParams& p) {
     extern __shared__ uint64_t count_lds[];
     const int c = int(blockIdx.x);
-    int32_t* counts_done = p.chunk_done + c;
-    int32_t* positions_done = p.chunk_done + kMaxCountBlocks + c;
-    count_chunk<8, true>(p.lay, c, p.count_blocks, count_lds, [&]() {
-        wait_for_own_stores();
-        __syncthreads();
-        if (threadIdx.x == 0) store_agent(counts_done, 1);
-    });
+    count_chunk<8, true>(p.lay, c, p.count_blocks, count_lds);
     wait_for_own_stores();
     __syncthreads();
-    if (threadIdx.x == 0) store_agent(positions_done, 1);
+    if (threadIdx.x == 0) store_agent(p.chunk_done + c, 1);      // for the publisher
+    open_all_gates(p);                                           // for the movers
 }
 
 // All flags[0..n) set?  Polls (bounded), then clears them for the next launch.  Every thread must call it.
@@ -329,10 +343,7 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     const LayoutTables& tab = p.lay.tab;
 
     await_and_clear_flags(p, p.chunk_done, p.count_blocks);
-    publish_ranks_flat<kThreads>(p.pub, tab, lds);
-    wait_for_own_stores();
-    await_and_clear_flags(p, p.chunk_done + kMaxCountBlocks, p.count_blocks);
-    open_all_gates(p);                                                        // stage 1
+    scan_rank_counts<kThreads>(&p.pub, tab, p.R, nullptr, lds.scan_tmp, &lds);
 
     // The expert tables have one writer per cache line and this workgroup has not touched them before, so
     // ordinary loads fetch what the counting workgroups wrote through.
@@ -341,10 +352,10 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     if (p.do_expand) {
         __syncthreads();
         write_expert_bases<kThreads, true>(tab, p.E, p.count_blocks, lds);
+        wait_for_own_stores();
+        __syncthreads();
+        open_all_gates(p);
     }
-    wait_for_own_stores();
-    __syncthreads();
-    open_all_gates(p);                                                        // stage 2
 }
 
 // First wavefront of a mover workgroup: its first look at the gate goes out together with its payload loads (on a
@@ -356,7 +367,7 @@ __device__ __forceinline__ const int* gate_of(const MoveParams& p, unsigned move
 
 __device__ __forceinline__ void pass_gate(const MoveParams& p, unsigned mover, int first_look) {
     const int* word = gate_of(p, mover);
-    const unsigned need = p.do_expand ? 2u : 1u;
+    const unsigned need = gate_target(p);
     unsigned seen = unsigned(first_look);
     unsigned polls = 0;
     while (seen < need && polls < kLayoutSpinLimit) {
@@ -368,6 +379,15 @@ __device__ __forceinline__ void pass_gate(const MoveParams& p, unsigned mover, i
         if (seen < need) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
         advance_gate(p, mover % unsigned(kDispatchGates));
     }
+}
+
+// Every mover workgroup of a single-launch dispatch works the rank bases out for itself, from the chunk totals the
+// counting workgroups stored, into its LDS (all threads; ends with a barrier).
+__device__ __forceinline__ const int* build_rank_bases(const MoveParams& p) {
+    extern __shared__ uint64_t count_lds[];
+    int* bases = reinterpret_cast<int*>(count_lds);
+    scan_rank_counts<kThreads>(nullptr, p.tab, p.R, bases, bases + p.R * p.tab.chunks_padded, nullptr);
+    return bases;
 }
 
 // ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
@@ -402,15 +422,21 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
     }
 
     const RouteInputs route_in = load_route_inputs(p, t, lane);
+    const int* flat_bases = nullptr;
+    uint32_t word;
     if constexpr (kFused) {
         // Payload and routing inputs are in flight; nothing that reads the layout may be issued before the first
         // wavefront has passed the gate.
         if (threadIdx.x < kWaveSize) pass_gate(p, mover, first_look);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        word = load_position_word<kFused>(p, t, lane);
+        flat_bases = build_rank_bases(p);
         if (!has_work) return;
+    } else {
+        word = load_position_word<kFused>(p, t, lane);
     }
-    const Route r = resolve_route<kFused>(p, route_in, t, lane, tile == 0);
+    const Route r = resolve_route<kFused>(p, route_in, word, flat_bases, t, lane, tile == 0);
     if (tile == 0) write_token_metadata(p, r, t, lane);
 
     int row_of_lane;
@@ -474,15 +500,21 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
     }
 
     const RouteInputs route_in = load_route_inputs(p, t, lane);
+    const int* flat_bases = nullptr;
+    uint32_t word;
     if constexpr (kFused) {
         // Payload and routing inputs are in flight; nothing that reads the layout may be issued before the first
         // wavefront has passed the gate.
         if (threadIdx.x < kWaveSize) pass_gate(p, mover, first_look);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        word = load_position_word<kFused>(p, t, lane);
+        flat_bases = build_rank_bases(p);
         if (!has_work) return;
+    } else {
+        word = load_position_word<kFused>(p, t, lane);
     }
-    const Route r = resolve_route<kFused>(p, route_in, t, lane, tile == 0);
+    const Route r = resolve_route<kFused>(p, route_in, word, flat_bases, t, lane, tile == 0);
     if (tile == 0) write_token_metadata(p, r, t, lane);
 
     vec16 out[kPairs];
@@ -610,7 +642,8 @@ size_t move_lds_bytes(const MoveParams& p) {
     if (!p.fused) return 0;
     const size_t publish = publish_lds_bytes(p.R, p.E, kThreads);
     const size_t bitmap = count_lds_bytes(p.R, p.E);
-    return bitmap > publish ? bitmap : publish;
+    const size_t bases = (size_t(p.R) * p.tab.chunks_padded + kWavesPerBlock) * sizeof(int);
+    return std::max(bases, std::max(bitmap, publish));
 }
 
 // Grid: the counting workgroups of a single-launch dispatch come first.

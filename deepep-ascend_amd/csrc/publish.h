@@ -107,36 +107,47 @@ __device__ void write_rank_bases(const LayoutTables& t, int R, const PublishLds&
     }
 }
 
-// The whole rank part in one pass, for the publishing workgroup of a single-launch dispatch (the movers of the
-// compact layout wait for nothing else): rank_counts, written by other workgroups of the launch and therefore read
-// at agent scope, as one flat array of R * chunks_padded <= 4 * kThreads entries; rank_bases stored at agent scope.
+// The rank part as one flat pass over rank_counts ([rank][chunk], R * chunks_padded <= 4 * kThreads entries; in a
+// single-launch dispatch written through by counting workgroups of the same launch, each line by one writer, and not
+// touched by the caller's workgroup before those have finished, so ordinary loads fetch them): the exclusive prefix sum over the
+// flattened table is, at entry (r, c), the first compact row of rank r's tokens of chunk c; at (r, 0) it is the start
+// of rank r's bucket.  Every thread of the workgroup must call it.
+//   bases != nullptr: the prefix of every entry is stored there (LDS of a mover workgroup, or rank_bases in memory);
+//   s != nullptr:     the per-rank outputs are published (the publishing workgroup).
+// scan_tmp: kThreads / 64 ints of LDS.  Ends with a barrier.
 template <int kThreads>
-__device__ void publish_ranks_flat(const PublishParams& q, const LayoutTables& t, const PublishLds& s) {
+__device__ void scan_rank_counts(const PublishParams* q, const LayoutTables& t, int R, int* bases, int* scan_tmp,
+                                 const PublishLds* s) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int flat = q.R * t.chunks_padded;            // a multiple of 4: a thread's entries share a row
+    const int flat = R * t.chunks_padded;              // a multiple of 4: a thread's entries share a row
     const int begin = tid * 4;
-    int v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = begin < flat ? load_agent(t.rank_counts + begin + u) : 0;
-    const int sum = v[0] + v[1] + v[2] + v[3];
+    vec16 v{0, 0, 0, 0};
+    if (begin < flat) v = load16(t.rank_counts + begin);
+    const int sum = int(v.x) + int(v.y) + int(v.z) + int(v.w);
     const int inc = wave_inclusive_sum(sum);
-    if (lane == kWaveSize - 1) s.scan_tmp[wave] = inc;
+    if (lane == kWaveSize - 1) scan_tmp[wave] = inc;
     __syncthreads();
     int run = inc - sum;
-    for (int w = 0; w < wave; ++w) run += s.scan_tmp[w];
+    for (int w = 0; w < wave; ++w) run += scan_tmp[w];
     if (begin < flat) {
-        store16_agent(t.rank_bases + begin, vec16{uint32_t(run), uint32_t(run + v[0]), uint32_t(run + v[0] + v[1]),
-                                                  uint32_t(run + v[0] + v[1] + v[2])});
-        if ((begin + 4) % t.chunks_padded == 0) s.totals[begin / t.chunks_padded] = run + sum;   // inclusive prefix of the rank
+        if (bases != nullptr) {
+            bases[begin] = run;
+            bases[begin + 1] = run + int(v.x);
+            bases[begin + 2] = run + int(v.x) + int(v.y);
+            bases[begin + 3] = run + int(v.x) + int(v.y) + int(v.z);
+        }
+        if (s != nullptr && (begin + 4) % t.chunks_padded == 0) s->totals[begin / t.chunks_padded] = run + sum;   // inclusive prefix of the rank
     }
     __syncthreads();
-    for (int r = tid; r < q.R; r += kThreads) {
-        const int total = s.totals[r] - (r > 0 ? s.totals[r - 1] : 0);
-        if (q.num_tokens_per_rank != nullptr) q.num_tokens_per_rank[r] = total;
-        if (q.host_counts != nullptr) q.host_counts[r] = -total - 1;
-        if (q.psum_rank != nullptr) q.psum_rank[r] = s.totals[r];
+    if (s != nullptr) {
+        for (int r = tid; r < R; r += kThreads) {
+            const int total = s->totals[r] - (r > 0 ? s->totals[r - 1] : 0);
+            if (q->num_tokens_per_rank != nullptr) q->num_tokens_per_rank[r] = total;
+            if (q->host_counts != nullptr) q->host_counts[r] = -total - 1;
+            if (q->psum_rank != nullptr) q->psum_rank[r] = s->totals[r];
+        }
+        if (tid == 0 && q->totals_out != nullptr) q->totals_out[0] = s->totals[R - 1];
     }
-    if (tid == 0 && q.totals_out != nullptr) q.totals_out[0] = s.totals[q.R - 1];
 }
 
 // ---- expert part: tables are [chunk][expert], so that thread e walks column e with coalesced accesses ----

@@ -8,8 +8,9 @@ routing.  Inputs are resident in HBM before the timed region; outputs are pre-si
 case so no host synchronisation sits inside a step.  Calls go straight through the C ABI.
 
 Prints one JSON line: whole-step achieved HBM GB/s (algorithmic bytes / time), per-op us/call,
-a roofline object for the dominant kernel (combine) and a CPU baseline (the torch-CPU oracle timed
-on a bounded sample of the same workload).
+a roofline object for the dominant kernel (combine), one for the dispatch call, and a CPU baseline (the
+torch-CPU oracle timed on the same workload, all tokens, a few passes).  --workload C5 prints the same for the
+low-latency pair of kernels.
 """
 import argparse
 import ctypes
@@ -26,10 +27,24 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch measured with rocprofv3 (--pmc FETCH_SIZE and --pmc WRITE_SIZE in separate runs, KiB per
 # dispatch, each scaled by what the same counter reads for a plain copy kernel of known size: x2.000 for
-# FETCH_SIZE, x1.000 for WRITE_SIZE on this machine).  Keyed by (workload, layout, payload, kernel).
+# FETCH_SIZE, x1.000 for WRITE_SIZE on this machine).  Keyed by (workload, layout, payload, operation); "dispatch" is
+# the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
-    ("C3", "compact", "fp8", "dispatch"): int((60115.8 * 2.0 + 320764.5 * 1.0) * 1024),
-    ("C3", "compact", "fp8", "combine"): int((308813.4 * 2.0 + 114944.0 * 1.0) * 1024),
+    # profiles/bench_C3_hbm_counters.md
+    ("C3", "compact", "fp8", "dispatch"): 452421301,
+    ("C3", "compact", "fp8", "combine"): 750130002,
+    ("C3", "expanded", "fp8", "dispatch"): 613820902,
+    ("C3", "expanded", "fp8", "combine"): 1074413300,
+    ("C3", "compact", "bf16", "dispatch"): 1093287 + 755651809,
+    ("C3", "compact", "bf16", "combine"): 750133226,
+    # profiles/bench_C4_C2_hbm_counters.md
+    ("C4", "compact", "fp8", "dispatch"): 420222622,
+    ("C4", "compact", "fp8", "combine"): 688673935,
+    ("C2", "compact", "bf16", "dispatch"): 97153228,
+    ("C2", "compact", "bf16", "combine"): 95447829,
+    # profiles/bench_C5_low_latency_hbm_counters.md
+    ("C5", "packed", "fp8", "ll_dispatch"): 23989529,
+    ("C5", "packed", "fp8", "ll_combine"): 30330119,
 }
 
 
@@ -273,9 +288,11 @@ def main():
                      "achieved": round(gbs(ab["combine"], combine_us), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs(ab["combine"], combine_us) / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(traffic_key + ("combine",))},
-        "roofline_dispatch": {"kernel": "dispatch_cast_kernel" if fp8 else "dispatch_copy_kernel", "bound": "hbm",
-                              "achieved": round(gbs(ab["dispatch"], move_us), 1), "peak": HBM_PEAK_GBS,
-                              "unit": "GB/s", "frac": round(gbs(ab["dispatch"], move_us) / HBM_PEAK_GBS, 4),
+        "roofline_dispatch": {"kernel": ("dispatch_cast_kernel" if fp8 else "dispatch_copy_kernel") +
+                                        " (whole call: one launch where the single launch applies, else layout_kernel + this)",
+                              "bound": "hbm", "achieved": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us), 1),
+                              "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us) / HBM_PEAK_GBS, 4),
                               "traffic": MEASURED_TRAFFIC_BYTES.get(traffic_key + ("dispatch",))},
         "wall_ms_timed_region": round(wall_ms, 3),
     }

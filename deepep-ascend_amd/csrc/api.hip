@@ -237,7 +237,8 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
         REQUIRE(!(a->do_expand == 0 && a->recv_topk_idx == nullptr && a->recv_capacity > 0), "recv_topk_idx is NULL");
     }
 
-    // Publishing targets of the layout results (shared by the layout kernel and, in light mode, the move kernel).
+    // Publishing targets of the layout results (the layout kernel's last workgroup, or the publishing workgroup of a
+    // single-launch dispatch).
     PublishParams pub{};
     pub.R = R; pub.E = E; pub.A = a->expert_alignment; pub.do_expand = a->do_expand ? 1 : 0;
     pub.psum_rank = a->psum_num_recv_tokens_per_rank;

@@ -10,9 +10,10 @@
 // its lane bit in an LDS bitmap word per rank and per expert (ds_or_b64), so that
 //   count  = popcount(bitmap)                      and
 //   position of token t among chunk tokens routed to the same bucket = popcount(bitmap & lanes below t)
-// with no ordering-dependent atomics: placement is a pure function of the input.  Chunk totals go
-// to global memory (transposed, so that a consumer prefix-sums along a row); the last workgroup to finish sums
-// them and publishes the public prefix sums.
+// with no ordering-dependent atomics: placement is a pure function of the input (layout_count.h).  Chunk
+// totals go to tables in the workspace; the last workgroup to finish sums them, writes the base tables the
+// move kernel places rows with, and publishes the public prefix sums (publish.h).  A single-launch dispatch
+// runs the same two steps inside the move kernel instead (dispatch.hip).
 #include "device_utils.h"
 #include "kernels.h"
 #include "layout_count.h"

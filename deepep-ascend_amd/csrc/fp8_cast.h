@@ -1,23 +1,26 @@
 // Per-1x128 FP8 e4m3 quantisation of BF16 channels, as a wave-level building block.
 //
-// Follows deep_ep/utils/math.py:30-39: amax over 128 channels clamped below at 1e-4, payload =
-// e4m3(fp32(x) * (448 / amax)), stored scale = amax / 448, both divisions IEEE fp32.  (The
-// low-latency CUDA kernel multiplies by a precomputed 1/448 instead,
-// csrc/kernels/legacy/utils.cuh:477-503; that differs in the last bit of the scale for about
-// half of all amax values, so it is not used here.)
+// amax over 128 channels clamped below at 1e-4, payload = e4m3(fp32(x) * (448 / amax)) with an IEEE fp32 division;
+// what is stored as the group's scale depends on which of the reference's two code paths the caller replaces.
 #pragma once
 
 #include "device_utils.h"
 
 namespace deep_ep_hip {
 
+enum class ScaleRule {
+    kDivide,       // stored scale = amax / 448, IEEE division: deep_ep/utils/math.py:30-39 (dispatch, stand-alone cast)
+    kReciprocal,   // stored scale = amax * fp32(1 / 448): what the low-latency kernel stores,
+                   // csrc/kernels/legacy/utils.cuh:477-479,499-501 (last bit differs from kDivide for many amax values)
+    kPow2,         // `round_scale` of the low-latency kernel, utils.cuh:481-498: see below
+};
+
 // Each lane holds 16 consecutive BF16 channels in (a, b); 8 consecutive lanes form one group of
 // 128 channels.  Writes the 16 e4m3 bytes to `out` and returns the group's stored scale.
 //
-// pow2_scale: the scale is rounded up to a power of two (csrc/kernels/legacy/utils.cuh:481-503, `round_scale`):
-// exponent = ceil(log2(amax * (1/448))) read off the fp32 bit pattern, payload = e4m3(x * 2^-exponent), stored
-// scale = 2^exponent.
-template <bool kPow2Scale = false>
+// kPow2: the scale is rounded up to a power of two: exponent = ceil(log2(amax * (1/448))) read off the fp32 bit
+// pattern, payload = e4m3(x * 2^-exponent), stored scale = 2^exponent.
+template <ScaleRule kRule = ScaleRule::kDivide>
 __device__ __forceinline__ float cast_16_channels(const vec16& a, const vec16& b, vec16& out) {
     const uint32_t wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     float f[16];
@@ -30,14 +33,14 @@ __device__ __forceinline__ float cast_16_channels(const vec16& a, const vec16& b
     }
     amax = fmaxf(group8_max(amax), 1e-4f);
     float scale, scale_inv;
-    if constexpr (kPow2Scale) {
+    if constexpr (kRule == ScaleRule::kPow2) {
         const uint32_t bits = __float_as_uint(amax * (1.0f / 448.0f));
         const int exponent = int((bits >> 23) & 0xffu) - 127 + ((bits & 0x7fffffu) != 0u ? 1 : 0);
         scale = __uint_as_float(uint32_t(127 - exponent) << 23);
         scale_inv = __uint_as_float(uint32_t(127 + exponent) << 23);
     } else {
         scale = 448.0f / amax;
-        scale_inv = amax / 448.0f;
+        scale_inv = kRule == ScaleRule::kReciprocal ? amax * (1.0f / 448.0f) : amax / 448.0f;
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) f[i] = f[i] * scale;

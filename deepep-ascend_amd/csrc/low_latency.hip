@@ -159,8 +159,8 @@ __device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int64_t
     if constexpr (kFp8) {
 #pragma unroll
         for (int q = 0; q < kPairs; ++q) {
-            const float scale_inv = p.round_scale ? cast_16_channels<true>(in[q][0], in[q][1], out[q])
-                                                  : cast_16_channels<false>(in[q][0], in[q][1], out[q]);
+            const float scale_inv = p.round_scale ? cast_16_channels<ScaleRule::kPow2>(in[q][0], in[q][1], out[q])
+                                                  : cast_16_channels<ScaleRule::kReciprocal>(in[q][0], in[q][1], out[q]);
             const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
             if ((lane >> 3) == q) my_scale = gathered;
         }

@@ -204,7 +204,8 @@ class Buffer:
                       num_max_dispatch_tokens_per_rank, hidden, num_experts)`;
             hook: with `return_recv_hook`, a callable to invoke before reading the outputs (the reference splits
                 send and receive around it; on one GPU everything is already enqueued and it does nothing).
-        FP8 scales follow the torch recipe (amax / 448 by IEEE division); with `round_scale` they are rounded up
+        FP8 scales are amax * fp32(1/448), as the reference's kernel stores them (csrc/kernels/legacy/utils.cuh:499-501);
+        with `round_scale` they are rounded up
         to powers of two (csrc/kernels/legacy/utils.cuh:481-503) and with `use_ue8m0` returned as exponent bytes
         packed four to an int32: `[E/R, R*M, hidden // 512]`, column-major in the last two dimensions.
         """

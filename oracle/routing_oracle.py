@@ -12,6 +12,10 @@ Each function names the reference source it restates (paths relative to the refe
                             csrc/kernels/legacy/layout.cu:10-122 (what is counted)
   per_token_cast_to_fp8()   deep_ep/utils/math.py:30-39 (eager semantics)
   per_token_cast_back()     deep_ep/utils/math.py:42-56
+  per_token_cast_to_fp8_ll() csrc/kernels/legacy/utils.cuh:477-479,499-501 as used by internode_ll.cu:223-243: the
+                            low-latency kernel's own recipe (same payload, stored scale = amax * fp32(1/448)); pinned in
+                            tests/test_oracle_fp8.py by exact arithmetic (the product of two fp32 numbers is exact in
+                            fp64, one rounding to fp32)
   world_dispatch()          deep_ep/utils/refs.py:10-123 with the process group replaced by an
                             explicit loop over logical source ranks
   dispatch()                one source rank's share of world_dispatch() (refs.py:55-90 send side +
@@ -107,6 +111,20 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     q = (g * (torch.tensor(448.0, dtype=torch.float32) / amax).unsqueeze(2)).to(torch.float8_e4m3fn)
     scales = amax / torch.tensor(448.0, dtype=torch.float32)
     return q.view(T, Hp)[:, :H].contiguous(), scales.view(T, Hp // 128)
+
+
+def per_token_cast_to_fp8_ll(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """What the reference's low-latency kernel emits without `round_scale` (csrc/kernels/legacy/utils.cuh:477-479,
+    499-501; internode_ll.cu:223-243): amax clamped below at 1e-4, payload = e4m3fn(x * (448 / amax)) as in
+    per_token_cast_to_fp8, but the stored scale is the fp32 product amax * fp32(1 / 448), not the quotient amax / 448
+    (the two differ in the last bit for many amax values)."""
+    assert x.dim() == 2 and x.shape[1] % 128 == 0
+    T, H = x.shape
+    g = x.to(torch.float32).view(T, H // 128, 128)
+    amax = g.abs().amax(dim=2).clamp(min=1e-4)
+    q = (g * (torch.tensor(448.0, dtype=torch.float32) / amax).unsqueeze(2)).to(torch.float8_e4m3fn)
+    scales = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+    return q.view(T, H).contiguous(), scales
 
 
 def per_token_cast_to_fp8_pow2(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -468,7 +486,7 @@ def ll_dispatch(xs: Sequence[torch.Tensor], topk_idxs: Sequence[torch.Tensor],
         x = xs[s]
         idx = topk_idxs[s].to(torch.int64)
         if use_fp8:
-            q, sc = per_token_cast_to_fp8_pow2(x) if round_scale else per_token_cast_to_fp8(x)
+            q, sc = per_token_cast_to_fp8_pow2(x) if round_scale else per_token_cast_to_fp8_ll(x)
         for le in range(E_l):
             e = dst_rank * E_l + le
             toks = (idx == e).any(dim=1).nonzero(as_tuple=True)[0]

@@ -185,3 +185,29 @@ def test_ue8m0_packing_round_trips_through_the_reference_decode_rule():
     # decode as deep_ep/utils/math.py:51-53 does
     back = (packed.view(torch.uint8).to(torch.int32) << 23).view(torch.float32)
     assert torch.equal(back.view(1, 8), s)
+
+
+# ---- the low-latency kernel's stored scale: amax * fp32(1/448) ----
+def test_low_latency_scale_is_the_fp32_product_with_the_reciprocal():
+    """csrc/kernels/legacy/utils.cuh:477-479,499-501.  The product of two fp32 numbers is exact in fp64, so
+    fp32(fp64(amax) * fp64(fp32(1/448))) is the correctly rounded fp32 product, computed without the oracle's code
+    path.  The payload is the torch recipe's (pinned above).  A restatement that divided instead would be caught: the
+    two rules disagree on a good share of the groups."""
+    g = torch.Generator().manual_seed(23)
+    x = (torch.randn((256, 512), generator=g) * torch.logspace(-5, 3, 256).unsqueeze(1)).to(torch.bfloat16)
+    x[0] = 0                                      # amax clamps to 1e-4
+    x[1, :128] = 448.0
+    q, s = oracle.per_token_cast_to_fp8_ll(x)
+    q_div, s_div = oracle.per_token_cast_to_fp8(x)
+    assert torch.equal(q.view(torch.uint8), q_div.view(torch.uint8))
+    amax = x.float().view(256, 4, 128).abs().amax(dim=2).clamp(min=1e-4).numpy()
+    inv448 = np.float64(np.float32(1.0) / np.float32(448.0))
+    exact = (amax.astype(np.float64) * inv448).astype(np.float32)
+    assert np.array_equal(s.numpy().view(np.int32), exact.view(np.int32))
+    differ = (s.view(torch.int32) != s_div.view(torch.int32)).float().mean().item()
+    assert 0.1 < differ < 0.9, differ             # the rules differ in the last bit on many groups, agree on others
+    assert abs(s.view(torch.int32) - s_div.view(torch.int32)).max().item() <= 1
+    assert float(s[1, 0]) == float(np.float32(448.0) * np.float32(inv448))
+    # the low-latency dispatch uses this rule, and only for the scales
+    px, ps, _, _, _ = oracle.ll_dispatch([x[:8]], [torch.zeros((8, 1), dtype=torch.int64)], 8, 1, 1, 0)
+    assert torch.equal(ps[0, :8], s[:8]) and torch.equal(px[0, :8].view(torch.uint8), q[:8].view(torch.uint8))

@@ -317,7 +317,7 @@ def test_low_latency_invariants():
                 b, m = int(begin[le, s]), int(n[le, s])
                 toks = info[le, b:b + m].tolist()
                 assert toks == sorted(toks) and all(e in idx[s, t].tolist() for t in toks)
-                q, sc = oracle.per_token_cast_to_fp8(x[s][toks]) if m else (None, None)
+                q, sc = oracle.per_token_cast_to_fp8_ll(x[s][toks]) if m else (None, None)
                 if m:
                     assert torch.equal(px[le, b:b + m].view(torch.uint8), q.view(torch.uint8)) and torch.equal(ps[le, b:b + m], sc)
         # weighted combine of "expert output = dequantised input": out ~= x * sum of weights of lanes on dst

@@ -31,20 +31,20 @@ HBM_PEAK_GBS = 8000.0
 # the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
-    ("C3", "compact", "fp8", "dispatch"): 452421301,
-    ("C3", "compact", "fp8", "combine"): 750130002,
-    ("C3", "expanded", "fp8", "dispatch"): 613820902,
-    ("C3", "expanded", "fp8", "combine"): 1074413300,
-    ("C3", "compact", "bf16", "dispatch"): 1093287 + 755651809,
-    ("C3", "compact", "bf16", "combine"): 750133226,
+    ("C3", "compact", "fp8", "dispatch"): 452674499,
+    ("C3", "compact", "fp8", "combine"): 750130200,
+    ("C3", "expanded", "fp8", "dispatch"): 614184496,
+    ("C3", "expanded", "fp8", "combine"): 1074413120,
+    ("C3", "compact", "bf16", "dispatch"): 1097549 + 755649847,
+    ("C3", "compact", "bf16", "combine"): 750132725,
     # profiles/bench_C4_C2_hbm_counters.md
-    ("C4", "compact", "fp8", "dispatch"): 420222622,
-    ("C4", "compact", "fp8", "combine"): 688673935,
-    ("C2", "compact", "bf16", "dispatch"): 97153228,
-    ("C2", "compact", "bf16", "combine"): 95447829,
+    ("C4", "compact", "fp8", "dispatch"): 420435041,
+    ("C4", "compact", "fp8", "combine"): 688673806,
+    ("C2", "compact", "bf16", "dispatch"): 97192571,
+    ("C2", "compact", "bf16", "combine"): 95447812,
     # profiles/bench_C5_low_latency_hbm_counters.md
-    ("C5", "packed", "fp8", "ll_dispatch"): 23989529,
-    ("C5", "packed", "fp8", "ll_combine"): 30330119,
+    ("C5", "packed", "fp8", "ll_dispatch"): 23981860,
+    ("C5", "packed", "fp8", "ll_combine"): 30328025,
 }
 
 

@@ -343,19 +343,28 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     const LayoutTables& tab = p.lay.tab;
 
     await_and_clear_flags(p, p.chunk_done, p.count_blocks);
-    scan_rank_counts<kThreads>(&p.pub, tab, p.R, nullptr, lds.scan_tmp, &lds);
 
-    // The expert tables have one writer per cache line and this workgroup has not touched them before, so
-    // ordinary loads fetch what the counting workgroups wrote through.
+    // The expert part first: the movers of an expanded dispatch are waiting for its base table, which therefore goes
+    // out before any of the call's outputs.  (The expert tables have one writer per cache line and this workgroup has
+    // not touched them before, so ordinary loads fetch what the counting workgroups wrote through.)
+    const bool bases_first = p.do_expand && p.E <= kThreads && p.count_blocks <= 32;
+    if (bases_first) {
+        write_expert_bases_from_registers<kThreads>(tab, p.R, p.E, p.pub.A, p.count_blocks, lds);
+        wait_for_own_stores();
+        __syncthreads();
+        open_all_gates(p);
+    }
     sum_expert_columns<kThreads>(tab, p.R, p.E, p.count_blocks, lds.totals);
     publish_experts<kThreads>(p.pub, lds);
-    if (p.do_expand) {
+    if (p.do_expand && !bases_first) {
         __syncthreads();
         write_expert_bases<kThreads, true>(tab, p.E, p.count_blocks, lds);
         wait_for_own_stores();
         __syncthreads();
         open_all_gates(p);
     }
+    __syncthreads();
+    scan_rank_counts<kThreads>(&p.pub, tab, p.R, nullptr, lds.scan_tmp, &lds);
 }
 
 // First wavefront of a mover workgroup: its first look at the gate goes out together with its payload loads (on a

@@ -216,6 +216,41 @@ __device__ void write_expert_bases(const LayoutTables& t, int E, int num_chunks,
     }
 }
 
+// The expert base table in one trip, for the publishing workgroup of a single-launch expanded dispatch, whose movers
+// wait for exactly this: thread e keeps its column of chunk totals in registers between the sum and the stores.
+// Needs E <= kThreads and num_chunks <= 32.  Leaves totals / aligned / aligned_incl as publish_experts expects to
+// recompute them; stores at agent scope.  A: expert alignment.
+template <int kThreads>
+__device__ void write_expert_bases_from_registers(const LayoutTables& t, int R, int E, int A, int num_chunks, const PublishLds& s) {
+    const int e = threadIdx.x;
+    int v[32];
+    int total = 0;
+    if (e < E) {
+        const int32_t* col = t.expert_counts + e;
+#pragma unroll
+        for (int u = 0; u < 32; ++u) v[u] = col[int64_t(min(u, num_chunks - 1)) * t.experts_padded];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) total += u < num_chunks ? v[u] : 0;
+        s.totals[R + e] = total;
+        const int al = (total + A - 1) / A * A;
+        s.aligned[e] = al;
+        s.aligned_incl[e] = al;
+    }
+    __syncthreads();
+    block_inclusive_scan<kThreads>(s.aligned_incl, E, s.scan_tmp);
+    if (e < E) {
+        int32_t* out = t.expert_bases + e;
+        int run = s.aligned_incl[e] - s.aligned[e];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            if (u < num_chunks) {
+                store_agent(out + int64_t(u) * t.experts_padded, run);
+                run += v[u];
+            }
+        }
+    }
+}
+
 // Everything at once, for a workgroup that publishes after all counting is over (the stand-alone layout kernel):
 // totals, public outputs, and - when the caller has room for them - the base tables.
 template <int kThreads>

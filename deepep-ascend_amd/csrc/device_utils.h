@@ -161,12 +161,13 @@ __device__ __forceinline__ int load_word(const int* p) {
     if constexpr (kAgent) return load_agent(p);
     else return *p;
 }
-// 16-byte agent-scope (write-through) store.  Written as an instruction because the language offers atomics of at
-// most 8 bytes; a store has no result register, so nothing the compiler tracks depends on its completion.
+// 16 bytes stored at agent scope (written through), as two 8-byte atomic stores: the language offers atomics of at most
+// 8 bytes, and a 16-byte store written as an instruction by hand would sit outside the compiler's hazard tracking
+// (a vector store of more than 8 bytes must not have its data registers overwritten in the next cycle).
 __device__ __forceinline__ void store16_agent(void* p, const vec16& v) {
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    const u32x4 t = {v.x, v.y, v.z, v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(t) : "memory");
+    unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+    __hip_atomic_store(q, (unsigned long long)(v.x) | ((unsigned long long)(v.y) << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(q + 1, (unsigned long long)(v.z) | ((unsigned long long)(v.w) << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Waits until every store this wavefront has issued is acknowledged.  After agent-scope stores this is all a

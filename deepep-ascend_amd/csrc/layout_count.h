@@ -137,7 +137,7 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
                         if (j > k && d[j] == d[k]) master = false;
                         if (j != k && e[j] == e[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
                     }
-                    pe = uint32_t(rank_in_chunk(p.R + e[k]));
+                    if (p.expert_bases) pe = uint32_t(rank_in_chunk(p.R + e[k]));      // only the expanded layout places rows by expert
                     if (master) pr = uint32_t(rank_in_chunk(d[k]));
                 }
                 packed[k] = pr | (pe << 16);

@@ -419,8 +419,9 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
             "handle tensors are NULL");
     REQUIRE(!any || a->combined_x != nullptr, "combined_x is NULL");
     REQUIRE(!any || a->x != nullptr || a->num_x_rows == 0, "x is NULL");
-    REQUIRE(!(a->do_expand && any && a->recv_src_metadata == nullptr), "the expanded layout needs recv_src_metadata");
     REQUIRE(a->num_recv_rows >= 0, "num_recv_rows must be >= 0");
+    REQUIRE(!(a->do_expand && any && a->num_recv_rows > 0 && a->recv_src_metadata == nullptr),
+            "the expanded layout needs recv_src_metadata");
     REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
     CombineParams p{};
     p.x = static_cast<const uint8_t*>(a->x);
@@ -499,11 +500,14 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         if (a->payload == DEEP_EP_HIP_PAYLOAD_BF16)
             REQUIRE(a->num_scales == 0 && a->x_scales == nullptr && a->recv_x_scales == nullptr,
                     "a BF16 payload carries no scales");
-        if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8)
-            REQUIRE(a->num_scales >= 0 && (a->num_scales == 0 || T == 0 || (a->x_scales != nullptr && a->recv_x_scales != nullptr)),
-                    "x_scales / recv_x_scales is NULL");
+        const bool no_rows = a->recv_capacity == 0;                       // empty outputs have no storage
+        if (a->payload == DEEP_EP_HIP_PAYLOAD_FP8) {
+            REQUIRE(a->num_scales >= 0, "num_scales must be >= 0");
+            REQUIRE(a->num_scales == 0 || T == 0 || a->x_scales != nullptr, "x_scales is NULL");
+            REQUIRE(a->num_scales == 0 || no_rows || a->recv_x_scales != nullptr, "recv_x_scales is NULL");
+        }
         if (a->payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8)
-            REQUIRE(H % 128 == 0 && a->num_scales == H / 128 && (a->recv_x_scales != nullptr || T == 0),
+            REQUIRE(H % 128 == 0 && a->num_scales == H / 128 && (a->recv_x_scales != nullptr || no_rows),
                     "the fused FP8 cast needs hidden %% 128 == 0, num_scales == hidden / 128 and recv_x_scales");
         REQUIRE(!with_topk || a->recv_capacity == 0 || (a->recv_topk_idx != nullptr && a->recv_topk_weights != nullptr),
                 "recv_topk_idx / recv_topk_weights is NULL");

@@ -89,7 +89,6 @@ void fill_fused(MoveParams& m, const LayoutParams& lay, const LaunchPlan& plan, 
     m.fused = 1;
     m.count_blocks = plan.chunks;
     m.lay = lay;
-    m.lay.count_only = 1;
     m.lay.vec_idx = (reinterpret_cast<uintptr_t>(lay.topk_idx) % 16 == 0) ? 1 : 0;
     m.chunk_done = reinterpret_cast<int32_t*>(ws + w.chunk_done);
     m.gates = reinterpret_cast<uint32_t*>(ws + w.gates);
@@ -108,7 +107,7 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.done_counter = off + 4;
     w.totals = off + 8;
     off = 256;
-    w.chunk_done = off;    off = align_up(off + size_t(kMaxCountBlocks) * 2 * 4, 256);
+    w.chunk_done = off;    off = align_up(off + size_t(kMaxCountBlocks) * 4, 256);
     w.gates = off;         off = align_up(off + size_t(kDispatchGates) * kDispatchGateStride * 4, 256);
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
     const size_t experts_padded = (size_t(num_experts) + 31) / 32 * 32;

@@ -19,7 +19,7 @@ struct WorkspaceLayout {
     size_t status;         // int32: device status bits
     size_t done_counter;   // uint32: workgroups of the layout kernel that have finished
     size_t totals;         // int32[2]: total compact rows, total expanded rows (incl. padding)
-    size_t chunk_done;     // int32[2][1024]: per-chunk completion flags of a single-launch dispatch
+    size_t chunk_done;     // int32[1024]: per-chunk completion flags of a single-launch dispatch (counting workgroup -> publisher)
     size_t gates;          // uint32[kDispatchGates], one per 128-byte line: stage counters of a single-launch dispatch
     size_t expert_start;   // int32[E]: first expanded row of each expert
     size_t rank_counts;    // int32[R][C padded to a multiple of 4]: per-chunk totals of the rank buckets, transposed
@@ -68,7 +68,6 @@ struct LayoutParams {
     const int64_t* topk_idx;
     const uint8_t* route_mask;       // [T, R] bool: when set, lane r of token t is "rank r, if the mask says so" (K = E = R)
     int T, K, E, R, E_l;
-    int count_only;       // 1: a counting workgroup of a single-launch dispatch (somebody else publishes)
     int vec_idx;          // topk_idx is 16-byte aligned (set by the launcher)
     uint8_t* is_token_in_rank;       // optional
     int64_t* copied_topk_idx;        // optional
@@ -121,7 +120,7 @@ struct MoveParams {
     int count_blocks;
     unsigned num_movers;     // mover workgroups (set by the launcher)
     LayoutParams lay;        // what the counting workgroups need (lay.pub is unused: `pub` above is published)
-    int32_t* chunk_done;     // [2][kMaxCountBlocks] flags of the counting workgroups: counts stored, positions stored
+    int32_t* chunk_done;     // [kMaxCountBlocks] flags of the counting workgroups for the publisher: totals and positions stored
     uint32_t* gates;         // [kDispatchGates] wrapping stage counters, kDispatchGateStride words apart
     // V1 (intranode) conventions
     int rank_lanes;          // routing lanes are ranks (mask routing or a cached send_head), K == R

@@ -57,13 +57,19 @@ struct LaunchPlan {
 // 180 us in one launch against 140 us in two; 8 192 workgroups of the same rows cast to FP8 take 92 us against 97 us.
 constexpr int64_t kMaxFusedMovers = 16384;
 
-LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_move, int payload, int H, int row_bytes,
-                         const deep_ep_hip_tuning& tuning) {
+LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_move, bool do_expand, int alignment, int payload, int H,
+                         int row_bytes, const deep_ep_hip_tuning& tuning) {
     LaunchPlan q{};
     q.chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
     q.chunks_padded = (q.chunks + 3) / 4 * 4;
-    q.fused = do_layout && do_move && T > 0 && K <= 8 && (R + E) <= 512 && R * q.chunks_padded <= 1024 &&
-              tuning.dispatch_launches != 2;
+    q.fused = do_layout && do_move && T > 0 && K <= 8 && (R + E) <= 512 && R * q.chunks_padded <= kTaggedRankWords &&
+              int64_t(T) * K <= kTaggedPosWords && tuning.dispatch_launches != 2;
+    if (q.fused && do_expand) {
+        // the tagged expert bases: the table must fit, and a row number must fit under the tag
+        const int64_t experts_padded = (int64_t(E) + 31) / 32 * 32;
+        q.fused = q.chunks * experts_padded <= kTaggedExpertWords &&
+                  int64_t(T) * K + int64_t(E) * alignment <= int64_t(kTagValueMask);
+    }
     if (q.fused && tuning.dispatch_launches != 1) {
         MoveParams probe{};
         probe.T = T; probe.H = H; probe.row_bytes = row_bytes; probe.payload = payload;
@@ -92,6 +98,17 @@ void fill_fused(MoveParams& m, const LayoutParams& lay, const LaunchPlan& plan, 
     m.lay.vec_idx = (reinterpret_cast<uintptr_t>(lay.topk_idx) % 16 == 0) ? 1 : 0;
     m.chunk_done = reinterpret_cast<int32_t*>(ws + w.chunk_done);
     m.gates = reinterpret_cast<uint32_t*>(ws + w.gates);
+    m.gates_finished = reinterpret_cast<uint32_t*>(ws + w.gates_finished);
+    m.generation = reinterpret_cast<uint32_t*>(ws + w.generation);
+    m.tagged = reinterpret_cast<uint32_t*>(ws + w.tagged);
+    m.tagged_words = int((w.tagged_end - w.tagged) / 4);
+    m.tagged_rank = reinterpret_cast<const uint32_t*>(ws + w.tagged_rank);
+    m.tagged_expert = reinterpret_cast<uint32_t*>(ws + w.tagged_expert);
+    // positions of this launch are read by its own movers: they go to the tagged table
+    m.pos = reinterpret_cast<const uint32_t*>(ws + w.tagged_pos);
+    m.lay.pos = reinterpret_cast<uint32_t*>(ws + w.tagged_pos);
+    m.lay.tagged_rank = reinterpret_cast<uint32_t*>(ws + w.tagged_rank);
+    m.lay.generation = m.generation;
 }
 
 }  // namespace
@@ -106,9 +123,18 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.status = off;
     w.done_counter = off + 4;
     w.totals = off + 8;
+    // A line of their own for the two words only agent-scope stores and atomics write: the line of the status word also
+    // takes ordinary stores (the row totals), and a cache that writes such a line back whole would undo them.
+    w.generation = off + 128;
+    w.gates_finished = off + 132;
     off = 256;
     w.chunk_done = off;    off = align_up(off + size_t(kMaxCountBlocks) * 4, 256);
     w.gates = off;         off = align_up(off + size_t(kDispatchGates) * kDispatchGateStride * 4, 256);
+    w.tagged = off;
+    w.tagged_rank = off;   off += size_t(kTaggedRankWords) * 4;
+    w.tagged_expert = off; off += size_t(kTaggedExpertWords) * 4;
+    w.tagged_pos = off;    off += size_t(kTaggedPosWords) * 4;
+    w.tagged_end = off;
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
     const size_t experts_padded = (size_t(num_experts) + 31) / 32 * 32;
     w.rank_counts = off;   off = align_up(off + chunks_padded * num_ranks * 4, 256);
@@ -252,7 +278,8 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
     // chunk), the first row of that chunk's share of the bucket; the move kernel adds the two.  Layout and move in
     // one call: the counting workgroups ride at the front of the move kernel (one launch); shapes that does not
     // cover run the layout kernel first.
-    const LaunchPlan plan = plan_launches(T, K, E, R, do_layout, do_move, a->payload, H, H * elem_in, a->tuning);
+    const LaunchPlan plan = plan_launches(T, K, E, R, do_layout, do_move, a->do_expand != 0, a->expert_alignment, a->payload, H,
+                                          H * elem_in, a->tuning);
     LayoutParams lay{};
     lay.topk_idx = a->topk_idx;
     lay.T = T; lay.K = K; lay.E = E; lay.R = R; lay.E_l = E / R;
@@ -342,6 +369,8 @@ size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_exp
 size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
 
 size_t deep_ep_hip_workspace_control_bytes(void) { return make_workspace_layout(1, 1, 1, 1).expert_start; }
+
+size_t deep_ep_hip_workspace_counter_bytes(void) { return make_workspace_layout(1, 1, 1, 1).tagged; }
 
 int deep_ep_hip_read_status(void* workspace, int32_t* status_out, int clear, void* stream) {
     REQUIRE(status_out != nullptr, "status_out is NULL");
@@ -520,7 +549,7 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
     pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
 
-    const LaunchPlan plan = plan_launches(T, K, E, R, do_layout, do_move, a->payload, H, H * elem_in, a->tuning);
+    const LaunchPlan plan = plan_launches(T, K, E, R, do_layout, do_move, false, 1, a->payload, H, H * elem_in, a->tuning);
     LayoutParams lay{};
     lay.topk_idx = a->topk_idx;
     lay.route_mask = with_topk ? nullptr : a->is_token_in_rank;

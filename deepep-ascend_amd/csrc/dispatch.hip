@@ -14,10 +14,10 @@
 //
 // Single-launch mode ("fused"): the first workgroups of the grid are counting workgroups (one 256-token
 // chunk each, the code of the layout kernel) and one publishing workgroup that writes the handle tensors.
-// Mover workgroups issue their payload loads, then wait (first wavefront polls an agent-scope word, the
-// others sit at a workgroup barrier) until every counting workgroup has stored its chunk totals and
-// positions, and work their row numbers out from those.  Counting workgroups have the lowest workgroup
-// ids, wait for nothing and are therefore resident before any mover can wait for them; every wait is bounded.
+// Mover workgroups issue their payload loads, then read the chunk totals and position words the counting
+// workgroups store (again, until a word shows the tag of this launch), and work their row numbers out from
+// those.  Counting workgroups have the lowest workgroup ids, wait for nothing and are therefore resident
+// before any mover can wait for them; every wait is bounded.
 #include <algorithm>
 
 #include "device_utils.h"
@@ -47,11 +47,7 @@ struct Route {
     float w;
 };
 
-// A word of the layout tables.  In a single-launch dispatch they were written by counting workgroups of the same
-// launch, possibly through another XCD's L2: the writers release them (write back) before any gate opens, and no
-// mover touches a table line before it has passed its gate, so this XCD's caches cannot hold an older copy of
-// the line and an ordinary load fetches what was written.  (Each table line has a single writer.)
-template <bool kFused>
+// A word of the layout tables a finished layout pass (an earlier launch, or a cached handle) left in memory.
 __device__ __forceinline__ int layout_word(const int32_t* at) {
     return *at;
 }
@@ -75,18 +71,18 @@ __device__ __forceinline__ RouteInputs load_route_inputs(const MoveParams& p, in
     return in;
 }
 
-// The word of the layout pass for (token, lane): the cached handle's slot, or the packed chunk-relative positions.
-template <bool kFused>
+// The word of the layout pass for (token, lane): the cached handle's slot, or the position word (kernels.h).
 __device__ __forceinline__ uint32_t load_position_word(const MoveParams& p, int t, int lane) {
     if (lane >= p.K) return 0xffffffffu;
     const int32_t* words = p.cached ? p.cached_slot : reinterpret_cast<const int32_t*>(p.pos);
-    return uint32_t(layout_word<kFused>(words + int64_t(t) * p.K + lane));
+    return uint32_t(layout_word(words + int64_t(t) * p.K + lane));
 }
 
-// flat_bases (single-launch dispatch): this workgroup's LDS copy of the exclusive prefix over rank_counts.
+// Single-launch dispatch: flat_bases is this workgroup's LDS copy of the exclusive prefix over the chunk totals of the
+// rank buckets, expert_base the first expanded row of (the token's chunk, the lane's expert).
 template <bool kFused>
 __device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteInputs& in, uint32_t word, const int* flat_bases,
-                                               int t, int lane, bool first_tile) {
+                                               int expert_base, int t, int lane, bool first_tile) {
     Route r{-1, -1, -1, -1, -1, in.w};
     const int chunk = t / kLayoutChunk;
 
@@ -99,8 +95,8 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteI
     const bool bases_by_lane = !kFused && !p.cached && p.R <= kWaveSize;
     int base_of_rank = 0, start_of_rank = 0;
     if (bases_by_lane && lane < p.R) {
-        base_of_rank = layout_word<kFused>(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded + chunk);
-        start_of_rank = layout_word<kFused>(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded);
+        base_of_rank = layout_word(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded + chunk);
+        start_of_rank = layout_word(p.tab.rank_bases + int64_t(lane) * p.tab.chunks_padded);
     }
 
     int slot = -1, epos = -1;
@@ -117,8 +113,8 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteI
             if (p.cached) {
                 slot = cached_v >= 0 ? cached_v - p.rank_idx * p.M : -1;
             } else {
-                slot = (packed & 0xffffu) == 0xffffu ? -1 : int(packed & 0xffffu);
-                epos = int(packed >> 16);
+                slot = (packed & kNoPosition) == kNoPosition ? -1 : int(packed & kNoPosition);
+                epos = int((packed >> kExpertPositionShift) & kNoPosition);
             }
         }
     }
@@ -136,8 +132,8 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteI
             start = __shfl(start_of_rank, from, kWaveSize);
         } else {
             const int64_t row = int64_t(r.d >= 0 && slot >= 0 ? r.d : 0) * p.tab.chunks_padded;
-            base = layout_word<kFused>(p.tab.rank_bases + row + chunk);
-            start = layout_word<kFused>(p.tab.rank_bases + row);
+            base = layout_word(p.tab.rank_bases + row + chunk);
+            start = layout_word(p.tab.rank_bases + row);
         }
         if (r.d >= 0 && slot >= 0) {
             r.row_c = base + slot;
@@ -169,8 +165,10 @@ __device__ __forceinline__ Route resolve_route(const MoveParams& p, const RouteI
         if (p.cached) {
             if (r.my_row >= 0 && r.my_row < p.recv_capacity)
                 r.erow = p.recv_src_metadata[int64_t(r.my_row) * (p.K + 2) + 2 + lane];
+        } else if constexpr (kFused) {
+            r.erow = expert_base + epos;
         } else {
-            r.erow = layout_word<kFused>(p.tab.expert_bases + int64_t(chunk) * p.tab.experts_padded + r.e) + epos;
+            r.erow = layout_word(p.tab.expert_bases + int64_t(chunk) * p.tab.experts_padded + r.e) + epos;
         }
     }
     return r;
@@ -269,46 +267,45 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
 // Grid: C counting workgroups (one 256-token chunk each), one publishing workgroup, then the movers.  A mover cannot
 // store a row before the layout is known, and the kernel is bound by its stores, so every microsecond before the
 // first store is a microsecond of the launch: the path from the counting workgroups to the movers is kept as short
-// as the hardware allows.  Hand-offs between workgroups of one launch cost a trip to the memory side each (about
-// 0.4 us on an idle GPU, more under load), and agent-scope atomics on one address serialise at about 11 ns each, so
-// no word of the protocol is touched by more than a few dozen workgroups:
-//   - counting workgroup c stores its chunk totals and the positions of its tokens (written through), waits for its
-//     own stores, raises counts_done[c] for the publisher and advances every gate once;
-//   - mover workgroup m watches gate m % kDispatchGates (each gate a cache line of its own) until it shows that all C
-//     counting workgroups have been there; it then works the rank bases out for itself (an exclusive prefix sum over
-//     the R x C chunk totals, into LDS: nobody sits between the counting workgroups and the movers), and passes the
-//     gate (advances it once more);
-//   - the publisher waits for all counts_done flags, clears them, and writes the per-rank and per-expert outputs of
-//     the call while the movers are already moving.  For the expanded layout, whose rows are placed through the
-//     expert regions, it also writes the expert base table and then advances every gate once: the movers of an
-//     expanded dispatch wait for C + 1.
-// Everything handed over is stored at agent scope (written through), so a workgroup only waits for its own
-// stores before it raises a flag: no cache-wide write-back or invalidate runs while the movers stream through
-// the same L2.
-// A gate is only ever advanced with a wrapping increment (0, 1, ..., limit, 0).  Gate g is passed by n_g movers,
-// limit = target + n_g - 1 with target = C (+ 1), and receives exactly target + n_g increments per launch, so it is
-// back at 0 when the launch ends and nobody has to know who was last.  No mover increments a gate before it has seen
-// the target, hence a gate value >= target means what it says, and the wrap to 0 happens only after all of the gate's
-// movers have passed.  Counting and publishing workgroups have the lowest workgroup ids and wait for nothing that is
-// dispatched after them, so every wait ends; each is bounded anyway and reports DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT.
+// as the hardware allows.  A hand-off between workgroups of one launch costs a trip to the memory side for the
+// writer's store and one for the reader's load (about a microsecond each on a busy GPU); a flag on top of the data
+// would add the writer's wait for its stores, the flag's own trip and a second read.  So the data is its own flag:
+//   - every word handed to the movers (chunk totals of the rank buckets, position words, expert bases) carries the
+//     tag of this launch in its upper bits (kernels.h) and is stored at agent scope (written through);
+//   - a mover workgroup reads what it needs at agent scope - each thread four chunk totals, each wavefront the
+//     position words of its token, and for the expanded layout the base of each lane's (chunk, expert) - and repeats
+//     a read (bounded) until the word shows the tag.  The first read of each goes out before the payload loads.  It
+//     then works the rank bases out for itself (an exclusive prefix sum over the R x C chunk totals, into LDS);
+//   - the publisher waits for the chunk_done flags the counting workgroups raise once their stores are acknowledged,
+//     clears them, and writes the per-rank and per-expert outputs of the call while the movers are already moving;
+//     for the expanded layout the tagged expert bases go out first.
+// The tag is generation + 1, and the generation word is advanced by whichever mover learns that every mover has read
+// its words: a mover that is done reading advances its gate (mover m uses gate m % kDispatchGates, each gate a cache
+// line of its own, because agent-scope atomics on one address serialise at about 11 ns each); the one that brings
+// a gate to its number of movers advances gates_finished; the one that brings that to the number of gates in use
+// advances the generation.  Gates and gates_finished wrap to 0 on the last increment, so nothing is reset between
+// launches.  No workgroup reads the generation after it has moved: counting workgroups and the publisher read it when
+// they start, and the movers' reads cannot complete before those have stored their words.  The launch that uses tag
+// kTagPeriod clears the tagged tables and starts over at generation 0, so a word can never show the tag of a launch
+// other than the running one.  Counting and publishing workgroups have the lowest workgroup ids and wait for nothing
+// that is dispatched after them, so every wait ends; each is bounded anyway and reports
+// DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT.
 constexpr unsigned kLayoutSpinLimit = 1u << 22;      // polls (each with a short sleep) before giving up: seconds
 
-// Value of a gate at which its movers may pass: every counting workgroup has advanced it once, and for the expanded
-// layout the publisher too.
-__device__ __forceinline__ unsigned gate_target(const MoveParams& p) {
-    return unsigned(p.count_blocks) + (p.do_expand ? 1u : 0u);
+__device__ __forceinline__ uint32_t launch_tag(const uint32_t* generation) {
+    return (uint32_t(load_agent(reinterpret_cast<const int*>(generation))) + 1u) << kTagShift;
+}
+
+__device__ __forceinline__ bool has_tag(uint32_t word, uint32_t tag) {
+    return (word & ~kTagValueMask) == tag;
+}
+
+__device__ __forceinline__ uint64_t load_agent64(const void* p) {
+    return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ unsigned movers_of_gate(const MoveParams& p, unsigned gate) {
     return (p.num_movers + unsigned(kDispatchGates) - 1u - gate) / unsigned(kDispatchGates);
-}
-
-__device__ __forceinline__ void advance_gate(const MoveParams& p, unsigned gate) {
-    atomicInc(p.gates + gate * kDispatchGateStride, gate_target(p) + movers_of_gate(p, gate) - 1u);
-}
-
-__device__ __forceinline__ void open_all_gates(const MoveParams& p) {
-    for (unsigned g = threadIdx.x; g < unsigned(kDispatchGates); g += kThreads) advance_gate(p, g);
 }
 
 __device__ __forceinline__ void fused_count_block(const MoveParams& p) {
@@ -318,7 +315,6 @@ __device__ __forceinline__ void fused_count_block(const MoveParams& p) {
     wait_for_own_stores();
     __syncthreads();
     if (threadIdx.x == 0) store_agent(p.chunk_done + c, 1);      // for the publisher
-    open_all_gates(p);                                           // for the movers
 }
 
 // All flags[0..n) set?  Polls (bounded), then clears them for the next launch.  Every thread must call it.
@@ -341,62 +337,164 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     extern __shared__ uint64_t count_lds[];
     const PublishLds lds = carve_publish_lds(reinterpret_cast<int*>(count_lds), p.R, p.E);
     const LayoutTables& tab = p.lay.tab;
+    const uint32_t tag = launch_tag(p.generation);
+    int32_t* tagged_bases = reinterpret_cast<int32_t*>(p.tagged_expert);
 
     await_and_clear_flags(p, p.chunk_done, p.count_blocks);
 
     // The expert part first: the movers of an expanded dispatch are waiting for its base table, which therefore goes
-    // out before any of the call's outputs.  (The expert tables have one writer per cache line and this workgroup has
+    // out before any of the call's outputs.  (The count tables have one writer per cache line and this workgroup has
     // not touched them before, so ordinary loads fetch what the counting workgroups wrote through.)
     const bool bases_first = p.do_expand && p.E <= kThreads && p.count_blocks <= 32;
-    if (bases_first) {
-        write_expert_bases_from_registers<kThreads>(tab, p.R, p.E, p.pub.A, p.count_blocks, lds);
-        wait_for_own_stores();
-        __syncthreads();
-        open_all_gates(p);
-    }
+    if (bases_first) write_expert_bases_from_registers<kThreads>(tab, tagged_bases, tag, p.R, p.E, p.pub.A, p.count_blocks, lds);
     sum_expert_columns<kThreads>(tab, p.R, p.E, p.count_blocks, lds.totals);
     publish_experts<kThreads>(p.pub, lds);
     if (p.do_expand && !bases_first) {
         __syncthreads();
-        write_expert_bases<kThreads, true>(tab, p.E, p.count_blocks, lds);
-        wait_for_own_stores();
-        __syncthreads();
-        open_all_gates(p);
+        write_expert_bases<kThreads, true>(tab, tagged_bases, tag, p.E, p.count_blocks, lds);
     }
     __syncthreads();
-    scan_rank_counts<kThreads>(&p.pub, tab, p.R, nullptr, lds.scan_tmp, &lds);
+    scan_rank_counts<kThreads>(p.pub, tab, p.R, lds);
 }
 
-// First wavefront of a mover workgroup: its first look at the gate goes out together with its payload loads (on a
-// busy GPU every trip to the memory side takes as long as they do); it then waits (bounded) until the layout is as
-// complete as this launch needs it and passes the gate.  The other wavefronts meet it at a workgroup barrier.
-__device__ __forceinline__ const int* gate_of(const MoveParams& p, unsigned mover) {
-    return reinterpret_cast<const int*>(p.gates + (mover % unsigned(kDispatchGates)) * kDispatchGateStride);
-}
+// What a mover reads of the layout before the layout is known to be there: issued ahead of the payload loads, so
+// that a mover that starts after the layout is complete (most of them) has paid no extra trip for it.
+struct FirstLook {
+    uint64_t totals_lo, totals_hi;     // this thread's four chunk totals
+    uint32_t position;                 // this lane's position word
+};
 
-__device__ __forceinline__ void pass_gate(const MoveParams& p, unsigned mover, int first_look) {
-    const int* word = gate_of(p, mover);
-    const unsigned need = gate_target(p);
-    unsigned seen = unsigned(first_look);
-    unsigned polls = 0;
-    while (seen < need && polls < kLayoutSpinLimit) {
-        __builtin_amdgcn_s_sleep(2);
-        seen = unsigned(load_agent(word));
-        ++polls;
+__device__ __forceinline__ FirstLook first_look(const MoveParams& p, int t, int lane, bool has_work) {
+    FirstLook f{0, 0, 0};
+    const int begin = int(threadIdx.x) * 4;
+    if (begin < p.R * p.tab.chunks_padded) {
+        f.totals_lo = load_agent64(p.tagged_rank + begin);
+        f.totals_hi = load_agent64(p.tagged_rank + begin + 2);
     }
-    if (threadIdx.x == 0) {
-        if (seen < need) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
-        advance_gate(p, mover % unsigned(kDispatchGates));
-    }
+    if (has_work && lane < p.K) f.position = uint32_t(load_agent(reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane));
+    return f;
 }
 
-// Every mover workgroup of a single-launch dispatch works the rank bases out for itself, from the chunk totals the
-// counting workgroups stored, into its LDS (all threads; ends with a barrier).
-__device__ __forceinline__ const int* build_rank_bases(const MoveParams& p) {
+// Has this wavefront's first look found everything it asked for?  (Wave-uniform.)
+__device__ __forceinline__ bool look_is_complete(const MoveParams& p, const FirstLook& look, uint32_t tag, bool has_work, int lane) {
+    bool ok = !(has_work && lane < p.K) || has_tag(look.position, tag);
+    if (int(threadIdx.x) * 4 < p.R * p.tab.chunks_padded)
+        ok = ok && has_tag(uint32_t(look.totals_lo), tag) && has_tag(uint32_t(look.totals_lo >> 32), tag) &&
+             has_tag(uint32_t(look.totals_hi), tag) && has_tag(uint32_t(look.totals_hi >> 32), tag);
+    return __all(ok);
+}
+
+// Every mover workgroup works the rank bases out for itself, into its LDS: thread i waits (bounded) for chunk totals
+// 4i .. 4i + 3 of the flattened [rank][chunk] table to show the tag, then the workgroup takes the exclusive prefix
+// sum.  All threads; ends with a barrier.  Returns false when the wait ran out.
+__device__ __forceinline__ bool build_rank_bases(const MoveParams& p, uint32_t tag, const FirstLook& look, const int*& bases_out) {
     extern __shared__ uint64_t count_lds[];
     int* bases = reinterpret_cast<int*>(count_lds);
-    scan_rank_counts<kThreads>(nullptr, p.tab, p.R, bases, bases + p.R * p.tab.chunks_padded, nullptr);
-    return bases;
+    const int flat = p.R * p.tab.chunks_padded;           // a multiple of 4: a thread's entries share a row
+    int* scan_tmp = bases + flat;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int begin = tid * 4;
+    uint64_t lo = look.totals_lo, hi = look.totals_hi;
+    bool complete = true;
+    if (begin < flat) {
+        unsigned polls = 0;
+        auto tagged = [&]() {
+            return has_tag(uint32_t(lo), tag) && has_tag(uint32_t(lo >> 32), tag) && has_tag(uint32_t(hi), tag) &&
+                   has_tag(uint32_t(hi >> 32), tag);
+        };
+        while (!tagged() && polls < kLayoutSpinLimit) {
+            __builtin_amdgcn_s_sleep(2);
+            lo = load_agent64(p.tagged_rank + begin);
+            hi = load_agent64(p.tagged_rank + begin + 2);
+            ++polls;
+        }
+        complete = tagged();
+    }
+    const int v0 = int(uint32_t(lo) & kTagValueMask), v1 = int(uint32_t(lo >> 32) & kTagValueMask);
+    const int v2 = int(uint32_t(hi) & kTagValueMask), v3 = int(uint32_t(hi >> 32) & kTagValueMask);
+    const int sum = v0 + v1 + v2 + v3;
+    const int inc = wave_inclusive_sum(sum);
+    if (lane == kWaveSize - 1) scan_tmp[wave] = inc;
+    const int all_complete = __syncthreads_and(complete ? 1 : 0);
+    int run = inc - sum;
+    for (int w = 0; w < wave; ++w) run += scan_tmp[w];
+    if (begin < flat) {
+        bases[begin] = run;
+        bases[begin + 1] = run + v0;
+        bases[begin + 2] = run + v0 + v1;
+        bases[begin + 3] = run + v0 + v1 + v2;
+    }
+    __syncthreads();
+    bases_out = bases;
+    return all_complete != 0;
+}
+
+// A wavefront's wait (bounded) for words of its own lanes: `word` holds each lane's first read of `at`; lanes with
+// wanted == false take no part.  Returns false when the wait ran out.
+__device__ __forceinline__ bool await_tagged_word(const int* at, bool wanted, uint32_t tag, uint32_t& word) {
+    unsigned polls = 0;
+    while (__any(wanted && !has_tag(word, tag)) && polls < kLayoutSpinLimit) {
+        __builtin_amdgcn_s_sleep(1);
+        if (wanted && !has_tag(word, tag)) word = uint32_t(load_agent(at));
+        ++polls;
+    }
+    return !__any(wanted && !has_tag(word, tag));
+}
+
+// The mover workgroup is done reading tagged words: its first thread advances the gate.  The value the gate had is
+// looked at only when the workgroup ends (settle_gate), so nobody waits for the atomic's answer.
+__device__ __forceinline__ unsigned advance_gate(const MoveParams& p, unsigned mover) {
+    const unsigned gate = mover % unsigned(kDispatchGates);
+    return atomicInc(p.gates + gate * kDispatchGateStride, movers_of_gate(p, gate) - 1u);
+}
+
+// First thread of a mover workgroup, last thing it does.  The mover that was the last of its gate reports the gate;
+// the one that reports the last gate advances the generation: by then every mover has read its tagged words.
+__device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover, unsigned seen, uint32_t tag) {
+    const unsigned gate = mover % unsigned(kDispatchGates);
+    if (seen != movers_of_gate(p, gate) - 1u) return;
+    const unsigned gates_in_use = p.num_movers < unsigned(kDispatchGates) ? p.num_movers : unsigned(kDispatchGates);
+    if (atomicInc(p.gates_finished, gates_in_use - 1u) != gates_in_use - 1u) return;
+    uint32_t next = tag >> kTagShift;                     // generation + 1
+    if (next == kTagPeriod) {
+        for (int i = 0; i < p.tagged_words; i += 4) store16_agent(p.tagged + i, vec16{0, 0, 0, 0});
+        wait_for_own_stores();
+        next = 0;
+    }
+    store_agent(reinterpret_cast<int*>(p.generation), int(next));
+}
+
+// Everything a mover wavefront needs from the layout of its own launch.
+struct FusedLayout {
+    const int* flat_bases;    // LDS: exclusive prefix over the chunk totals of the rank buckets
+    uint32_t position;        // this lane's position word (tag included)
+    int expert_base;          // expanded layout: first row of (this token's chunk, this lane's expert)
+    unsigned gate_seen;       // first thread: what advance_gate returned
+    uint32_t tag;
+    bool complete;            // false: a wait ran out (status already set); the wavefront stores nothing
+};
+
+__device__ __forceinline__ FusedLayout await_layout(const MoveParams& p, unsigned mover, const FirstLook& look, uint32_t tag,
+                                                    const RouteInputs& in, int t, int lane, bool has_work) {
+    FusedLayout f{nullptr, look.position, 0, 0u, tag, true};
+    // position words: each wavefront waits for those of its own token
+    const bool wants_position = has_work && lane < p.K;
+    bool complete = await_tagged_word(reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane, wants_position, tag, f.position);
+    if (p.do_expand) {
+        int64_t e = p.route_mask != nullptr ? (in.mask_byte != 0 ? int64_t(lane) : int64_t(-1)) : in.raw;
+        const bool wants_base = wants_position && e >= 0 && e < p.E;
+        const int* at = reinterpret_cast<const int*>(p.tagged_expert) + int64_t(t / kLayoutChunk) * p.tab.experts_padded + (wants_base ? int(e) : 0);
+        uint32_t word = wants_base ? uint32_t(load_agent(at)) : 0u;
+        complete = await_tagged_word(at, wants_base, tag, word) && complete;
+        f.expert_base = int(word & kTagValueMask);
+    }
+    complete = build_rank_bases(p, tag, look, f.flat_bases) && complete;      // ends with a workgroup barrier
+    if (threadIdx.x == 0) f.gate_seen = advance_gate(p, mover);
+    // One wavefront's failure is the workgroup's: build_rank_bases has already combined the threads' waits for the
+    // totals; a wait for a position or an expert base that ran out stops that wavefront only.
+    if (!complete && lane == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+    f.complete = complete;
+    return f;
 }
 
 // ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
@@ -411,15 +509,18 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
     }
     const int lane = threadIdx.x & 63;
     const unsigned mover = blockIdx.x - (kFused ? unsigned(p.count_blocks) + 1u : 0u);
-    int first_look = 0;
-    if constexpr (kFused)
-        if (threadIdx.x < kWaveSize) first_look = load_agent(gate_of(p, mover));
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(mover, p.num_movers) : mover;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
     const bool has_work = work < unsigned(p.T) * unsigned(p.tiles);
     if (!has_work && !kFused) return;
     const int t = has_work ? int(work / unsigned(p.tiles)) : 0;
     const int tile = has_work ? int(work - unsigned(t) * unsigned(p.tiles)) : 0;
+    uint32_t tag = 0;
+    FirstLook look{0, 0, 0};
+    if constexpr (kFused) {
+        tag = launch_tag(p.generation);
+        look = first_look(p, t, lane, has_work);
+    }
 
     vec16 v[kVecs];
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
@@ -433,19 +534,23 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
     const RouteInputs route_in = load_route_inputs(p, t, lane);
     const int* flat_bases = nullptr;
     uint32_t word;
+    int expert_base = 0;
+    unsigned gate_seen = 0;
     if constexpr (kFused) {
-        // Payload and routing inputs are in flight; nothing that reads the layout may be issued before the first
-        // wavefront has passed the gate.
-        if (threadIdx.x < kWaveSize) pass_gate(p, mover, first_look);
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        word = load_position_word<kFused>(p, t, lane);
-        flat_bases = build_rank_bases(p);
-        if (!has_work) return;
+        // Payload and routing inputs are in flight; wait for this launch's layout.
+        const FusedLayout f = await_layout(p, mover, look, tag, route_in, t, lane, has_work);
+        gate_seen = f.gate_seen;
+        if (!has_work || !f.complete) {
+            if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+            return;
+        }
+        word = f.position;
+        flat_bases = f.flat_bases;
+        expert_base = f.expert_base;
     } else {
-        word = load_position_word<kFused>(p, t, lane);
+        word = load_position_word(p, t, lane);
     }
-    const Route r = resolve_route<kFused>(p, route_in, word, flat_bases, t, lane, tile == 0);
+    const Route r = resolve_route<kFused>(p, route_in, word, flat_bases, expert_base, t, lane, tile == 0);
     if (tile == 0) write_token_metadata(p, r, t, lane);
 
     int row_of_lane;
@@ -466,6 +571,8 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
                     p.sf[int64_t(t) * p.sf_ts + int64_t(g) * p.sf_hs];
         }
     }
+    if constexpr (kFused)
+        if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
 }
 
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
@@ -480,15 +587,18 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
     }
     const int lane = threadIdx.x & 63;
     const unsigned mover = blockIdx.x - (kFused ? unsigned(p.count_blocks) + 1u : 0u);
-    int first_look = 0;
-    if constexpr (kFused)
-        if (threadIdx.x < kWaveSize) first_look = load_agent(gate_of(p, mover));
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(mover, p.num_movers) : mover;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
     const bool has_work = work < unsigned(p.T) * unsigned(p.tiles);
     if (!has_work && !kFused) return;
     const int t = has_work ? int(work / unsigned(p.tiles)) : 0;
     const int tile = has_work ? int(work - unsigned(t) * unsigned(p.tiles)) : 0;
+    uint32_t tag = 0;
+    FirstLook look{0, 0, 0};
+    if constexpr (kFused) {
+        tag = launch_tag(p.generation);
+        look = first_look(p, t, lane, has_work);
+    }
 
     vec16 in[kPairs][2];
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
@@ -509,31 +619,49 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
     }
 
     const RouteInputs route_in = load_route_inputs(p, t, lane);
-    const int* flat_bases = nullptr;
-    uint32_t word;
-    if constexpr (kFused) {
-        // Payload and routing inputs are in flight; nothing that reads the layout may be issued before the first
-        // wavefront has passed the gate.
-        if (threadIdx.x < kWaveSize) pass_gate(p, mover, first_look);
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        word = load_position_word<kFused>(p, t, lane);
-        flat_bases = build_rank_bases(p);
-        if (!has_work) return;
-    } else {
-        word = load_position_word<kFused>(p, t, lane);
-    }
-    const Route r = resolve_route<kFused>(p, route_in, word, flat_bases, t, lane, tile == 0);
-    if (tile == 0) write_token_metadata(p, r, t, lane);
 
     vec16 out[kPairs];
     float my_scale = 0.f;   // lane L < 8*kPairs ends up holding the scale of group (tile*kPairs*8 + L)
+    auto cast_tile = [&]() {
 #pragma unroll
-    for (int q = 0; q < kPairs; ++q) {
-        const float scale_inv = cast_16_channels(in[q][0], in[q][1], out[q]);
-        const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
-        if ((lane >> 3) == q) my_scale = gathered;
+        for (int q = 0; q < kPairs; ++q) {
+            const float scale_inv = cast_16_channels(in[q][0], in[q][1], out[q]);
+            const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
+            if ((lane >> 3) == q) my_scale = gathered;
+        }
+    };
+
+    const int* flat_bases = nullptr;
+    uint32_t word;
+    int expert_base = 0;
+    unsigned gate_seen = 0;
+    bool cast_done = false;
+    if constexpr (kFused) {
+        // Payload and routing inputs are in flight.  A wavefront whose first look found the layout (any wavefront that
+        // starts after the first microseconds of the launch) resolves its rows while the payload arrives, as in a
+        // launch of its own.  One that has to wait for the layout converts its tile first: when the layout appears,
+        // every resident wavefront of the chip is released at once, and the conversions (a few hundred vector
+        // instructions each, eight wavefronts to a SIMD) would otherwise queue up between that moment and the first
+        // stores of the launch.
+        if (!look_is_complete(p, look, tag, has_work, lane)) {
+            cast_tile();
+            cast_done = true;
+        }
+        const FusedLayout f = await_layout(p, mover, look, tag, route_in, t, lane, has_work);
+        gate_seen = f.gate_seen;
+        if (!has_work || !f.complete) {
+            if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+            return;
+        }
+        word = f.position;
+        flat_bases = f.flat_bases;
+        expert_base = f.expert_base;
+    } else {
+        word = load_position_word(p, t, lane);
     }
+    const Route r = resolve_route<kFused>(p, route_in, word, flat_bases, expert_base, t, lane, tile == 0);
+    if (tile == 0) write_token_metadata(p, r, t, lane);
+    if (!cast_done) cast_tile();
     const int group = tile * kPairs * 8 + lane;
     const bool owns_scale = lane < kPairs * 8 && group * 128 < p.H;
 
@@ -552,6 +680,8 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
         if (owns_scale)
             p.recv_sf[int64_t(row) * p.rsf_ts + int64_t(group) * p.rsf_hs] = __float_as_uint(my_scale);
     }
+    if constexpr (kFused)
+        if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
 }
 
 // ---- zero the alignment padding rows of the expanded layout ----

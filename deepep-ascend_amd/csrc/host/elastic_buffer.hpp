@@ -542,11 +542,12 @@ public:
         return workspace_.has_value() ? workspace_->slice(0, 0, 4).view(torch::kInt32).item<int>() : 0;
     }
 
-    // The bookkeeping words at the head of the workspace (status, launch protocol), copied to the host after a full
-    // synchronisation: between launches everything but the status word and the two row totals reads zero.
+    // The counters and flags at the head of the workspace (status, launch protocol), copied to the host after a full
+    // synchronisation: between launches everything but the status word (word 0), the two row totals (words 2 and 3) and
+    // the launch generation (word 32) reads zero.
     torch::Tensor workspace_control_words() {
         c10::hip::device_synchronize();
-        const int64_t n = static_cast<int64_t>(deep_ep_hip_workspace_control_bytes());
+        const int64_t n = static_cast<int64_t>(deep_ep_hip_workspace_counter_bytes());
         if (not workspace_.has_value()) return torch::zeros({n / 4}, torch::kInt32);
         return workspace_->slice(0, 0, n).view(torch::kInt32).cpu();
     }

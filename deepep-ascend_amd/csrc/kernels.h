@@ -8,25 +8,52 @@
 
 namespace deep_ep_hip {
 
-// Single-launch dispatch: number of gates the movers spread over, and the distance between two gates in 32-bit
-// words (one cache line each).
+// Single-launch dispatch: number of completion counters ("gates") the movers spread over, and the distance between
+// two of them in 32-bit words (one cache line each).
 constexpr int kDispatchGates = 256;
 constexpr int kDispatchGateStride = 32;
 constexpr int kMaxCountBlocks = 1024;
+
+// Single-launch dispatch: words that counting and publishing workgroups hand to the movers of the same launch carry
+// the launch's tag in their upper bits, so that a reader knows a word of this launch from what an earlier launch left
+// at the same place and needs no separate flag (and the writer need not wait for its store before it raises one).
+// The tagged tables live in the zero-initialised bookkeeping part of the workspace, which only these kernels write:
+// every word there is zero, or carries the tag of a launch since the tables were last cleared.  Tags run through
+// 1 .. kTagPeriod; the launch that uses the last one clears the tables.
+constexpr int kTagShift = 18;
+constexpr uint32_t kTagValueMask = (1u << kTagShift) - 1u;
+constexpr uint32_t kTagPeriod = (1u << (32 - kTagShift)) - 1u;      // 16383
+constexpr int kTaggedRankWords = 1024;       // R x chunks (padded to a multiple of 4)
+constexpr int kTaggedExpertWords = 8192;     // chunks x experts (padded to a multiple of 32)
+constexpr int kTaggedPosWords = 65536;       // tokens x lanes
+
+// A position word: bits 0-8 the slot of the token inside its chunk for the lane's destination rank (master lanes
+// only), bits 9-17 the position of the lane inside its chunk for its expert, kNoPosition = none; a single-launch
+// dispatch puts its tag above them.
+constexpr uint32_t kNoPosition = 0x1ffu;
+constexpr int kExpertPositionShift = 9;
 
 // Byte offsets of the regions carved out of the caller's workspace.
 struct WorkspaceLayout {
     size_t status;         // int32: device status bits
     size_t done_counter;   // uint32: workgroups of the layout kernel that have finished
     size_t totals;         // int32[2]: total compact rows, total expanded rows (incl. padding)
+    size_t generation;     // uint32: single-launch dispatches since the tagged tables were cleared (tag = generation + 1)
+    size_t gates_finished; // uint32: gates whose movers have all read the tagged tables
     size_t chunk_done;     // int32[1024]: per-chunk completion flags of a single-launch dispatch (counting workgroup -> publisher)
-    size_t gates;          // uint32[kDispatchGates], one per 128-byte line: stage counters of a single-launch dispatch
+    size_t gates;          // uint32[kDispatchGates], one per 128-byte line: movers that have read the tagged tables
+    size_t tagged;         // start of the tagged tables; everything before it reads zero between launches but for
+                           // status, totals and generation
+    size_t tagged_rank;    // uint32[kTaggedRankWords]: rank_counts of the running single-launch dispatch, tagged
+    size_t tagged_expert;  // uint32[kTaggedExpertWords]: its expert_bases, tagged
+    size_t tagged_pos;     // uint32[kTaggedPosWords]: its position words, tagged
+    size_t tagged_end;
     size_t expert_start;   // int32[E]: first expanded row of each expert
     size_t rank_counts;    // int32[R][C padded to a multiple of 4]: per-chunk totals of the rank buckets, transposed
     size_t rank_bases;     // int32[R][C padded]: first compact row of every (rank, chunk)
     size_t expert_counts;  // int32[C][E padded to a multiple of 32]: per-chunk totals of the expert buckets
     size_t expert_bases;   // int32[C][E padded]: first expanded row of every (chunk, expert)
-    size_t pos;            // uint32[Tmax*K]: chunk-relative positions, rank slot | expert position << 16
+    size_t pos;            // uint32[Tmax*K]: position words of a dispatch in two launches
     size_t total_bytes;
 };
 
@@ -77,6 +104,10 @@ struct LayoutParams {
     LayoutTables tab;                // the base tables are optional (layout-only calls have no use for them)
     int expert_bases;                // 1: also tab.expert_bases (expanded layout)
     uint32_t* pos;                   // optional (layout-only calls skip the per-lane positions)
+    // Single-launch dispatch (else NULL): chunk totals of the rank buckets go to tagged_rank as well, tagged like the
+    // position words, with the tag *generation names when the workgroup starts.
+    uint32_t* tagged_rank;
+    const uint32_t* generation;
 };
 
 hipError_t launch_layout_kernel(const LayoutParams& p, hipStream_t stream);
@@ -121,7 +152,13 @@ struct MoveParams {
     unsigned num_movers;     // mover workgroups (set by the launcher)
     LayoutParams lay;        // what the counting workgroups need (lay.pub is unused: `pub` above is published)
     int32_t* chunk_done;     // [kMaxCountBlocks] flags of the counting workgroups for the publisher: totals and positions stored
-    uint32_t* gates;         // [kDispatchGates] wrapping stage counters, kDispatchGateStride words apart
+    uint32_t* gates;         // [kDispatchGates] wrapping counters of the movers that are done reading, kDispatchGateStride words apart
+    uint32_t* gates_finished;    // wrapping counter of the gates all of whose movers are done
+    uint32_t* generation;        // see WorkspaceLayout
+    uint32_t* tagged;            // the tagged tables, tagged_words long: cleared by the launch that uses the last tag
+    int tagged_words;
+    const uint32_t* tagged_rank;
+    uint32_t* tagged_expert;
     // V1 (intranode) conventions
     int rank_lanes;          // routing lanes are ranks (mask routing or a cached send_head), K == R
     int slot_is_row;         // cached_slot holds rows of the receive buffer, not rank * M + slot

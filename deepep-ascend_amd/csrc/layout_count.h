@@ -25,23 +25,20 @@ inline size_t count_lds_bytes(int R, int E) {
     return size_t(R + E) * (kLayoutChunk / kWaveSize) * sizeof(uint64_t) + size_t(R + E) * sizeof(uint32_t);
 }
 
-struct NoHook {
-    __device__ void operator()() const {}
-};
-
 // bitmap: LDS of count_lds_bytes(R, E) bytes.  Must be called by all 256 threads of the workgroup.
-// kThrough: positions and chunk totals are stored at agent scope (a workgroup of the same launch reads them).
-// counts_stored() is called by every thread once the chunk totals have been stored, before the positions are
-// worked out.
-template <int KMAX, bool kThrough, class Hook = NoHook>
-__device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chunk, const int num_chunks,
-                                            uint64_t* bitmap, Hook counts_stored = Hook()) {
+// kThrough: positions and chunk totals are stored at agent scope (workgroups of the same launch read them); the
+// position words and the copy of the rank totals in p.tagged_rank carry the launch's tag.
+template <int KMAX, bool kThrough>
+__device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chunk, const int num_chunks, uint64_t* bitmap) {
     constexpr int kThreads = kLayoutChunk;
     constexpr int kWaves = kThreads / kWaveSize;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int t = chunk * kThreads + tid;
     const int n = p.R + p.E;
     const bool active = t < p.T;
+    uint32_t tag = 0;
+    if constexpr (kThrough)
+        if (p.generation != nullptr) tag = (uint32_t(load_agent(reinterpret_cast<const int*>(p.generation))) + 1u) << kTagShift;
 
     // The index loads go out first (they are the longest wait of the pass), before anything that could alias
     // them is stored; the bitmap is cleared while they are in flight.
@@ -106,12 +103,19 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
         int32_t* at = j < p.R ? p.tab.rank_counts + int64_t(j) * p.tab.chunks_padded + chunk
                               : p.tab.expert_counts + int64_t(chunk) * p.tab.experts_padded + (j - p.R);
         store_word<kThrough>(at, c0 + c1 + c2 + c3);
+        if constexpr (kThrough)
+            if (j < p.R && p.tagged_rank != nullptr)
+                store_agent(reinterpret_cast<int*>(p.tagged_rank) + j * p.tab.chunks_padded + chunk, int(uint32_t(c0 + c1 + c2 + c3) | tag));
     }
     const int pad = p.tab.chunks_padded - num_chunks;  // the padding columns of the rank table are cleared by the first workgroup
-    if (chunk == 0)
-        for (int i = tid; i < p.R * pad; i += kThreads)
-            store_word<kThrough>(p.tab.rank_counts + int64_t(i / pad) * p.tab.chunks_padded + num_chunks + i % pad, 0);
-    counts_stored();
+    if (chunk == 0) {
+        for (int i = tid; i < p.R * pad; i += kThreads) {
+            const int at = (i / pad) * p.tab.chunks_padded + num_chunks + i % pad;
+            store_word<kThrough>(p.tab.rank_counts + at, 0);
+            if constexpr (kThrough)
+                if (p.tagged_rank != nullptr) store_agent(reinterpret_cast<int*>(p.tagged_rank) + at, int(tag));
+        }
+    }
     __syncthreads();
 
     const uint64_t below = lanes_below(lane);
@@ -123,13 +127,12 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
 
     if (active) {
         if (p.pos != nullptr) {
-            // One word per (token, lane): low 16 bits = slot of the token inside its chunk for the lane's
-            // destination rank (master lanes only), high 16 bits = position of the lane inside its chunk for
-            // its expert; 0xffff = none.
+            // One word per (token, lane): the slot of the token inside its chunk for the lane's destination rank
+            // (master lanes only) and the position of the lane inside its chunk for its expert (kernels.h).
             uint32_t packed[KMAX];
 #pragma unroll
             for (int k = 0; k < KMAX; ++k) {
-                uint32_t pr = 0xffffu, pe = 0xffffu;
+                uint32_t pr = kNoPosition, pe = kNoPosition;
                 if (e[k] >= 0) {
                     bool master = true;
 #pragma unroll
@@ -140,7 +143,7 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
                     if (p.expert_bases) pe = uint32_t(rank_in_chunk(p.R + e[k]));      // only the expanded layout places rows by expert
                     if (master) pr = uint32_t(rank_in_chunk(d[k]));
                 }
-                packed[k] = pr | (pe << 16);
+                packed[k] = pr | (pe << kExpertPositionShift) | tag;
             }
             if (KMAX == 8 && p.K == 8) {
                 vec16* dst = reinterpret_cast<vec16*>(p.pos + int64_t(t) * 8);

@@ -109,15 +109,11 @@ __device__ void write_rank_bases(const LayoutTables& t, int R, const PublishLds&
 
 // The rank part as one flat pass over rank_counts ([rank][chunk], R * chunks_padded <= 4 * kThreads entries; in a
 // single-launch dispatch written through by counting workgroups of the same launch, each line by one writer, and not
-// touched by the caller's workgroup before those have finished, so ordinary loads fetch them): the exclusive prefix sum over the
-// flattened table is, at entry (r, c), the first compact row of rank r's tokens of chunk c; at (r, 0) it is the start
-// of rank r's bucket.  Every thread of the workgroup must call it.
-//   bases != nullptr: the prefix of every entry is stored there (LDS of a mover workgroup, or rank_bases in memory);
-//   s != nullptr:     the per-rank outputs are published (the publishing workgroup).
-// scan_tmp: kThreads / 64 ints of LDS.  Ends with a barrier.
+// touched by the caller's workgroup before those have finished, so ordinary loads fetch them): the inclusive prefix
+// sum over the flattened table is, at the last entry of row r, the end of rank r's bucket.  Publishes the per-rank
+// outputs.  Every thread of the workgroup must call it; s.scan_tmp: kThreads / 64 ints of LDS.
 template <int kThreads>
-__device__ void scan_rank_counts(const PublishParams* q, const LayoutTables& t, int R, int* bases, int* scan_tmp,
-                                 const PublishLds* s) {
+__device__ void scan_rank_counts(const PublishParams& q, const LayoutTables& t, int R, const PublishLds& s) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int flat = R * t.chunks_padded;              // a multiple of 4: a thread's entries share a row
     const int begin = tid * 4;
@@ -125,29 +121,19 @@ __device__ void scan_rank_counts(const PublishParams* q, const LayoutTables& t, 
     if (begin < flat) v = load16(t.rank_counts + begin);
     const int sum = int(v.x) + int(v.y) + int(v.z) + int(v.w);
     const int inc = wave_inclusive_sum(sum);
-    if (lane == kWaveSize - 1) scan_tmp[wave] = inc;
+    if (lane == kWaveSize - 1) s.scan_tmp[wave] = inc;
     __syncthreads();
     int run = inc - sum;
-    for (int w = 0; w < wave; ++w) run += scan_tmp[w];
-    if (begin < flat) {
-        if (bases != nullptr) {
-            bases[begin] = run;
-            bases[begin + 1] = run + int(v.x);
-            bases[begin + 2] = run + int(v.x) + int(v.y);
-            bases[begin + 3] = run + int(v.x) + int(v.y) + int(v.z);
-        }
-        if (s != nullptr && (begin + 4) % t.chunks_padded == 0) s->totals[begin / t.chunks_padded] = run + sum;   // inclusive prefix of the rank
-    }
+    for (int w = 0; w < wave; ++w) run += s.scan_tmp[w];
+    if (begin < flat && (begin + 4) % t.chunks_padded == 0) s.totals[begin / t.chunks_padded] = run + sum;   // inclusive prefix of the rank
     __syncthreads();
-    if (s != nullptr) {
-        for (int r = tid; r < R; r += kThreads) {
-            const int total = s->totals[r] - (r > 0 ? s->totals[r - 1] : 0);
-            if (q->num_tokens_per_rank != nullptr) q->num_tokens_per_rank[r] = total;
-            if (q->host_counts != nullptr) q->host_counts[r] = -total - 1;
-            if (q->psum_rank != nullptr) q->psum_rank[r] = s->totals[r];
-        }
-        if (tid == 0 && q->totals_out != nullptr) q->totals_out[0] = s->totals[R - 1];
+    for (int r = tid; r < R; r += kThreads) {
+        const int total = s.totals[r] - (r > 0 ? s.totals[r - 1] : 0);
+        if (q.num_tokens_per_rank != nullptr) q.num_tokens_per_rank[r] = total;
+        if (q.host_counts != nullptr) q.host_counts[r] = -total - 1;
+        if (q.psum_rank != nullptr) q.psum_rank[r] = s.totals[r];
     }
+    if (tid == 0 && q.totals_out != nullptr) q.totals_out[0] = s.totals[R - 1];
 }
 
 // ---- expert part: tables are [chunk][expert], so that thread e walks column e with coalesced accesses ----
@@ -194,12 +180,13 @@ __device__ void publish_experts(const PublishParams& q, const PublishLds& s) {
     if (q.host_counts != nullptr) __threadfence_system();
 }
 
-// expert_bases[c][e] = start of expert e's region + sum of expert_counts[0..c)[e].  kThrough: stored at agent scope.
+// table[c][e] = start of expert e's region + sum of expert_counts[0..c)[e], each word ORed with `tag`.
+// kThrough: stored at agent scope.
 template <int kThreads, bool kThrough>
-__device__ void write_expert_bases(const LayoutTables& t, int E, int num_chunks, const PublishLds& s) {
+__device__ void write_expert_bases(const LayoutTables& t, int32_t* table, uint32_t tag, int E, int num_chunks, const PublishLds& s) {
     for (int e = threadIdx.x; e < E; e += kThreads) {
         const int32_t* col = t.expert_counts + e;
-        int32_t* out = t.expert_bases + e;
+        int32_t* out = table + e;
         int run = s.aligned_incl[e] - s.aligned[e];
         for (int c0 = 0; c0 < num_chunks; c0 += 16) {
             int v[16];
@@ -208,7 +195,7 @@ __device__ void write_expert_bases(const LayoutTables& t, int E, int num_chunks,
 #pragma unroll
             for (int u = 0; u < 16; ++u) {
                 if (c0 + u < num_chunks) {
-                    store_word<kThrough>(out + int64_t(c0 + u) * t.experts_padded, run);
+                    store_word<kThrough>(out + int64_t(c0 + u) * t.experts_padded, int(uint32_t(run) | tag));
                     run += v[u];
                 }
             }
@@ -219,9 +206,10 @@ __device__ void write_expert_bases(const LayoutTables& t, int E, int num_chunks,
 // The expert base table in one trip, for the publishing workgroup of a single-launch expanded dispatch, whose movers
 // wait for exactly this: thread e keeps its column of chunk totals in registers between the sum and the stores.
 // Needs E <= kThreads and num_chunks <= 32.  Leaves totals / aligned / aligned_incl as publish_experts expects to
-// recompute them; stores at agent scope.  A: expert alignment.
+// recompute them; stores at agent scope, each word ORed with `tag`.  A: expert alignment.
 template <int kThreads>
-__device__ void write_expert_bases_from_registers(const LayoutTables& t, int R, int E, int A, int num_chunks, const PublishLds& s) {
+__device__ void write_expert_bases_from_registers(const LayoutTables& t, int32_t* table, uint32_t tag, int R, int E, int A,
+                                                  int num_chunks, const PublishLds& s) {
     const int e = threadIdx.x;
     int v[32];
     int total = 0;
@@ -239,12 +227,12 @@ __device__ void write_expert_bases_from_registers(const LayoutTables& t, int R, 
     __syncthreads();
     block_inclusive_scan<kThreads>(s.aligned_incl, E, s.scan_tmp);
     if (e < E) {
-        int32_t* out = t.expert_bases + e;
+        int32_t* out = table + e;
         int run = s.aligned_incl[e] - s.aligned[e];
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
             if (u < num_chunks) {
-                store_agent(out + int64_t(u) * t.experts_padded, run);
+                store_agent(out + int64_t(u) * t.experts_padded, int(uint32_t(run) | tag));
                 run += v[u];
             }
         }
@@ -264,7 +252,7 @@ __device__ void publish_layout(const PublishParams& q, const LayoutTables& t, in
     publish_experts<kThreads>(q, s);
     if (t.expert_bases != nullptr && expert_bases) {
         __syncthreads();
-        write_expert_bases<kThreads, false>(t, q.E, num_chunks, s);
+        write_expert_bases<kThreads, false>(t, t.expert_bases, 0u, q.E, num_chunks, s);
     }
 }
 

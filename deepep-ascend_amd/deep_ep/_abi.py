@@ -239,6 +239,7 @@ EXPORTS = {
     "deep_ep_hip_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "deep_ep_hip_workspace_status_offset": (c_size_t, []),
     "deep_ep_hip_workspace_control_bytes": (c_size_t, []),
+    "deep_ep_hip_workspace_counter_bytes": (c_size_t, []),
     "deep_ep_hip_read_status": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "deep_ep_hip_launch_layout": (c_int, [POINTER(LayoutArgs), c_void_p]),
     "deep_ep_hip_launch_dispatch": (c_int, [POINTER(DispatchArgs), c_void_p]),

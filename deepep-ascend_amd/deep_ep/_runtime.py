@@ -222,10 +222,11 @@ class ElasticBuffer:
         return True
 
     def workspace_control_words(self) -> torch.Tensor:
-        """The bookkeeping words at the head of the workspace (status, launch protocol), copied to the host after a full
-        synchronisation: between launches everything but the status word and the two row totals reads zero."""
+        """The counters and flags at the head of the workspace (status, launch protocol), copied to the host after a full
+        synchronisation: between launches everything but the status word (word 0), the two row totals (words 2 and 3) and
+        the launch generation (word 32) reads zero."""
         torch.cuda.synchronize(self.device)
-        n = _abi.lib.deep_ep_hip_workspace_control_bytes()
+        n = _abi.lib.deep_ep_hip_workspace_counter_bytes()
         if self._workspace is None:
             return torch.zeros(n // 4, dtype=torch.int32)
         return self._workspace[:n].view(torch.int32).cpu()

@@ -1,6 +1,6 @@
 """The single-launch dispatch (layout and move in one call without a host wait: counting workgroups ride at the front
-of the move kernel and hand the layout to the movers through gates in the workspace) against the CPU oracle, and
-the state it must leave behind: every launch finds and leaves the bookkeeping words of the workspace at zero."""
+of the move kernel and hand the layout to the movers through tagged words in the workspace) against the CPU oracle,
+and the state it must leave behind: every launch finds and leaves the counters and flags of the workspace at zero."""
 import pytest
 import torch
 
@@ -17,6 +17,7 @@ FUSED = ["C1", "C2", "tiny_masked", "one_token", "k1_e_eq_r", "ragged_chunks", "
 def _control_words(buf):
     words = buf.runtime.workspace_control_words().clone()
     words[2:4] = 0          # the two row totals a dispatch leaves for the kernels that follow it
+    words[32] = 0           # the launch generation
     return words
 
 
@@ -66,8 +67,8 @@ def test_single_launch_matches_the_oracle(name, do_expand, payload, monkeypatch)
 
 
 def test_launches_of_changing_shape_share_one_workspace(monkeypatch):
-    """Gates, flags and tables are reused by launches of different token counts, layouts and launch modes; each must
-    find them clean."""
+    """Counters, flags and tables are reused by launches of different token counts, layouts and launch modes; no launch
+    may take a word an earlier one left behind for its own."""
     import deep_ep
     E, R, K, H = 32, 4, 6, 512
     buf = deep_ep.ElasticBuffer(deep_ep.LogicalGroup(1, R), num_max_tokens_per_rank=4096, hidden=H, num_topk=K)
@@ -83,8 +84,9 @@ def test_launches_of_changing_shape_share_one_workspace(monkeypatch):
 
 
 def test_many_back_to_back_launches_without_host_sync(monkeypatch):
-    """50 single-launch dispatches queued without a host wait in between: the gates of launch n must have wrapped to
-    zero before launch n + 1 reads them (stream order), whatever the number of movers per gate."""
+    """50 single-launch dispatches queued without a host wait in between: the counters of launch n must have wrapped to
+    zero and its generation must have advanced before launch n + 1 starts (stream order), whatever the number of
+    movers per gate."""
     import deep_ep
     monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", 1)
     case = rc.small("b2b", 1500, 1024, 64, 8, 8, seed=77, masked_ratio=0.05)
@@ -97,4 +99,45 @@ def test_many_back_to_back_launches_without_host_sync(monkeypatch):
         assert_equal(recv[:ref.num_recv_tokens], ref.recv_x, "recv_x")
         assert_equal(handle.dst_buffer_slot_idx, ref.dst_buffer_slot_idx, "dst_buffer_slot_idx")
     buf.check_device_status()
+    assert int(_control_words(buf).abs().sum()) == 0
+
+
+def test_the_launch_tag_wraps_without_taking_a_stale_word(monkeypatch):
+    """The words counting workgroups hand to the movers carry the launch's tag, 1 .. 16383; the launch that uses the
+    last tag clears the tagged tables and the count starts over.  More launches than there are tags, of three
+    alternating shapes and both layouts (so that words of older launches lie about under every tag, beyond the token
+    range of the smaller shapes too): the launches around the wrap and the last one must be exact, and the generation
+    word must read launches mod 16383."""
+    import deep_ep
+    monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", 1)
+    period = 16383
+    E, R, K, H = 16, 4, 4, 128
+    buf = deep_ep.ElasticBuffer(deep_ep.LogicalGroup(2, R), num_max_tokens_per_rank=1024, hidden=H, num_topk=K)
+    cases, refs = [], {}
+    for i, T in enumerate((700, 40, 300)):           # the largest first: the buffer sizes its workspace on first use
+        case = rc.small(f"wrap{T}", T, H, E, R, K, seed=500 + T, masked_ratio=0.1)
+        case.M = 1024
+        cases.append((case, case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()))
+        for do_expand in (False, True):
+            refs[i, do_expand] = oracle.dispatch(case.x, case.topk_idx, case.topk_weights, E, R, buf.rank_idx, case.M,
+                                                 do_expand=do_expand, expert_alignment=2)
+    assert int(buf.runtime.workspace_control_words()[32]) == 0
+    launches = period + 150
+    kept = {}
+    for n in range(launches):
+        i, do_expand = n % 3, (n // 3) % 2 == 1
+        case, x, idx, w = cases[i]
+        out = buf.dispatch(x, idx, w, num_experts=E, do_cpu_sync=False, do_expand=do_expand, expert_alignment=2)
+        if n < 4 or abs(n - period) < 40 or n >= launches - 6:
+            kept[n] = (i, do_expand, out)
+    torch.cuda.synchronize()
+    buf.check_device_status()
+    assert int(buf.runtime.workspace_control_words()[32]) == launches % period
+    for n, (i, do_expand, (recv, ridx, rw, handle, _)) in kept.items():
+        ref = refs[i, do_expand]
+        rows = ref.num_expanded_tokens if do_expand else ref.num_recv_tokens
+        valid = ref.expanded_row_is_valid if do_expand else torch.ones(rows, dtype=torch.bool)
+        assert_equal(recv[:rows].cpu()[valid], ref.recv_x[valid], f"recv_x of launch {n}")
+        assert_equal(handle.dst_buffer_slot_idx, ref.dst_buffer_slot_idx, f"dst_buffer_slot_idx of launch {n}")
+        assert_equal(handle.recv_src_metadata[:ref.num_recv_tokens], ref.recv_src_metadata, f"recv_src_metadata of launch {n}")
     assert int(_control_words(buf).abs().sum()) == 0

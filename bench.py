@@ -288,8 +288,8 @@ def main():
                      "achieved": round(gbs(ab["combine"], combine_us), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs(ab["combine"], combine_us) / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(traffic_key + ("combine",))},
-        "roofline_dispatch": {"kernel": ("dispatch_cast_kernel" if fp8 else "dispatch_copy_kernel") +
-                                        " (whole call: one launch where the single launch applies, else layout_kernel + this)",
+        "roofline_dispatch": {"kernel": ("dispatch_cast" if fp8 else "dispatch_copy") + "_single_launch_kernel (whole call; where the "
+                                        "single launch does not apply: layout_kernel + " + ("dispatch_cast_kernel)" if fp8 else "dispatch_copy_kernel)"),
                               "bound": "hbm", "achieved": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us), 1),
                               "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round(gbs(ab["layout"] + ab["dispatch"], dispatch_us) / HBM_PEAK_GBS, 4),

@@ -108,6 +108,8 @@ void fill_fused(MoveParams& m, const LayoutParams& lay, const LaunchPlan& plan, 
     m.pos = reinterpret_cast<const uint32_t*>(ws + w.tagged_pos);
     m.lay.pos = reinterpret_cast<uint32_t*>(ws + w.tagged_pos);
     m.lay.tagged_rank = reinterpret_cast<uint32_t*>(ws + w.tagged_rank);
+    m.tagged_expert_counts = reinterpret_cast<const uint32_t*>(ws + w.tagged_expert_counts);
+    m.lay.tagged_expert_counts = m.do_expand ? reinterpret_cast<uint32_t*>(ws + w.tagged_expert_counts) : nullptr;
     m.lay.generation = m.generation;
 }
 
@@ -134,6 +136,7 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.tagged_rank = off;   off += size_t(kTaggedRankWords) * 4;
     w.tagged_expert = off; off += size_t(kTaggedExpertWords) * 4;
     w.tagged_pos = off;    off += size_t(kTaggedPosWords) * 4;
+    w.tagged_expert_counts = off; off += size_t(kTaggedExpertWords) * 4;
     w.tagged_end = off;
     w.expert_start = off;  off = align_up(off + size_t(num_experts) * 4, 256);
     const size_t experts_padded = (size_t(num_experts) + 31) / 32 * 32;

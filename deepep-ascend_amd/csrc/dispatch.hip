@@ -19,6 +19,7 @@
 // those.  Counting workgroups have the lowest workgroup ids, wait for nothing and are therefore resident
 // before any mover can wait for them; every wait is bounded.
 #include <algorithm>
+#include <atomic>
 
 #include "device_utils.h"
 #include "fp8_cast.h"
@@ -296,10 +297,6 @@ __device__ __forceinline__ uint32_t launch_tag(const uint32_t* generation) {
     return (uint32_t(load_agent(reinterpret_cast<const int*>(generation))) + 1u) << kTagShift;
 }
 
-__device__ __forceinline__ bool has_tag(uint32_t word, uint32_t tag) {
-    return (word & ~kTagValueMask) == tag;
-}
-
 __device__ __forceinline__ uint64_t load_agent64(const void* p) {
     return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -340,13 +337,19 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     const uint32_t tag = launch_tag(p.generation);
     int32_t* tagged_bases = reinterpret_cast<int32_t*>(p.tagged_expert);
 
-    await_and_clear_flags(p, p.chunk_done, p.count_blocks);
-
-    // The expert part first: the movers of an expanded dispatch are waiting for its base table, which therefore goes
-    // out before any of the call's outputs.  (The count tables have one writer per cache line and this workgroup has
-    // not touched them before, so ordinary loads fetch what the counting workgroups wrote through.)
+    // The movers of an expanded dispatch are waiting for the expert base table, which therefore goes out before
+    // anything else, from the tagged chunk totals as they arrive.
     const bool bases_first = p.do_expand && p.E <= kThreads && p.count_blocks <= 32;
-    if (bases_first) write_expert_bases_from_registers<kThreads>(tab, tagged_bases, tag, p.R, p.E, p.pub.A, p.count_blocks, lds);
+    if (bases_first) {
+        const bool complete = write_expert_bases_from_registers<kThreads>(tab, p.tagged_expert_counts, tagged_bases, tag, kLayoutSpinLimit,
+                                                                          p.R, p.E, p.pub.A, p.count_blocks, lds);
+        if (!complete && threadIdx.x == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+    }
+
+    // Everything else reads the count tables with ordinary loads, once the counting workgroups have flagged that their
+    // stores are acknowledged.  (The tables have one writer per cache line and this workgroup has not touched them
+    // before, so ordinary loads fetch what was written through.)
+    await_and_clear_flags(p, p.chunk_done, p.count_blocks);
     sum_expert_columns<kThreads>(tab, p.R, p.E, p.count_blocks, lds.totals);
     publish_experts<kThreads>(p.pub, lds);
     if (p.do_expand && !bases_first) {
@@ -358,7 +361,9 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
 }
 
 // What a mover reads of the layout before the layout is known to be there: issued ahead of the payload loads, so
-// that a mover that starts after the layout is complete (most of them) has paid no extra trip for it.
+// that a mover that starts after the layout is complete (most of them) has paid no extra trip for it.  Ordinary
+// loads, which this XCD's L2 may answer: a word that shows the tag of this launch is this launch's word wherever it
+// was cached, and one that does not is read again at agent scope.
 struct FirstLook {
     uint64_t totals_lo, totals_hi;     // this thread's four chunk totals
     uint32_t position;                 // this lane's position word
@@ -368,10 +373,11 @@ __device__ __forceinline__ FirstLook first_look(const MoveParams& p, int t, int 
     FirstLook f{0, 0, 0};
     const int begin = int(threadIdx.x) * 4;
     if (begin < p.R * p.tab.chunks_padded) {
-        f.totals_lo = load_agent64(p.tagged_rank + begin);
-        f.totals_hi = load_agent64(p.tagged_rank + begin + 2);
+        const vec16 v = load16(p.tagged_rank + begin);
+        f.totals_lo = uint64_t(v.x) | (uint64_t(v.y) << 32);
+        f.totals_hi = uint64_t(v.z) | (uint64_t(v.w) << 32);
     }
-    if (has_work && lane < p.K) f.position = uint32_t(load_agent(reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane));
+    if (has_work && lane < p.K) f.position = p.pos[int64_t(t) * p.K + lane];
     return f;
 }
 
@@ -384,32 +390,20 @@ __device__ __forceinline__ bool look_is_complete(const MoveParams& p, const Firs
     return __all(ok);
 }
 
-// Every mover workgroup works the rank bases out for itself, into its LDS: thread i waits (bounded) for chunk totals
-// 4i .. 4i + 3 of the flattened [rank][chunk] table to show the tag, then the workgroup takes the exclusive prefix
-// sum.  All threads; ends with a barrier.  Returns false when the wait ran out.
-__device__ __forceinline__ bool build_rank_bases(const MoveParams& p, uint32_t tag, const FirstLook& look, const int*& bases_out) {
+__device__ __forceinline__ bool totals_tagged(uint64_t lo, uint64_t hi, uint32_t tag) {
+    return has_tag(uint32_t(lo), tag) && has_tag(uint32_t(lo >> 32), tag) && has_tag(uint32_t(hi), tag) && has_tag(uint32_t(hi >> 32), tag);
+}
+
+// Every mover workgroup works the rank bases out for itself, into its LDS: the exclusive prefix sum over the flattened
+// [rank][chunk] table of chunk totals, of which thread i brings entries 4i .. 4i + 3 (tags still on).  `complete`: this
+// thread's waits all ended well.  All threads; ends with a barrier.  Returns whether every thread's did.
+__device__ __forceinline__ bool build_rank_bases(const MoveParams& p, uint64_t lo, uint64_t hi, bool complete, const int*& bases_out) {
     extern __shared__ uint64_t count_lds[];
     int* bases = reinterpret_cast<int*>(count_lds);
     const int flat = p.R * p.tab.chunks_padded;           // a multiple of 4: a thread's entries share a row
     int* scan_tmp = bases + flat;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int begin = tid * 4;
-    uint64_t lo = look.totals_lo, hi = look.totals_hi;
-    bool complete = true;
-    if (begin < flat) {
-        unsigned polls = 0;
-        auto tagged = [&]() {
-            return has_tag(uint32_t(lo), tag) && has_tag(uint32_t(lo >> 32), tag) && has_tag(uint32_t(hi), tag) &&
-                   has_tag(uint32_t(hi >> 32), tag);
-        };
-        while (!tagged() && polls < kLayoutSpinLimit) {
-            __builtin_amdgcn_s_sleep(2);
-            lo = load_agent64(p.tagged_rank + begin);
-            hi = load_agent64(p.tagged_rank + begin + 2);
-            ++polls;
-        }
-        complete = tagged();
-    }
     const int v0 = int(uint32_t(lo) & kTagValueMask), v1 = int(uint32_t(lo >> 32) & kTagValueMask);
     const int v2 = int(uint32_t(hi) & kTagValueMask), v3 = int(uint32_t(hi >> 32) & kTagValueMask);
     const int sum = v0 + v1 + v2 + v3;
@@ -427,18 +421,6 @@ __device__ __forceinline__ bool build_rank_bases(const MoveParams& p, uint32_t t
     __syncthreads();
     bases_out = bases;
     return all_complete != 0;
-}
-
-// A wavefront's wait (bounded) for words of its own lanes: `word` holds each lane's first read of `at`; lanes with
-// wanted == false take no part.  Returns false when the wait ran out.
-__device__ __forceinline__ bool await_tagged_word(const int* at, bool wanted, uint32_t tag, uint32_t& word) {
-    unsigned polls = 0;
-    while (__any(wanted && !has_tag(word, tag)) && polls < kLayoutSpinLimit) {
-        __builtin_amdgcn_s_sleep(1);
-        if (wanted && !has_tag(word, tag)) word = uint32_t(load_agent(at));
-        ++polls;
-    }
-    return !__any(wanted && !has_tag(word, tag));
 }
 
 // The mover workgroup is done reading tagged words: its first thread advances the gate.  The value the gate had is
@@ -464,6 +446,69 @@ __device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover,
     store_agent(reinterpret_cast<int*>(p.generation), int(next));
 }
 
+// A wavefront's wait (bounded) for the tagged words its threads want.  Returns whether this thread still misses one.
+// While the layout is not there, thousands of wavefronts repeat their reads, and every request of theirs stands in
+// front of the counting workgroups' stores somewhere: so a waiting wavefront first watches the one kind of word that
+// comes last - the expert base of its first routing lane, else its token's position words: one 32-byte request per
+// round - and only when that has arrived reads the rest again, whatever is still missing in one trip per round.
+__device__ __forceinline__ bool await_tagged_words(uint32_t tag, bool wants_position, const int* position_at, uint32_t& position,
+                                                   bool wants_totals, const uint32_t* totals_at, uint64_t& lo, uint64_t& hi,
+                                                   bool wants_base, const int* base_at, uint32_t& base_word) {
+    unsigned polls = 0;
+    const uint64_t base_lanes = __ballot(wants_base);
+    if (base_lanes != 0) {
+        const bool watches = wants_base && lane_id() == __builtin_ctzll(base_lanes);
+        while (__any(watches && !has_tag(base_word, tag)) && polls < kLayoutSpinLimit) {
+            __builtin_amdgcn_s_sleep(4);
+            if (watches) base_word = uint32_t(load_agent(base_at));
+            ++polls;
+        }
+    } else {
+        while (__any(wants_position && !has_tag(position, tag)) && polls < kLayoutSpinLimit) {
+            __builtin_amdgcn_s_sleep(4);
+            if (wants_position && !has_tag(position, tag)) position = uint32_t(load_agent(position_at));
+            ++polls;
+        }
+    }
+    bool missing;
+    for (;;) {
+        const bool no_position = wants_position && !has_tag(position, tag);
+        const bool no_totals = wants_totals && !totals_tagged(lo, hi, tag);
+        const bool no_base = wants_base && !has_tag(base_word, tag);
+        missing = no_position || no_totals || no_base;
+        if (!__any(missing) || polls >= kLayoutSpinLimit) break;
+        if (polls != 0) __builtin_amdgcn_s_sleep(1);
+        if (no_position) position = uint32_t(load_agent(position_at));
+        if (no_totals) {
+            lo = load_agent64(totals_at);
+            hi = load_agent64(totals_at + 2);
+        }
+        if (no_base) base_word = uint32_t(load_agent(base_at));
+        ++polls;
+    }
+    return missing;
+}
+
+// Mover workgroups that run beside a counting or the publishing workgroup on one CU read nothing but the layout until
+// the layout is there.  A CU's vector memory pipeline takes the requests of all its wavefronts in order, and the payload
+// loads of seven mover workgroups keep it busy for microseconds: stores of a counting workgroup that shares the CU
+// queue up behind them (measured: positions issued 3.5 us after the launch on a quiet CU, 6 to 8 us beside prefetching
+// movers), and every mover of the launch waits for those stores.  Workgroups are handed to the CUs breadth first -
+// workgroup i of a launch starts on CU i % num_cus while the first seven or eight per CU are being placed (read back
+// from the hardware id registers on MI355X) - so the neighbours of workgroups 0 .. count_blocks are known by index.
+// Should a GPU place workgroups differently, the rule holds back other movers: slower, never wrong.
+__device__ __forceinline__ bool shares_cu_with_layout_work(const MoveParams& p) {
+    return blockIdx.x % unsigned(p.num_cus) <= unsigned(p.count_blocks) && blockIdx.x < unsigned(p.num_cus) * 8u;
+}
+
+// Such a workgroup's wait (bounded; await_layout reports a wait that ran out): repeats the first look until it is complete.
+__device__ __forceinline__ void hold_for_layout(const MoveParams& p, uint32_t tag, FirstLook& look, int t, int lane, bool has_work) {
+    uint32_t no_base = 0;
+    const int begin = int(threadIdx.x) * 4;
+    await_tagged_words(tag, has_work && lane < p.K, reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane, look.position,
+                       begin < p.R * p.tab.chunks_padded, p.tagged_rank + begin, look.totals_lo, look.totals_hi, false, nullptr, no_base);
+}
+
 // Everything a mover wavefront needs from the layout of its own launch.
 struct FusedLayout {
     const int* flat_bases;    // LDS: exclusive prefix over the chunk totals of the rank buckets
@@ -477,29 +522,37 @@ struct FusedLayout {
 __device__ __forceinline__ FusedLayout await_layout(const MoveParams& p, unsigned mover, const FirstLook& look, uint32_t tag,
                                                     const RouteInputs& in, int t, int lane, bool has_work) {
     FusedLayout f{nullptr, look.position, 0, 0u, tag, true};
-    // position words: each wavefront waits for those of its own token
+    // What this thread waits for: the position word of its lane, four chunk totals, and for the expanded layout the
+    // base of its lane's (chunk, expert).  Whatever is missing is read again, all of it in one trip per round.
     const bool wants_position = has_work && lane < p.K;
-    bool complete = await_tagged_word(reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane, wants_position, tag, f.position);
+    const int* position_at = reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane;
+    const int begin = int(threadIdx.x) * 4;
+    const bool wants_totals = begin < p.R * p.tab.chunks_padded;
+    uint64_t lo = look.totals_lo, hi = look.totals_hi;
+    bool wants_base = false;
+    const int* base_at = nullptr;
+    uint32_t base_word = 0;
     if (p.do_expand) {
-        int64_t e = p.route_mask != nullptr ? (in.mask_byte != 0 ? int64_t(lane) : int64_t(-1)) : in.raw;
-        const bool wants_base = wants_position && e >= 0 && e < p.E;
-        const int* at = reinterpret_cast<const int*>(p.tagged_expert) + int64_t(t / kLayoutChunk) * p.tab.experts_padded + (wants_base ? int(e) : 0);
-        uint32_t word = wants_base ? uint32_t(load_agent(at)) : 0u;
-        complete = await_tagged_word(at, wants_base, tag, word) && complete;
-        f.expert_base = int(word & kTagValueMask);
+        const int64_t e = p.route_mask != nullptr ? (in.mask_byte != 0 ? int64_t(lane) : int64_t(-1)) : in.raw;
+        wants_base = wants_position && e >= 0 && e < p.E;
+        base_at = reinterpret_cast<const int*>(p.tagged_expert) + int64_t(t / kLayoutChunk) * p.tab.experts_padded + (wants_base ? int(e) : 0);
+        if (wants_base) base_word = uint32_t(*base_at);       // an ordinary load first, as in first_look
     }
-    complete = build_rank_bases(p, tag, look, f.flat_bases) && complete;      // ends with a workgroup barrier
-    if (threadIdx.x == 0) f.gate_seen = advance_gate(p, mover);
-    // One wavefront's failure is the workgroup's: build_rank_bases has already combined the threads' waits for the
-    // totals; a wait for a position or an expert base that ran out stops that wavefront only.
-    if (!complete && lane == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+    const bool missing = await_tagged_words(tag, wants_position, position_at, f.position, wants_totals, p.tagged_rank + begin, lo, hi,
+                                            wants_base, base_at, base_word);
+    f.expert_base = int(base_word & kTagValueMask);
+    const bool complete = build_rank_bases(p, lo, hi, !missing, f.flat_bases);      // ends with a workgroup barrier
+    if (threadIdx.x == 0) {
+        f.gate_seen = advance_gate(p, mover);
+        if (!complete) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+    }
     f.complete = complete;
     return f;
 }
 
 // ---- pass-through payload (BF16, or FP8 with caller-provided scale packs) ----
 template <int kVecs, bool kFused>
-__global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
+__device__ __forceinline__ void dispatch_copy(const MoveParams& p) {
     if constexpr (kFused) {
         if (blockIdx.x <= unsigned(p.count_blocks)) {
             if (blockIdx.x < unsigned(p.count_blocks)) fused_count_block(p);
@@ -520,6 +573,7 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
     if constexpr (kFused) {
         tag = launch_tag(p.generation);
         look = first_look(p, t, lane, has_work);
+        if (shares_cu_with_layout_work(p)) hold_for_layout(p, tag, look, t, lane, has_work);
     }
 
     vec16 v[kVecs];
@@ -577,7 +631,7 @@ __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParam
 
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
 template <int kPairs, bool kFused>
-__global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
+__device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
     if constexpr (kFused) {
         if (blockIdx.x <= unsigned(p.count_blocks)) {
             if (blockIdx.x < unsigned(p.count_blocks)) fused_count_block(p);
@@ -598,6 +652,7 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
     if constexpr (kFused) {
         tag = launch_tag(p.generation);
         look = first_look(p, t, lane, has_work);
+        if (shares_cu_with_layout_work(p)) hold_for_layout(p, tag, look, t, lane, has_work);
     }
 
     vec16 in[kPairs][2];
@@ -682,6 +737,26 @@ __global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParam
     }
     if constexpr (kFused)
         if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+}
+
+// The kernels.  The single-launch forms also hold the counting and publishing code, whose register needs must not cost
+// the movers their occupancy: they are held to six wavefronts per SIMD (80 registers), the number the movers' own code
+// reaches; five resident workgroups per CU are what the move needs to saturate the memory pipeline.
+template <int kVecs>
+__global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
+    dispatch_copy<kVecs, false>(p);
+}
+template <int kVecs>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void dispatch_copy_single_launch_kernel(const MoveParams p) {
+    dispatch_copy<kVecs, true>(p);
+}
+template <int kPairs>
+__global__ __launch_bounds__(kThreads) void dispatch_cast_kernel(const MoveParams p) {
+    dispatch_cast<kPairs, false>(p);
+}
+template <int kPairs>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void dispatch_cast_single_launch_kernel(const MoveParams p) {
+    dispatch_cast<kPairs, true>(p);
 }
 
 // ---- zero the alignment padding rows of the expanded layout ----
@@ -795,8 +870,8 @@ template <int kVecs>
 hipError_t launch_copy(MoveParams p, hipStream_t stream) {
     p.tiles = (p.row_bytes + kVecs * 1024 - 1) / (kVecs * 1024);
     const unsigned blocks = move_grid(p, int64_t(p.T) * p.tiles);
-    if (p.fused) hipLaunchKernelGGL((dispatch_copy_kernel<kVecs, true>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
-    else hipLaunchKernelGGL((dispatch_copy_kernel<kVecs, false>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    if (p.fused) hipLaunchKernelGGL((dispatch_copy_single_launch_kernel<kVecs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    else hipLaunchKernelGGL((dispatch_copy_kernel<kVecs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 
@@ -804,8 +879,8 @@ template <int kPairs>
 hipError_t launch_cast(MoveParams p, hipStream_t stream) {
     p.tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
     const unsigned blocks = move_grid(p, int64_t(p.T) * p.tiles);
-    if (p.fused) hipLaunchKernelGGL((dispatch_cast_kernel<kPairs, true>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
-    else hipLaunchKernelGGL((dispatch_cast_kernel<kPairs, false>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    if (p.fused) hipLaunchKernelGGL((dispatch_cast_single_launch_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    else hipLaunchKernelGGL((dispatch_cast_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 
@@ -837,9 +912,24 @@ int64_t dispatch_move_workgroups(const MoveParams& p) {
     return (int64_t(p.T) * tiles + kWavesPerBlock - 1) / kWavesPerBlock;
 }
 
+// Compute units of the current device (asked once per device).
+static int compute_units() {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cached[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
     p.rcp_E_l = 1.0f / float(p.E_l);
+    p.num_cus = p.fused ? compute_units() : 0;
     const int tile = move_tile(p);
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
         switch (tile) {

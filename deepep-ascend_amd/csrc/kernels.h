@@ -46,6 +46,7 @@ struct WorkspaceLayout {
                            // status, totals and generation
     size_t tagged_rank;    // uint32[kTaggedRankWords]: rank_counts of the running single-launch dispatch, tagged
     size_t tagged_expert;  // uint32[kTaggedExpertWords]: its expert_bases, tagged
+    size_t tagged_expert_counts;   // uint32[kTaggedExpertWords]: expert_counts of an expanded single-launch dispatch, tagged
     size_t tagged_pos;     // uint32[kTaggedPosWords]: its position words, tagged
     size_t tagged_end;
     size_t expert_start;   // int32[E]: first expanded row of each expert
@@ -107,6 +108,7 @@ struct LayoutParams {
     // Single-launch dispatch (else NULL): chunk totals of the rank buckets go to tagged_rank as well, tagged like the
     // position words, with the tag *generation names when the workgroup starts.
     uint32_t* tagged_rank;
+    uint32_t* tagged_expert_counts;  // expanded layout (else NULL): likewise the chunk totals of the expert buckets, for the publisher
     const uint32_t* generation;
 };
 
@@ -150,6 +152,7 @@ struct MoveParams {
     int fused;
     int count_blocks;
     unsigned num_movers;     // mover workgroups (set by the launcher)
+    int num_cus;             // compute units of the device (set by the launcher)
     LayoutParams lay;        // what the counting workgroups need (lay.pub is unused: `pub` above is published)
     int32_t* chunk_done;     // [kMaxCountBlocks] flags of the counting workgroups for the publisher: totals and positions stored
     uint32_t* gates;         // [kDispatchGates] wrapping counters of the movers that are done reading, kDispatchGateStride words apart
@@ -159,6 +162,7 @@ struct MoveParams {
     int tagged_words;
     const uint32_t* tagged_rank;
     uint32_t* tagged_expert;
+    const uint32_t* tagged_expert_counts;
     // V1 (intranode) conventions
     int rank_lanes;          // routing lanes are ranks (mask routing or a cached send_head), K == R
     int slot_is_row;         // cached_slot holds rows of the receive buffer, not rank * M + slot

@@ -70,21 +70,41 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
     for (int i = tid; i < n * kWaves; i += kThreads) bitmap[i] = 0ull;
     __syncthreads();
 
+    // Straight-line code from here on, no branch per routing lane: the LDS atomics of all lanes issue back to back, and
+    // so do the LDS reads of the position step further down.  A lane without an expert ORs nothing into a word of its
+    // own (not one word for all of them: atomics of one wavefront on one address take turns).
+    // With few ranks most lanes of a wavefront would meet on the same few rank words, so the rank bitmaps are taken by
+    // ballot instead: one per rank over "this token goes to rank r", no atomics.
+    constexpr int kBallotRanks = 16;
+    const bool ranks_by_ballot = p.R <= kBallotRanks;
     int e[KMAX], d[KMAX];
     int flags = 0;
     const float rcp_experts_per_rank = 1.0f / float(p.E_l);
     const uint64_t my_bit = 1ull << lane;
+    const int idle_word = min(lane, n * kWaves - 1);
+    uint64_t my_ranks = 0;                       // bit r: this token goes to rank r
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
-        int ev = -1;
+        const bool valid = raw[k] >= 0 && raw[k] < p.E;
         if (raw[k] >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
-        else if (raw[k] >= 0) ev = int(raw[k]);
-        e[k] = ev;
-        d[k] = ev >= 0 ? small_div(ev, rcp_experts_per_rank) : -1;
-        if (ev >= 0) {
-            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[(p.R + ev) * kWaves + wave]), my_bit);
-            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[d[k] * kWaves + wave]), my_bit);
+        e[k] = valid ? int(raw[k]) : -1;
+        d[k] = valid ? small_div(e[k], rcp_experts_per_rank) : -1;
+        const uint64_t bit = valid ? my_bit : 0ull;
+        atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[valid ? (p.R + e[k]) * kWaves + wave : idle_word]), bit);
+        if (valid) my_ranks |= 1ull << (d[k] & 63);            // used when num_ranks <= kBallotRanks
+    }
+    if (ranks_by_ballot) {
+        uint64_t mine = 0;
+        for (int r = 0; r < p.R; ++r) {
+            const uint64_t members = __ballot((my_ranks >> r) & 1ull);
+            if (lane == r) mine = members;
         }
+        if (lane < p.R) bitmap[lane * kWaves + wave] = mine;
+    } else {
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+            atomicOr(reinterpret_cast<unsigned long long*>(&bitmap[d[k] >= 0 ? d[k] * kWaves + wave : idle_word]),
+                     d[k] >= 0 ? my_bit : 0ull);
     }
     if (p.copied_topk_idx != nullptr && active) {
 #pragma unroll
@@ -103,9 +123,13 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
         int32_t* at = j < p.R ? p.tab.rank_counts + int64_t(j) * p.tab.chunks_padded + chunk
                               : p.tab.expert_counts + int64_t(chunk) * p.tab.experts_padded + (j - p.R);
         store_word<kThrough>(at, c0 + c1 + c2 + c3);
-        if constexpr (kThrough)
+        if constexpr (kThrough) {
             if (j < p.R && p.tagged_rank != nullptr)
                 store_agent(reinterpret_cast<int*>(p.tagged_rank) + j * p.tab.chunks_padded + chunk, int(uint32_t(c0 + c1 + c2 + c3) | tag));
+            if (j >= p.R && p.tagged_expert_counts != nullptr)
+                store_agent(reinterpret_cast<int*>(p.tagged_expert_counts) + chunk * p.tab.experts_padded + (j - p.R),
+                            int(uint32_t(c0 + c1 + c2 + c3) | tag));
+        }
     }
     const int pad = p.tab.chunks_padded - num_chunks;  // the padding columns of the rank table are cleared by the first workgroup
     if (chunk == 0) {
@@ -120,9 +144,10 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
 
     const uint64_t below = lanes_below(lane);
     const int wave_shift = wave > 0 ? 10 * (wave - 1) : 0;
-    auto rank_in_chunk = [&](int bucket) {
-        const int earlier = wave > 0 ? int((before_wave[bucket] >> wave_shift) & 0x3ffu) : 0;
-        return __popcll(bitmap[bucket * kWaves + wave] & below) + earlier;
+    const uint32_t earlier_mask = wave > 0 ? 0x3ffu : 0u;
+    // Position inside the chunk = bits of this wavefront's word below the lane + bits of the wavefronts before it.
+    auto position = [&](uint64_t word, uint32_t before) {
+        return uint32_t(__popcll(word & below)) + ((before >> wave_shift) & earlier_mask);
     };
 
     if (active) {
@@ -130,20 +155,54 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
             // One word per (token, lane): the slot of the token inside its chunk for the lane's destination rank
             // (master lanes only) and the position of the lane inside its chunk for its expert (kernels.h).
             uint32_t packed[KMAX];
+            uint64_t word_r[KMAX];
+            uint32_t before_r[KMAX];
 #pragma unroll
             for (int k = 0; k < KMAX; ++k) {
-                uint32_t pr = kNoPosition, pe = kNoPosition;
-                if (e[k] >= 0) {
-                    bool master = true;
+                const int bucket = d[k] >= 0 ? d[k] : 0;
+                word_r[k] = bitmap[bucket * kWaves + wave];
+                before_r[k] = before_wave[bucket];
+            }
+            // The master lane of a destination rank is the last lane that names it.
+            bool master[KMAX];
+            if (p.R <= 64) {
+                // walk the lanes backwards with the set of ranks seen so far
+                uint64_t later_ranks = 0;
 #pragma unroll
-                    for (int j = 0; j < KMAX; ++j) {
-                        if (j > k && d[j] == d[k]) master = false;
-                        if (j != k && e[j] == e[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
-                    }
-                    if (p.expert_bases) pe = uint32_t(rank_in_chunk(p.R + e[k]));      // only the expanded layout places rows by expert
-                    if (master) pr = uint32_t(rank_in_chunk(d[k]));
+                for (int k = KMAX - 1; k >= 0; --k) {
+                    const uint64_t rank_bit = d[k] >= 0 ? 1ull << (d[k] & 63) : 0ull;
+                    master[k] = (rank_bit & ~later_ranks) != 0;
+                    later_ranks |= rank_bit;
                 }
-                packed[k] = pr | (pe << kExpertPositionShift) | tag;
+            } else {
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k) {
+                    master[k] = d[k] >= 0;
+#pragma unroll
+                    for (int j = k + 1; j < KMAX; ++j)
+                        if (d[j] == d[k]) master[k] = false;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) {
+#pragma unroll
+                for (int j = k + 1; j < KMAX; ++j)
+                    if (e[k] >= 0 && e[j] == e[k]) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+                packed[k] = (master[k] ? position(word_r[k], before_r[k]) : kNoPosition) | tag;
+            }
+            if (p.expert_bases) {                         // only the expanded layout places rows by expert
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k) {
+                    const int bucket = e[k] >= 0 ? p.R + e[k] : 0;
+                    word_r[k] = bitmap[bucket * kWaves + wave];
+                    before_r[k] = before_wave[bucket];
+                }
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k)
+                    packed[k] |= (e[k] >= 0 ? position(word_r[k], before_r[k]) : kNoPosition) << kExpertPositionShift;
+            } else {
+#pragma unroll
+                for (int k = 0; k < KMAX; ++k) packed[k] |= kNoPosition << kExpertPositionShift;
             }
             if (KMAX == 8 && p.K == 8) {
                 vec16* dst = reinterpret_cast<vec16*>(p.pos + int64_t(t) * 8);

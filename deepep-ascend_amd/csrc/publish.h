@@ -203,40 +203,65 @@ __device__ void write_expert_bases(const LayoutTables& t, int32_t* table, uint32
     }
 }
 
+// Does `word` carry the tag of the running single-launch dispatch (kernels.h)?
+__device__ __forceinline__ bool has_tag(uint32_t word, uint32_t tag) {
+    return (word & ~kTagValueMask) == tag;
+}
+
 // The expert base table in one trip, for the publishing workgroup of a single-launch expanded dispatch, whose movers
-// wait for exactly this: thread e keeps its column of chunk totals in registers between the sum and the stores.
-// Needs E <= kThreads and num_chunks <= 32.  Leaves totals / aligned / aligned_incl as publish_experts expects to
-// recompute them; stores at agent scope, each word ORed with `tag`.  A: expert alignment.
+// wait for exactly this.  Thread e reads its column of the tagged chunk totals at agent scope, again (at most
+// spin_limit times) until every word shows the tag - no flag of the counting workgroups is waited for, which would
+// only be raised once all their stores are acknowledged - keeps the column in registers between the sum and the
+// stores, and stores the bases at agent scope, each ORed with `tag`.  Needs E <= kThreads and num_chunks <= 32.
+// Leaves totals / aligned / aligned_incl as publish_experts expects to recompute them.  A: expert alignment.
+// Returns whether every thread got its column.
 template <int kThreads>
-__device__ void write_expert_bases_from_registers(const LayoutTables& t, int32_t* table, uint32_t tag, int R, int E, int A,
-                                                  int num_chunks, const PublishLds& s) {
+__device__ bool write_expert_bases_from_registers(const LayoutTables& t, const uint32_t* tagged_counts, int32_t* table, uint32_t tag,
+                                                  unsigned spin_limit, int R, int E, int A, int num_chunks, const PublishLds& s) {
     const int e = threadIdx.x;
     int v[32];
     int total = 0;
+    bool complete = true;
     if (e < E) {
-        const int32_t* col = t.expert_counts + e;
+        unsigned polls = 0;
+        for (;;) {
+            complete = true;
 #pragma unroll
-        for (int u = 0; u < 32; ++u) v[u] = col[int64_t(min(u, num_chunks - 1)) * t.experts_padded];
+            for (int u = 0; u < 32; ++u) {
+                // a row start common to the workgroup plus the thread's column: one address register serves all 32 loads
+                const int row_start = __builtin_amdgcn_readfirstlane(min(u, num_chunks - 1) * t.experts_padded);
+                v[u] = load_agent(reinterpret_cast<const int*>(tagged_counts) + row_start + e);
+            }
 #pragma unroll
-        for (int u = 0; u < 32; ++u) total += u < num_chunks ? v[u] : 0;
+            for (int u = 0; u < 32; ++u) complete = complete && has_tag(uint32_t(v[u]), tag);
+            if (complete || polls == spin_limit) break;
+            __builtin_amdgcn_s_sleep(4);
+            ++polls;
+        }
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            v[u] = int(uint32_t(v[u]) & kTagValueMask);
+            total += u < num_chunks ? v[u] : 0;
+        }
         s.totals[R + e] = total;
         const int al = (total + A - 1) / A * A;
         s.aligned[e] = al;
         s.aligned_incl[e] = al;
     }
-    __syncthreads();
+    const int all_complete = __syncthreads_and(complete ? 1 : 0);
     block_inclusive_scan<kThreads>(s.aligned_incl, E, s.scan_tmp);
     if (e < E) {
-        int32_t* out = table + e;
         int run = s.aligned_incl[e] - s.aligned[e];
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
             if (u < num_chunks) {
-                store_agent(out + int64_t(u) * t.experts_padded, int(uint32_t(run) | tag));
+                const int row_start = __builtin_amdgcn_readfirstlane(u * t.experts_padded);
+                store_agent(table + row_start + e, int(uint32_t(run) | tag));
                 run += v[u];
             }
         }
     }
+    return all_complete != 0;
 }
 
 // Everything at once, for a workgroup that publishes after all counting is over (the stand-alone layout kernel):

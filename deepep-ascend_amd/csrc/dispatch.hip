@@ -381,6 +381,19 @@ __device__ __forceinline__ FirstLook first_look(const MoveParams& p, int t, int 
     return f;
 }
 
+// The same words read again at agent scope, by a wavefront whose first look came back without the layout: issued before
+// the wavefront turns to converting its tile, so that the answer travels while it computes.
+__device__ __forceinline__ FirstLook second_look(const MoveParams& p, int t, int lane, bool has_work) {
+    FirstLook f{0, 0, 0};
+    const int begin = int(threadIdx.x) * 4;
+    if (begin < p.R * p.tab.chunks_padded) {
+        f.totals_lo = load_agent64(p.tagged_rank + begin);
+        f.totals_hi = load_agent64(p.tagged_rank + begin + 2);
+    }
+    if (has_work && lane < p.K) f.position = uint32_t(load_agent(reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane));
+    return f;
+}
+
 // Has this wavefront's first look found everything it asked for?  (Wave-uniform.)
 __device__ __forceinline__ bool look_is_complete(const MoveParams& p, const FirstLook& look, uint32_t tag, bool has_work, int lane) {
     bool ok = !(has_work && lane < p.K) || has_tag(look.position, tag);
@@ -699,6 +712,7 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
         // instructions each, eight wavefronts to a SIMD) would otherwise queue up between that moment and the first
         // stores of the launch.
         if (!look_is_complete(p, look, tag, has_work, lane)) {
+            look = second_look(p, t, lane, has_work);
             cast_tile();
             cast_done = true;
         }

@@ -31,20 +31,20 @@ HBM_PEAK_GBS = 8000.0
 # the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
-    ("C3", "compact", "fp8", "dispatch"): 452674499,
-    ("C3", "compact", "fp8", "combine"): 750130200,
-    ("C3", "expanded", "fp8", "dispatch"): 614184496,
-    ("C3", "expanded", "fp8", "combine"): 1074413120,
-    ("C3", "compact", "bf16", "dispatch"): 1097549 + 755649847,
-    ("C3", "compact", "bf16", "combine"): 750132725,
+    ("C3", "compact", "fp8", "dispatch"): 452269424,
+    ("C3", "compact", "fp8", "combine"): 750131170,
+    ("C3", "expanded", "fp8", "dispatch"): 613857063,
+    ("C3", "expanded", "fp8", "combine"): 1074420271,
+    ("C3", "compact", "bf16", "dispatch"): 1057781 + 755662315,
+    ("C3", "compact", "bf16", "combine"): 750132877,
     # profiles/bench_C4_C2_hbm_counters.md
-    ("C4", "compact", "fp8", "dispatch"): 420435041,
-    ("C4", "compact", "fp8", "combine"): 688673806,
-    ("C2", "compact", "bf16", "dispatch"): 97192571,
-    ("C2", "compact", "bf16", "combine"): 95447812,
+    ("C4", "compact", "fp8", "dispatch"): 420065108,
+    ("C4", "compact", "fp8", "combine"): 688673724,
+    ("C2", "compact", "bf16", "dispatch"): 97379235,
+    ("C2", "compact", "bf16", "combine"): 95447828,
     # profiles/bench_C5_low_latency_hbm_counters.md
-    ("C5", "packed", "fp8", "ll_dispatch"): 23981860,
-    ("C5", "packed", "fp8", "ll_combine"): 30328025,
+    ("C5", "packed", "fp8", "ll_dispatch"): 23981872,
+    ("C5", "packed", "fp8", "ll_combine"): 30328008,
 }
 
 

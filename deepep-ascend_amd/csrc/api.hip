@@ -52,8 +52,8 @@ struct LaunchPlan {
     bool fused;       // one launch: counting workgroups at the front of the move kernel
 };
 
-// Past this many mover workgroups the per-workgroup cost of the single-launch protocol (a look at a gate, one
-// atomic, a workgroup barrier) outweighs the launch it saves: 28 672 workgroups of 8192 BF16 rows of 14 KB take
+// Past this many mover workgroups the per-workgroup cost of the single-launch protocol (a look at the layout, one
+// atomic, two workgroup barriers) outweighs the launch it saves: 28 672 workgroups of 8192 BF16 rows of 14 KB take
 // 180 us in one launch against 140 us in two; 8 192 workgroups of the same rows cast to FP8 take 92 us against 97 us.
 constexpr int64_t kMaxFusedMovers = 16384;
 

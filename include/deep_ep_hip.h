@@ -71,7 +71,9 @@ const char* deep_ep_hip_last_error(void);
 typedef struct {
     int32_t dispatch_launches; /* dispatch with both phases in one call: 0 = a single launch (counting workgroups at
                                   the front of the move kernel) where the shape allows it (num_topk <= 8, num_ranks +
-                                  num_experts <= 512, num_ranks * ceil(num_tokens / 256) <= 1024) and it pays (at most
+                                  num_experts <= 512, num_ranks * ceil(num_tokens / 256) <= 1024, num_tokens * num_topk
+                                  <= 65536; with do_expand also ceil(num_tokens / 256) * num_experts <= 8192 and
+                                  num_tokens * num_topk + num_experts * expert_alignment < 2^18) and it pays (at most
                                   16384 mover workgroups); 1 = a single launch wherever the shape allows it; 2 = always
                                   layout kernel + move kernel */
     int32_t cast_pairs;        /* fused FP8 cast: 1024-channel segments per wavefront (1, 2, 4, 7, 8) */
@@ -91,9 +93,11 @@ typedef struct {
 size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_experts, int num_ranks);
 /* Byte offset, inside the workspace, of the int32 status word. */
 size_t deep_ep_hip_workspace_status_offset(void);
-/* Leading bytes of the workspace that hold the status word and the launch bookkeeping the kernels expect to find
- * zero at the start of a launch (and leave zero at its end).  After DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT, zero these
- * bytes before the workspace is used again. */
+/* Leading bytes of the workspace that hold the status word and the launch bookkeeping of the kernels: counters and
+ * flags they expect to find zero at the start of a launch (and leave zero at its end), and the tables through which the
+ * workgroups of a single-launch dispatch hand each other the layout, which must never hold anything but zeros or what
+ * those kernels wrote.  After DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT, zero these bytes before the workspace is used again
+ * (deep_ep_hip_read_status with clear != 0 does). */
 size_t deep_ep_hip_workspace_control_bytes(void);
 /* The first part of those bytes: counters and flags that read zero whenever no launch is running, but for the status
  * word (offset 0), the two row totals a dispatch leaves for the kernels that follow it (offsets 8 and 12) and the
@@ -348,7 +352,8 @@ typedef struct {
     deep_ep_hip_tuning tuning;
 } deep_ep_hip_ll_dispatch_args;
 
-/* Bytes of (zero-initialised, reusable) workspace a low-latency dispatch of this shape needs. */
+/* Bytes of (zero-initialised, reusable) workspace a low-latency dispatch of this shape needs.  A memory of its own: it
+ * must not overlap the workspace of deep_ep_hip_launch_dispatch (see deep_ep_hip_workspace_control_bytes). */
 size_t deep_ep_hip_ll_workspace_bytes(int num_src_ranks, int src_token_stride, int num_topk, int num_local_experts);
 int deep_ep_hip_launch_ll_dispatch(const deep_ep_hip_ll_dispatch_args* args, void* stream);
 

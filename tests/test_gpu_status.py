@@ -79,7 +79,7 @@ def test_status_read_through_the_c_abi(static):
 
 
 def test_clearing_read_repairs_the_workspace_after_a_timeout():
-    """A single-launch dispatch that gave up leaves its gates and flags mid-protocol.  The state is forced from the
+    """A single-launch dispatch that gave up leaves its counters, flags and tagged tables mid-protocol.  The state is forced from the
     host here (the flag set and the bookkeeping words scribbled over): the clearing read must report the flag and
     leave every bookkeeping word zero, and the next dispatch must be exact."""
     from deep_ep import _abi
@@ -90,7 +90,7 @@ def test_clearing_read_repairs_the_workspace_after_a_timeout():
     want = _dispatch(_abi.lib.deep_ep_hip_launch_dispatch, case, False, own)
     control = _abi.lib.deep_ep_hip_workspace_control_bytes()
     words = own[:control].view(torch.int32)
-    words[4:] = 3                                                         # gates and flags as a launch that gave up might leave them
+    words[4:] = -1                                                        # counters, flags, generation and tagged tables scribbled over
     words[0] = _abi.STATUS_LAYOUT_TIMEOUT
     host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
     stream = torch.cuda.current_stream().cuda_stream

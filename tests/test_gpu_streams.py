@@ -127,7 +127,7 @@ def test_host_argument_errors():
 
 def test_calls_on_two_streams_share_the_workspace_in_order():
     """An asynchronous dispatch on the communication stream that nobody has waited for yet, followed at once by plain
-    calls on the compute stream with other routing: the buffer's workspace (positions, tables, gates) is shared, so the
+    calls on the compute stream with other routing: the buffer's workspace (positions, tables, counters) is shared, so the
     second call has to queue behind the first by itself.  Both results are checked against the oracle."""
     a = rc.small("two_streams_a", 3000, 1024, 64, 8, 8, seed=61, masked_ratio=0.05)
     b = rc.small("two_streams_b", 2900, 1024, 64, 8, 8, seed=62, masked_ratio=0.3)

@@ -443,20 +443,28 @@ __device__ __forceinline__ unsigned advance_gate(const MoveParams& p, unsigned m
     return atomicInc(p.gates + gate * kDispatchGateStride, movers_of_gate(p, gate) - 1u);
 }
 
-// First thread of a mover workgroup, last thing it does.  The mover that was the last of its gate reports the gate;
-// the one that reports the last gate advances the generation: by then every mover has read its tagged words.
+// First wavefront of a mover workgroup (all its lanes), last thing it does; `seen` counts on its first lane.  The mover
+// that was the last of its gate reports the gate; the one that reports the last gate advances the generation: by then
+// every mover has read its tagged words.  The launch that used the last tag clears the tagged tables first, all lanes
+// together (a third of a megabyte: some 15 us once in 16383 launches).
 __device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover, unsigned seen, uint32_t tag) {
-    const unsigned gate = mover % unsigned(kDispatchGates);
-    if (seen != movers_of_gate(p, gate) - 1u) return;
-    const unsigned gates_in_use = p.num_movers < unsigned(kDispatchGates) ? p.num_movers : unsigned(kDispatchGates);
-    if (atomicInc(p.gates_finished, gates_in_use - 1u) != gates_in_use - 1u) return;
+    const int lane = lane_id();
+    int last = 0;
+    if (lane == 0) {
+        const unsigned gate = mover % unsigned(kDispatchGates);
+        if (seen == movers_of_gate(p, gate) - 1u) {
+            const unsigned gates_in_use = p.num_movers < unsigned(kDispatchGates) ? p.num_movers : unsigned(kDispatchGates);
+            last = atomicInc(p.gates_finished, gates_in_use - 1u) == gates_in_use - 1u ? 1 : 0;
+        }
+    }
+    if (__builtin_amdgcn_readfirstlane(last) == 0) return;
     uint32_t next = tag >> kTagShift;                     // generation + 1
     if (next == kTagPeriod) {
-        for (int i = 0; i < p.tagged_words; i += 4) store16_agent(p.tagged + i, vec16{0, 0, 0, 0});
+        for (int i = lane * 4; i < p.tagged_words; i += kWaveSize * 4) store16_agent(p.tagged + i, vec16{0, 0, 0, 0});
         wait_for_own_stores();
         next = 0;
     }
-    store_agent(reinterpret_cast<int*>(p.generation), int(next));
+    if (lane == 0) store_agent(reinterpret_cast<int*>(p.generation), int(next));
 }
 
 // A wavefront's wait (bounded) for the tagged words its threads want.  Returns whether this thread still misses one.
@@ -608,7 +616,7 @@ __device__ __forceinline__ void dispatch_copy(const MoveParams& p) {
         const FusedLayout f = await_layout(p, mover, look, tag, route_in, t, lane, has_work);
         gate_seen = f.gate_seen;
         if (!has_work || !f.complete) {
-            if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+            if (threadIdx.x < kWaveSize) settle_gate(p, mover, gate_seen, tag);
             return;
         }
         word = f.position;
@@ -639,7 +647,7 @@ __device__ __forceinline__ void dispatch_copy(const MoveParams& p) {
         }
     }
     if constexpr (kFused)
-        if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+        if (threadIdx.x < kWaveSize) settle_gate(p, mover, gate_seen, tag);
 }
 
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
@@ -719,7 +727,7 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
         const FusedLayout f = await_layout(p, mover, look, tag, route_in, t, lane, has_work);
         gate_seen = f.gate_seen;
         if (!has_work || !f.complete) {
-            if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+            if (threadIdx.x < kWaveSize) settle_gate(p, mover, gate_seen, tag);
             return;
         }
         word = f.position;
@@ -750,7 +758,7 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
             p.recv_sf[int64_t(row) * p.rsf_ts + int64_t(group) * p.rsf_hs] = __float_as_uint(my_scale);
     }
     if constexpr (kFused)
-        if (threadIdx.x == 0) settle_gate(p, mover, gate_seen, tag);
+        if (threadIdx.x < kWaveSize) settle_gate(p, mover, gate_seen, tag);
 }
 
 // The kernels.  The single-launch forms also hold the counting and publishing code, whose register needs must not cost

@@ -102,7 +102,8 @@ size_t deep_ep_hip_workspace_control_bytes(void);
 /* The first part of those bytes: counters and flags that read zero whenever no launch is running, but for the status
  * word (offset 0), the two row totals a dispatch leaves for the kernels that follow it (offsets 8 and 12) and the
  * launch generation (offset 128).  The rest of the control bytes are the tables through which the workgroups of a
- * single-launch dispatch hand each other the layout; only the kernels write there. */
+ * single-launch dispatch hand each other the layout; only the kernels write there.  (A size to look at, not to zero:
+ * the generation and those tables belong together, so zero all of the control bytes or none.) */
 size_t deep_ep_hip_workspace_counter_bytes(void);
 /* A status read that does not synchronise the device, for loops that run without host waits (graph replays, serving
  * loops).  Enqueues on `stream` one small kernel that copies the status word of `workspace` (NULL: the built-in

@@ -293,8 +293,11 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
 // DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT.
 constexpr unsigned kLayoutSpinLimit = 1u << 22;      // polls (each with a short sleep) before giving up: seconds
 
+// The tag of the running launch.  An ordinary (cached) load: the generation word does not change while anyone reads it -
+// it is advanced only after every mover has read its tagged words, which it cannot do without the tag - and with tens of
+// thousands of wavefronts asking, a read that went to memory every time would make the word's memory channel a hot spot.
 __device__ __forceinline__ uint32_t launch_tag(const uint32_t* generation) {
-    return (uint32_t(load_agent(reinterpret_cast<const int*>(generation))) + 1u) << kTagShift;
+    return (*generation + 1u) << kTagShift;
 }
 
 __device__ __forceinline__ uint64_t load_agent64(const void* p) {

@@ -38,7 +38,7 @@ __device__ __forceinline__ void count_chunk(const LayoutParams& p, const int chu
     const bool active = t < p.T;
     uint32_t tag = 0;
     if constexpr (kThrough)
-        if (p.generation != nullptr) tag = (uint32_t(load_agent(reinterpret_cast<const int*>(p.generation))) + 1u) << kTagShift;
+        if (p.generation != nullptr) tag = (*p.generation + 1u) << kTagShift;     // constant while the launch reads it
 
     // The index loads go out first (they are the longest wait of the pass), before anything that could alias
     // them is stored; the bitmap is cleared while they are in flight.

@@ -264,10 +264,78 @@ __device__ bool write_expert_bases_from_registers(const LayoutTables& t, const u
     return all_complete != 0;
 }
 
+// publish_layout for the common sizes (at most 32 chunks, num_experts <= kThreads, R * chunks_padded <= 4 * kThreads) in one
+// trip to memory instead of four: every thread first loads all it will ever need - four entries of the flattened rank
+// table and its expert's column of chunk totals, kept in registers - and totals, prefix sums, public outputs and both
+// base tables are worked out from those.
+template <int kThreads>
+__device__ void publish_layout_in_one_trip(const PublishParams& q, const LayoutTables& t, int num_chunks, bool expert_bases, int* lds) {
+    const PublishLds s = carve_publish_lds(lds, q.R, q.E);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int flat = q.R * t.chunks_padded;              // a multiple of 4: a thread's entries share a row
+    const int begin = tid * 4;
+    vec16 rv{0, 0, 0, 0};
+    if (begin < flat) rv = load16(t.rank_counts + begin);
+    int v[32];
+    if (tid < q.E) {
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            const int row_start = __builtin_amdgcn_readfirstlane(min(u, num_chunks - 1) * t.experts_padded);
+            v[u] = t.expert_counts[row_start + tid];
+        }
+    }
+
+    // rank part: exclusive prefix over the flattened table = first compact row of every (rank, chunk)
+    const int sum = int(rv.x) + int(rv.y) + int(rv.z) + int(rv.w);
+    const int inc = wave_inclusive_sum(sum);
+    if (lane == kWaveSize - 1) s.scan_tmp[wave] = inc;
+    __syncthreads();
+    int run = inc - sum;
+    for (int w = 0; w < wave; ++w) run += s.scan_tmp[w];
+    if (begin < flat) {
+        if (t.rank_bases != nullptr) {
+            const uint32_t b0 = uint32_t(run), b1 = b0 + rv.x, b2 = b1 + rv.y, b3 = b2 + rv.z;
+            store16(t.rank_bases + begin, vec16{b0, b1, b2, b3});
+        }
+        if ((begin + 4) % t.chunks_padded == 0) s.totals[begin / t.chunks_padded] = run + sum;   // inclusive prefix of the rank
+    }
+    if (tid < q.E) {
+        int total = 0;
+#pragma unroll
+        for (int u = 0; u < 32; ++u) total += u < num_chunks ? v[u] : 0;
+        s.totals[q.R + tid] = total;
+    }
+    __syncthreads();
+    for (int r = tid; r < q.R; r += kThreads) {
+        const int total = s.totals[r] - (r > 0 ? s.totals[r - 1] : 0);
+        if (q.num_tokens_per_rank != nullptr) q.num_tokens_per_rank[r] = total;
+        if (q.host_counts != nullptr) q.host_counts[r] = -total - 1;
+        if (q.psum_rank != nullptr) q.psum_rank[r] = s.totals[r];
+    }
+    if (tid == 0 && q.totals_out != nullptr) q.totals_out[0] = s.totals[q.R - 1];
+
+    publish_experts<kThreads>(q, s);
+    if (t.expert_bases != nullptr && expert_bases && tid < q.E) {
+        int at = s.aligned_incl[tid] - s.aligned[tid];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            if (u < num_chunks) {
+                const int row_start = __builtin_amdgcn_readfirstlane(u * t.experts_padded);
+                t.expert_bases[row_start + tid] = at;
+                at += v[u];
+            }
+        }
+    }
+}
+
 // Everything at once, for a workgroup that publishes after all counting is over (the stand-alone layout kernel):
 // totals, public outputs, and - when the caller has room for them - the base tables.
 template <int kThreads>
 __device__ void publish_layout(const PublishParams& q, const LayoutTables& t, int num_chunks, bool expert_bases, int* lds) {
+    if (num_chunks <= 32 && q.E <= kThreads && q.R * t.chunks_padded <= 4 * kThreads) {
+        publish_layout_in_one_trip<kThreads>(q, t, num_chunks, expert_bases, lds);
+        return;
+    }
     const PublishLds s = carve_publish_lds(lds, q.R, q.E);
     sum_rank_rows<kThreads>(t, q.R, s.totals);
     sum_expert_columns<kThreads>(t, q.R, q.E, num_chunks, s.totals);

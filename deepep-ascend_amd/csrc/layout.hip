@@ -32,10 +32,11 @@ __global__ __launch_bounds__(kThreads) void layout_kernel(const LayoutParams p) 
     extern __shared__ uint64_t bitmap[];   // [(R + E)][kWaves]
     __shared__ int is_last;
     const int tid = threadIdx.x;
-    count_chunk<KMAX, false>(p, int(blockIdx.x), int(gridDim.x), bitmap);
+    count_chunk<KMAX, true>(p, int(blockIdx.x), int(gridDim.x), bitmap);
 
-    // Hand the chunk totals to whichever workgroup finishes last: release our stores, take a ticket.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    // Hand the chunk totals to whichever workgroup finishes last: they were stored at agent scope (written through), so
+    // waiting for our own stores is all the release there is - no write-back of the whole L2 - then take a ticket.
+    wait_for_own_stores();
     __syncthreads();
     if (tid == 0) {
         const unsigned ticket = atomicAdd(p.done_counter, 1u);

@@ -31,20 +31,20 @@ HBM_PEAK_GBS = 8000.0
 # the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
-    ("C3", "compact", "fp8", "dispatch"): 452269424,
-    ("C3", "compact", "fp8", "combine"): 750131170,
-    ("C3", "expanded", "fp8", "dispatch"): 613857063,
-    ("C3", "expanded", "fp8", "combine"): 1074420271,
-    ("C3", "compact", "bf16", "dispatch"): 1057781 + 755662315,
-    ("C3", "compact", "bf16", "combine"): 750132877,
+    ("C3", "compact", "fp8", "dispatch"): 452247573,
+    ("C3", "compact", "fp8", "combine"): 750129318,
+    ("C3", "expanded", "fp8", "dispatch"): 613799036,
+    ("C3", "expanded", "fp8", "combine"): 1074420624,
+    ("C3", "compact", "bf16", "dispatch"): 1843283 + 755660688,
+    ("C3", "compact", "bf16", "combine"): 750132217,
     # profiles/bench_C4_C2_hbm_counters.md
-    ("C4", "compact", "fp8", "dispatch"): 420065108,
-    ("C4", "compact", "fp8", "combine"): 688673724,
-    ("C2", "compact", "bf16", "dispatch"): 97379235,
-    ("C2", "compact", "bf16", "combine"): 95447828,
+    ("C4", "compact", "fp8", "dispatch"): 420060643,
+    ("C4", "compact", "fp8", "combine"): 688673965,
+    ("C2", "compact", "bf16", "dispatch"): 97417243,
+    ("C2", "compact", "bf16", "combine"): 95447471,
     # profiles/bench_C5_low_latency_hbm_counters.md
-    ("C5", "packed", "fp8", "ll_dispatch"): 23981872,
-    ("C5", "packed", "fp8", "ll_combine"): 30328008,
+    ("C5", "packed", "fp8", "ll_dispatch"): 23981965,
+    ("C5", "packed", "fp8", "ll_combine"): 30328020,
 }
 
 

@@ -273,10 +273,11 @@ __device__ __forceinline__ uint64_t destination_lanes(const MoveParams& p, const
 // would add the writer's wait for its stores, the flag's own trip and a second read.  So the data is its own flag:
 //   - every word handed to the movers (chunk totals of the rank buckets, position words, expert bases) carries the
 //     tag of this launch in its upper bits (kernels.h) and is stored at agent scope (written through);
-//   - a mover workgroup reads what it needs at agent scope - each thread four chunk totals, each wavefront the
-//     position words of its token, and for the expanded layout the base of each lane's (chunk, expert) - and repeats
-//     a read (bounded) until the word shows the tag.  The first read of each goes out before the payload loads.  It
-//     then works the rank bases out for itself (an exclusive prefix sum over the R x C chunk totals, into LDS);
+//   - a mover workgroup reads what it needs - each thread four chunk totals, each wavefront the position words of
+//     its token, and for the expanded layout the base of each lane's (chunk, expert) - first with ordinary loads that
+//     go out before the payload loads (first_look), and, where a word does not show the tag yet, again at agent scope
+//     (bounded: second_look, await_tagged_words).  It then works the rank bases out for itself (an exclusive prefix
+//     sum over the R x C chunk totals, into LDS);
 //   - the publisher waits for the chunk_done flags the counting workgroups raise once their stores are acknowledged,
 //     clears them, and writes the per-rank and per-expert outputs of the call while the movers are already moving;
 //     for the expanded layout the tagged expert bases go out first.
@@ -349,9 +350,9 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
         if (!complete && threadIdx.x == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
     }
 
-    // Everything else reads the count tables with ordinary loads, once the counting workgroups have flagged that their
-    // stores are acknowledged.  (The tables have one writer per cache line and this workgroup has not touched them
-    // before, so ordinary loads fetch what was written through.)
+    // Everything else waits until the counting workgroups have flagged that their stores are acknowledged.  The expert
+    // table (a row per chunk: one writer per cache line, and this workgroup has not touched it before) is then read
+    // with ordinary loads, the rank table (lines shared by the writers of 16 chunks) at agent scope.
     await_and_clear_flags(p, p.chunk_done, p.count_blocks);
     sum_expert_columns<kThreads>(tab, p.R, p.E, p.count_blocks, lds.totals);
     publish_experts<kThreads>(p.pub, lds);

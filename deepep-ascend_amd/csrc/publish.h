@@ -107,18 +107,24 @@ __device__ void write_rank_bases(const LayoutTables& t, int R, const PublishLds&
     }
 }
 
-// The rank part as one flat pass over rank_counts ([rank][chunk], R * chunks_padded <= 4 * kThreads entries; in a
-// single-launch dispatch written through by counting workgroups of the same launch, each line by one writer, and not
-// touched by the caller's workgroup before those have finished, so ordinary loads fetch them): the inclusive prefix
-// sum over the flattened table is, at the last entry of row r, the end of rank r's bucket.  Publishes the per-rank
-// outputs.  Every thread of the workgroup must call it; s.scan_tmp: kThreads / 64 ints of LDS.
+// The rank part as one flat pass over rank_counts ([rank][chunk], R * chunks_padded <= 4 * kThreads entries), for the
+// publishing workgroup of a single-launch dispatch.  A line of that table holds the totals of up to 16 chunks, written
+// through by as many counting workgroups of the same launch, some of them on this XCD: it is read at agent scope, past
+// any partial copy of the line a cache may hold.  The inclusive prefix sum over the flattened table is, at the last
+// entry of row r, the end of rank r's bucket.  Publishes the per-rank outputs.  Every thread of the workgroup must
+// call it; s.scan_tmp: kThreads / 64 ints of LDS.
 template <int kThreads>
 __device__ void scan_rank_counts(const PublishParams& q, const LayoutTables& t, int R, const PublishLds& s) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int flat = R * t.chunks_padded;              // a multiple of 4: a thread's entries share a row
     const int begin = tid * 4;
     vec16 v{0, 0, 0, 0};
-    if (begin < flat) v = load16(t.rank_counts + begin);
+    if (begin < flat) {
+        const unsigned long long* at = reinterpret_cast<const unsigned long long*>(t.rank_counts + begin);
+        const unsigned long long lo = __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long hi = __hip_atomic_load(at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v = vec16{uint32_t(lo), uint32_t(lo >> 32), uint32_t(hi), uint32_t(hi >> 32)};
+    }
     const int sum = int(v.x) + int(v.y) + int(v.z) + int(v.w);
     const int inc = wave_inclusive_sum(sum);
     if (lane == kWaveSize - 1) s.scan_tmp[wave] = inc;

@@ -478,18 +478,18 @@ __device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover,
 // round - and only when that has arrived reads the rest again, whatever is still missing in one trip per round.
 __device__ __forceinline__ bool await_tagged_words(uint32_t tag, bool wants_position, const int* position_at, uint32_t& position,
                                                    bool wants_totals, const uint32_t* totals_at, uint64_t& lo, uint64_t& hi,
-                                                   bool wants_base, const int* base_at, uint32_t& base_word) {
+                                                   bool wants_base, const int* base_at, uint32_t& base_word, unsigned spin_limit) {
     unsigned polls = 0;
     const uint64_t base_lanes = __ballot(wants_base);
     if (base_lanes != 0) {
         const bool watches = wants_base && lane_id() == __builtin_ctzll(base_lanes);
-        while (__any(watches && !has_tag(base_word, tag)) && polls < kLayoutSpinLimit) {
+        while (__any(watches && !has_tag(base_word, tag)) && polls < spin_limit) {
             __builtin_amdgcn_s_sleep(4);
             if (watches) base_word = uint32_t(load_agent(base_at));
             ++polls;
         }
     } else {
-        while (__any(wants_position && !has_tag(position, tag)) && polls < kLayoutSpinLimit) {
+        while (__any(wants_position && !has_tag(position, tag)) && polls < spin_limit) {
             __builtin_amdgcn_s_sleep(4);
             if (wants_position && !has_tag(position, tag)) position = uint32_t(load_agent(position_at));
             ++polls;
@@ -501,7 +501,7 @@ __device__ __forceinline__ bool await_tagged_words(uint32_t tag, bool wants_posi
         const bool no_totals = wants_totals && !totals_tagged(lo, hi, tag);
         const bool no_base = wants_base && !has_tag(base_word, tag);
         missing = no_position || no_totals || no_base;
-        if (!__any(missing) || polls >= kLayoutSpinLimit) break;
+        if (!__any(missing) || polls >= spin_limit) break;
         if (polls != 0) __builtin_amdgcn_s_sleep(1);
         if (no_position) position = uint32_t(load_agent(position_at));
         if (no_totals) {
@@ -531,7 +531,8 @@ __device__ __forceinline__ void hold_for_layout(const MoveParams& p, uint32_t ta
     uint32_t no_base = 0;
     const int begin = int(threadIdx.x) * 4;
     await_tagged_words(tag, has_work && lane < p.K, reinterpret_cast<const int*>(p.pos) + int64_t(t) * p.K + lane, look.position,
-                       begin < p.R * p.tab.chunks_padded, p.tagged_rank + begin, look.totals_lo, look.totals_hi, false, nullptr, no_base);
+                       begin < p.R * p.tab.chunks_padded, p.tagged_rank + begin, look.totals_lo, look.totals_hi, false, nullptr, no_base,
+                       p.mover_spin_limit);
 }
 
 // Everything a mover wavefront needs from the layout of its own launch.
@@ -564,7 +565,7 @@ __device__ __forceinline__ FusedLayout await_layout(const MoveParams& p, unsigne
         if (wants_base) base_word = uint32_t(*base_at);       // an ordinary load first, as in first_look
     }
     const bool missing = await_tagged_words(tag, wants_position, position_at, f.position, wants_totals, p.tagged_rank + begin, lo, hi,
-                                            wants_base, base_at, base_word);
+                                            wants_base, base_at, base_word, p.mover_spin_limit);
     f.expert_base = int(base_word & kTagValueMask);
     const bool complete = build_rank_bases(p, lo, hi, !missing, f.flat_bases);      // ends with a workgroup barrier
     if (threadIdx.x == 0) {

@@ -62,6 +62,7 @@ inline deep_ep_hip_tuning& process_tuning() {
         t.ll_threads = env("DEEP_EP_HIP_LL_THREADS");
         t.ll_two_kernels = env("DEEP_EP_HIP_LL_TWO_KERNELS");
         t.ll_combine_vecs = env("DEEP_EP_HIP_LL_COMBINE_VECS");
+        t.mover_spin_limit = env("DEEP_EP_HIP_MOVER_SPIN_LIMIT");
         return t;
     }();
     return tuning;
@@ -79,6 +80,7 @@ inline int32_t* tuning_field(const std::string& name) {
     if (name == "ll_threads") return &t.ll_threads;
     if (name == "ll_two_kernels") return &t.ll_two_kernels;
     if (name == "ll_combine_vecs") return &t.ll_combine_vecs;
+    if (name == "mover_spin_limit") return &t.mover_spin_limit;
     throw EPException("unknown tuning field: " + name);
 }
 

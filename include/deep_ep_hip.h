@@ -85,7 +85,12 @@ typedef struct {
     int32_t ll_threads;        /* low-latency dispatch, single-kernel path: workgroup size (256, 512, 1024) */
     int32_t ll_two_kernels;    /* 1: low-latency dispatch always as count kernel + move kernel */
     int32_t ll_combine_vecs;   /* low-latency combine: KB of row per wavefront (1, 2, 4) */
-    int32_t reserved[6];
+    int32_t mover_spin_limit;  /* single-launch dispatch: how often a mover workgroup repeats a read of the layout its own
+                                  launch is still computing before it gives up, stores nothing and sets
+                                  DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT (0 = 2^22, seconds; 1 makes the first workgroups of a
+                                  launch give up at once: for tests of that path - every kernel still runs to its end and
+                                  the workspace stays consistent) */
+    int32_t reserved[5];
 } deep_ep_hip_tuning;
 
 /* Bytes of workspace needed for dispatches of up to num_max_tokens tokens.  The workspace must

@@ -132,3 +132,40 @@ def test_status_read_in_a_replayed_graph():
         assert int(host[0]) == status
         (x * 2).sum().item()                                              # eager work of the program between replays
     buf.check_device_status()
+
+
+def test_a_dispatch_that_gives_up_says_so_and_leaves_the_workspace_usable(monkeypatch):
+    """A real LAYOUT_TIMEOUT, forced from the host: with `mover_spin_limit = 1` the mover workgroups that start before
+    the layout of their own launch is there give up after one read.  Every kernel still runs to its end.  The call must
+    be flagged (its outputs are invalid), the counters and flags of the workspace must be back at zero, and after the
+    status has been taken the next dispatch on the same buffer must be exact again."""
+    import deep_ep
+    import routing_oracle as oracle
+    from deep_ep import _abi
+    from test_gpu_parity import assert_equal
+    case = rc.small("gives_up", 6000, 1024, 64, 8, 8, seed=35, masked_ratio=0.05)
+    buf = _buffer(case)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    ref = oracle.dispatch(case.x, case.topk_idx, case.topk_weights, case.E, case.R, 0, case.M)
+    monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", 1)
+    buf.dispatch(x, idx, w, num_experts=case.E, do_cpu_sync=False)          # allocates the workspace
+    buf.check_device_status()
+
+    monkeypatch.setattr(deep_ep.tuning, "mover_spin_limit", 1)
+    buf.dispatch(x, idx, w, num_experts=case.E, do_cpu_sync=False)
+    torch.cuda.synchronize()
+    words = buf.runtime.workspace_control_words().clone()
+    assert int(words[0]) & _abi.STATUS_LAYOUT_TIMEOUT, "no workgroup of the launch was early enough to give up"
+    words[0] = 0
+    words[2:4] = 0
+    words[32] = 0
+    assert int(words.abs().sum()) == 0, "counters or flags left mid-protocol"
+    with pytest.raises(RuntimeError):
+        buf.check_device_status()
+
+    monkeypatch.setattr(deep_ep.tuning, "mover_spin_limit", 0)
+    recv, ridx, rw, handle, _ = buf.dispatch(x, idx, w, num_experts=case.E, do_cpu_sync=False)
+    assert_equal(recv[:ref.num_recv_tokens], ref.recv_x, "recv_x")
+    assert_equal(ridx[:ref.num_recv_tokens], ref.recv_topk_idx, "recv_topk_idx")
+    assert_equal(handle.dst_buffer_slot_idx, ref.dst_buffer_slot_idx, "dst_buffer_slot_idx")
+    buf.check_device_status()

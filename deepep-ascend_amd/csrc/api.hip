@@ -72,7 +72,7 @@ LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_mov
     }
     if (q.fused && tuning.dispatch_launches != 1) {
         MoveParams probe{};
-        probe.T = T; probe.H = H; probe.row_bytes = row_bytes; probe.payload = payload;
+        probe.T = T; probe.H = H; probe.row_bytes = row_bytes; probe.payload = payload; probe.do_expand = do_expand ? 1 : 0;
         probe.cast_pairs = tuning.cast_pairs; probe.copy_vecs = tuning.copy_vecs;
         q.fused = dispatch_move_workgroups(probe) <= kMaxFusedMovers;
     }

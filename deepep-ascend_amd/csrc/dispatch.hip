@@ -919,8 +919,12 @@ static int move_tile(const MoveParams& p) {
     if (p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8) {
         // Two segments (2048 channels, 8 wavefronts per SIMD) measured best at hidden 7168: 92.8 us per dispatch
         // against 93.7 (4 segments) and 96.9 (7 segments, one wavefront per token).
+        // The expanded layout stores eight rows per token instead of five: in a large call (64 MB of input and more)
+        // one segment per wavefront is ahead there (8192 x 7168: move phase 119 us against 122 us, whole call 130
+        // against 131 us).
         if (p.cast_pairs != 0) return p.cast_pairs;
-        return p.H <= 1024 ? 1 : 2;
+        const bool large = int64_t(p.T) * p.row_bytes >= (int64_t(64) << 20);
+        return (p.H <= 1024 || (p.do_expand && large)) ? 1 : 2;
     }
     // Large, bandwidth-bound calls: one 1 KB segment per wavefront measured best for this write-heavy stream (8192
     // BF16 rows of 14 KB: 143 us per dispatch against 155-159 us with 2, 4, 7 or 8 segments).  Small, latency-bound

@@ -33,8 +33,8 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
     ("C3", "compact", "fp8", "dispatch"): 452247573,
     ("C3", "compact", "fp8", "combine"): 750129318,
-    ("C3", "expanded", "fp8", "dispatch"): 613799036,
-    ("C3", "expanded", "fp8", "combine"): 1074420624,
+    ("C3", "expanded", "fp8", "dispatch"): 615720237,
+    ("C3", "expanded", "fp8", "combine"): 1074414320,
     ("C3", "compact", "bf16", "dispatch"): 1843283 + 755660688,
     ("C3", "compact", "bf16", "combine"): 750132217,
     # profiles/bench_C4_C2_hbm_counters.md

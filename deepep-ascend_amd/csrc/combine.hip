@@ -74,8 +74,13 @@ __device__ __forceinline__ void accumulate_rows(float (&acc)[kVecs][8], uint64_t
     }
 }
 
-template <int kVecs>
+// kLayout: what the rows of x are.  Each gets a kernel of its own, so that the sequencing registers of the expanded
+// layout do not cost the compact layout occupancy.
+enum : int { kCompactRows = 0, kExpandedRows = 1, kExpandedRowsReducedPerRank = 2 };
+
+template <int kVecs, int kLayout>
 __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p) {
+    constexpr bool kExpanded = kLayout != kCompactRows;
     const int lane = threadIdx.x & 63;
     const unsigned work = wave_work_index(blockIdx.x, kWavesPerBlock);
     if (work >= unsigned(p.T) * unsigned(p.tiles)) return;
@@ -132,7 +137,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
             d = small_div(e, 1.0f / float(p.E_l));
             if (v >= 0) {
                 row_c = (d > 0 ? p.psum_rank[d - 1] : 0) + (v - p.rank_idx * p.M);
-                if (!p.do_expand && row_c >= p.num_x_rows) {
+                if (!kExpanded && row_c >= p.num_x_rows) {
                     atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
                     row_c = -1;
                 }
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
         const int rj = read_lane(row_c, j);
         if (d >= 0 && dj == d && rj >= 0) my_row = rj;
     }
-    if (p.do_expand && my_row >= 0 && my_row < p.num_meta_rows) {
+    if (kExpanded && my_row >= 0 && my_row < p.num_meta_rows) {
         erow = p.meta[int64_t(my_row) * (p.K + 2) + 2 + lane];
         if (erow >= p.num_x_rows) {
             atomicOr(p.status, DEEP_EP_HIP_STATUS_ROW_OVERFLOW);
@@ -156,7 +161,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
     if (tile == 0 && p.out_w != nullptr && lane < p.K && !p.rank_mode) {
         float w = 0.f;
         if (p.topk_weights != nullptr) {
-            if (p.do_expand) {
+            if (kExpanded) {
                 if (erow >= 0) w = p.topk_weights[erow];
             } else if (my_row >= 0) {
                 w = p.topk_weights[int64_t(my_row) * p.K + lane];
@@ -165,31 +170,67 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
         p.out_w[int64_t(t) * p.K + lane] = w;
     }
 
-    if (!p.do_expand) {
+    if constexpr (kLayout == kCompactRows) {
         accumulate_rows<kVecs>(acc, __ballot(row_c >= 0), row_c, p.x, row_bytes, tile, lane);
-    } else if (!p.multi_red) {
+    } else if constexpr (kLayout == kExpandedRows) {
         accumulate_rows<kVecs>(acc, __ballot(erow >= 0), erow, p.x, row_bytes, tile, lane);
     } else {
+        // One term per destination rank, in ascending order of the rank's master lane; a rank's rows are summed in
+        // lane order and the sum is rounded to BF16 before it is added.  The rows are put into that order first (each
+        // lane learns the place of its row in the sequence), so that their loads go out kBatch at a time across the
+        // ranks: a load round per rank would cost a memory round trip for one or two rows each.
+        int place = -1, ends_term = 0, alone = 0, total = 0;
         uint64_t masters = __ballot(row_c >= 0);
         while (masters) {
             const int j = __builtin_ctzll(masters);
             masters &= masters - 1;
             const int dj = read_lane(d, j);
             const uint64_t members = __ballot(d == dj && erow >= 0);
-            if (__popcll(members) == 1) {
-                accumulate_rows<kVecs>(acc, members, erow, p.x, row_bytes, tile, lane);   // bf16 round trip is exact
-            } else {
-                float part[kVecs][8];
+            if (d == dj && erow >= 0) {
+                place = total + __popcll(members & ((uint64_t(1) << lane) - 1));
+                ends_term = (members >> lane) == 1 ? 1 : 0;
+                alone = __popcll(members) == 1 ? 1 : 0;         // its BF16 round trip is exact: added as it is
+            }
+            total += __popcll(members);
+        }
+        const int flags_of_lane = ends_term | (alone << 1);
+        float part[kVecs][8];
 #pragma unroll
-                for (int i = 0; i < kVecs; ++i)
+        for (int i = 0; i < kVecs; ++i)
 #pragma unroll
-                    for (int c = 0; c < 8; ++c) part[i][c] = 0.f;
-                accumulate_rows<kVecs>(part, members, erow, p.x, row_bytes, tile, lane);
+            for (int c = 0; c < 8; ++c) part[i][c] = 0.f;
+        for (int first = 0; first < total; first += kBatch) {
+            int rows[kBatch], flags[kBatch];
 #pragma unroll
-                for (int i = 0; i < kVecs; ++i)
+            for (int b = 0; b < kBatch; ++b) {
+                rows[b] = -1;
+                flags[b] = 0;
+                if (first + b < total) {
+                    const int j = __builtin_ctzll(__ballot(place == first + b));
+                    rows[b] = read_lane(erow, j);
+                    flags[b] = read_lane(flags_of_lane, j);
+                }
+            }
+            vec16 v[kBatch][kVecs];
 #pragma unroll
-                    for (int c = 0; c < 8; ++c)
-                        acc[i][c] += __uint_as_float(f32_to_bf16_bits(part[i][c]) << 16);
+            for (int b = 0; b < kBatch; ++b) load_row<kVecs>(v[b], p.x, rows[b], row_bytes, tile, lane);
+#pragma unroll
+            for (int b = 0; b < kBatch; ++b) {
+                if (rows[b] < 0) continue;
+                if (flags[b] & 2) {
+                    add_row<kVecs>(acc, v[b]);
+                    continue;
+                }
+                add_row<kVecs>(part, v[b]);
+                if (flags[b] & 1) {
+#pragma unroll
+                    for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) {
+                            acc[i][c] += __uint_as_float(f32_to_bf16_bits(part[i][c]) << 16);
+                            part[i][c] = 0.f;
+                        }
+                }
             }
         }
     }
@@ -209,22 +250,32 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const CombineParams p
     }
 }
 
+template <int kVecs, int kLayout>
+hipError_t launch_layout(const CombineParams& p, unsigned blocks, hipStream_t stream) {
+    hipLaunchKernelGGL((combine_kernel<kVecs, kLayout>), dim3(blocks), dim3(kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
 template <int kVecs>
 hipError_t launch(CombineParams p, hipStream_t stream) {
     const int row_bytes = p.H * 2;
     p.tiles = (row_bytes + kVecs * 1024 - 1) / (kVecs * 1024);
     const int64_t waves = int64_t(p.T) * p.tiles;
     const unsigned blocks = unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(combine_kernel<kVecs>, dim3(blocks), dim3(kThreads), 0, stream, p);
-    return hipGetLastError();
+    if (!p.do_expand || p.rank_mode) return launch_layout<kVecs, kCompactRows>(p, blocks, stream);
+    if (!p.multi_red) return launch_layout<kVecs, kExpandedRows>(p, blocks, stream);
+    return launch_layout<kVecs, kExpandedRowsReducedPerRank>(p, blocks, stream);
 }
 
 }  // namespace
 
 hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;
+    // Column tile per wavefront, in KB of a BF16 row.  Compact rows: 1 KB (512 channels, 41 registers, eight wavefronts
+    // per SIMD) measured best - 8192 tokens x 7168: 117.9 us against 122.7 (2 KB) and 119.6 (4 KB); after a cache flush
+    // 123.6 / 126.6 / 124.4; 4096 x 2048: 18.2 / 18.2 / 19.7.  Expanded rows are insensitive (181.7 / 181.7 / 180.5 us).
     int vecs = p.vecs;
-    if (vecs == 0) vecs = (p.H * 2 <= 1024) ? 1 : 2;
+    if (vecs == 0) vecs = (p.do_expand && !p.rank_mode && p.H * 2 > 1024) ? 2 : 1;
     switch (vecs) {
         case 1: return launch<1>(p, stream);
         case 4: return launch<4>(p, stream);

@@ -70,6 +70,9 @@ LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_mov
         q.fused = q.chunks * experts_padded <= kTaggedExpertWords &&
                   int64_t(T) * K + int64_t(E) * alignment <= int64_t(kTagValueMask);
     }
+    // The single-launch cast kernels exist for tiles of one and two segments (wider ones would spill registers under
+    // the occupancy the counting code is held to): a forced wider tile takes two launches.
+    if (payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8 && tuning.cast_pairs > 2) q.fused = false;
     if (q.fused && tuning.dispatch_launches != 1) {
         MoveParams probe{};
         probe.T = T; probe.H = H; probe.row_bytes = row_bytes; probe.payload = payload; probe.do_expand = do_expand ? 1 : 0;

@@ -906,8 +906,14 @@ template <int kPairs>
 hipError_t launch_cast(MoveParams p, hipStream_t stream) {
     p.tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
     const unsigned blocks = move_grid(p, int64_t(p.T) * p.tiles);
-    if (p.fused) hipLaunchKernelGGL((dispatch_cast_single_launch_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
-    else hipLaunchKernelGGL((dispatch_cast_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+    if constexpr (kPairs <= 2) {
+        if (p.fused) {
+            hipLaunchKernelGGL((dispatch_cast_single_launch_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
+            return hipGetLastError();
+        }
+    }
+    if (p.fused) return hipErrorInvalidConfiguration;      // the launch plan keeps wider tiles out of the single launch
+    hipLaunchKernelGGL((dispatch_cast_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }
 

@@ -76,7 +76,7 @@ typedef struct {
                                   num_tokens * num_topk + num_experts * expert_alignment < 2^18) and it pays (at most
                                   16384 mover workgroups); 1 = a single launch wherever the shape allows it; 2 = always
                                   layout kernel + move kernel */
-    int32_t cast_pairs;        /* fused FP8 cast: 1024-channel segments per wavefront (1, 2, 4, 7, 8) */
+    int32_t cast_pairs;        /* fused FP8 cast: 1024-channel segments per wavefront (1, 2, 4, 7, 8; above 2: two launches) */
     int32_t copy_vecs;         /* pass-through payloads: KB of row per wavefront (1, 2, 4, 7, 8) */
     int32_t plain_loads;       /* 1: payload loads allocate in the caches (for inputs known to be cache resident) */
     int32_t xcd_remap;         /* 1: consecutive workgroups of a dispatch share an XCD */

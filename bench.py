@@ -236,14 +236,17 @@ def main():
     dispatch_us = timed(lambda: dispatch(_abi.PHASE_LAYOUT | _abi.PHASE_MOVE), k, args.l2_flush)
     combine_us = timed(combine, k, args.l2_flush)
 
-    def distribution(fn, iters, flush):
+    def distribution(fn, iters, flush, before=None):
         """min / p50 / p95 / mean in us over single launches, each bracketed by its own pair of HIP events (the
-        events add a few us to every sample).  flush: a 256 MB buffer is zeroed before each launch."""
+        events add a few us to every sample).  flush: a 256 MB buffer is zeroed before each launch.  before: run
+        (untimed) ahead of every launch."""
         buf = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev) if flush else None
         samples = []
         for _ in range(iters):
             if flush:
                 buf.zero_()
+            if before is not None:
+                before()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream); fn(); e1.record(stream)
             e1.synchronize()
@@ -257,6 +260,10 @@ def main():
     dist = {"dispatch": distribution(full_dispatch, k, False), "combine": distribution(combine, k, False),
             "dispatch_after_cache_flush": distribution(full_dispatch, k, True),
             "combine_after_cache_flush": distribution(combine, k, True)}
+    # The input as a producing layer leaves it: just written by another kernel, hence in the memory-side cache.
+    x_source = x.clone()
+    dist["dispatch_after_input_written"] = distribution(full_dispatch, k, False, before=lambda: x.copy_(x_source))
+    del x_source
 
     def gbs(nbytes, us):
         return nbytes / us * 1e-3

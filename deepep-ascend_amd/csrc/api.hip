@@ -147,7 +147,13 @@ WorkspaceLayout make_workspace_layout(int num_max_tokens, int num_topk, int num_
     w.rank_bases = off;    off = align_up(off + chunks_padded * num_ranks * 4, 256);
     w.expert_counts = off; off = align_up(off + chunks * experts_padded * 4, 256);
     w.expert_bases = off;  off = align_up(off + chunks * experts_padded * 4, 256);
-    w.pos = off;           off = align_up(off + lanes * 4, 256);
+    // Position words of a dispatch in two launches (tag 0).  Shapes the tagged table holds use that table: its words are
+    // rewritten by whichever layout pass runs next, and a single-launch dispatch takes no word without its own tag.
+    if (lanes <= size_t(kTaggedPosWords)) {
+        w.pos = w.tagged_pos;
+    } else {
+        w.pos = off;       off = align_up(off + lanes * 4, 256);
+    }
     w.total_bytes = off;
     return w;
 }

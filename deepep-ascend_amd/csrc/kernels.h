@@ -25,7 +25,7 @@ constexpr uint32_t kTagValueMask = (1u << kTagShift) - 1u;
 constexpr uint32_t kTagPeriod = (1u << (32 - kTagShift)) - 1u;      // 16383
 constexpr int kTaggedRankWords = 1024;       // R x chunks (padded to a multiple of 4)
 constexpr int kTaggedExpertWords = 8192;     // chunks x experts (padded to a multiple of 32)
-constexpr int kTaggedPosWords = 65536;       // tokens x lanes
+constexpr int kTaggedPosWords = 131072;      // tokens x lanes
 
 // A position word: bits 0-8 the slot of the token inside its chunk for the lane's destination rank (master lanes
 // only), bits 9-17 the position of the lane inside its chunk for its expert, kNoPosition = none; a single-launch

@@ -72,7 +72,7 @@ typedef struct {
     int32_t dispatch_launches; /* dispatch with both phases in one call: 0 = a single launch (counting workgroups at
                                   the front of the move kernel) where the shape allows it (num_topk <= 8, num_ranks +
                                   num_experts <= 512, num_ranks * ceil(num_tokens / 256) <= 1024, num_tokens * num_topk
-                                  <= 65536; with do_expand also ceil(num_tokens / 256) * num_experts <= 8192 and
+                                  <= 131072; with do_expand also ceil(num_tokens / 256) * num_experts <= 8192 and
                                   num_tokens * num_topk + num_experts * expert_alignment < 2^18) and it pays (at most
                                   16384 mover workgroups); 1 = a single launch wherever the shape allows it; 2 = always
                                   layout kernel + move kernel */

@@ -33,8 +33,8 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
     ("C3", "compact", "fp8", "dispatch"): 452144809,
     ("C3", "compact", "fp8", "combine"): 751990947,
-    ("C3", "expanded", "fp8", "dispatch"): 615736930,
-    ("C3", "expanded", "fp8", "combine"): 1074426494,
+    ("C3", "expanded", "fp8", "dispatch"): 1863755 + 613017589,
+    ("C3", "expanded", "fp8", "combine"): 1074421479,
     ("C3", "compact", "bf16", "dispatch"): 1843283 + 755646776,
     ("C3", "compact", "bf16", "combine"): 751993607,
     # profiles/bench_C4_C2_hbm_counters.md

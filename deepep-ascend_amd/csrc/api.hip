@@ -73,6 +73,11 @@ LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_mov
     // The single-launch cast kernels exist for tiles of one and two segments (wider ones would spill registers under
     // the occupancy the counting code is held to): a forced wider tile takes two launches.
     if (payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8 && tuning.cast_pairs > 2) q.fused = false;
+    // The expanded layout of a large call (64 MB of input and more) is faster in two launches: every mover of a single
+    // launch waits for the publisher's expert bases, a second hand-off, while a move kernel of its own streams from its
+    // first microsecond (8192 x 7168: 123-128 us against 130-134 us; from 4096 tokens down the single launch is ahead,
+    // 66.5 against 72.8 us).
+    if (q.fused && do_expand && tuning.dispatch_launches != 1 && int64_t(T) * row_bytes >= (int64_t(64) << 20)) q.fused = false;
     if (q.fused && tuning.dispatch_launches != 1) {
         MoveParams probe{};
         probe.T = T; probe.H = H; probe.row_bytes = row_bytes; probe.payload = payload; probe.do_expand = do_expand ? 1 : 0;

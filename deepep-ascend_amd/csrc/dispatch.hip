@@ -882,8 +882,48 @@ __global__ __launch_bounds__(kThreads) void fill_tail_kernel(const FillTailParam
         p.recv_topk_idx[i] = -1;
 }
 
+// An attribute of the current device, asked once per device; `fallback` when the runtime does not answer.
+static int device_attribute(hipDeviceAttribute_t attribute, std::atomic<int>* cached, int fallback) {
+    constexpr int kMaxDevices = 64;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fallback;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, attribute, dev) != hipSuccess || n <= 0) n = fallback;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+static int compute_units() {
+    static std::atomic<int> cached[64];
+    return device_attribute(hipDeviceAttributeMultiprocessorCount, cached, 256);
+}
+
+static int lds_bytes_per_cu() {
+    static std::atomic<int> cached[64];
+    return device_attribute(hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, cached, 160 * 1024);
+}
+
+// How many workgroups of a move kernel launched on a finished layout a CU should hold at a time (0: as many as fit).
+// The fused cast streams fastest with fewer than the eight its registers allow - measured side by side at 8192 x 7168,
+// move phase in us with 8 / 7 / 6 / 5 / 4 per CU: compact layout 82.6 / 81.6 / 81.7 / 82.0 / 83.6 (16384 tokens: 162.5 with
+// eight, 156.5 with six), expanded layout 114.9 / 115.1 / 114.7 / 113.4 / 116.0 - while the BF16 copy does not care down
+// to six and loses 3 us at five.  Launches that would not fill two rounds of eight per CU are left alone.
+static int move_workgroups_per_cu(const MoveParams& p) {
+    if (p.fused || p.payload != DEEP_EP_HIP_PAYLOAD_CAST_FP8) return 0;
+    if (int64_t(p.num_movers) < int64_t(compute_units()) * 16) return 0;
+    return p.do_expand ? 5 : 6;
+}
+
 size_t move_lds_bytes(const MoveParams& p) {
-    if (!p.fused) return 0;
+    if (!p.fused) {
+        // The limit is set with LDS the kernel never touches: a share that is just too large for one workgroup more,
+        // whatever granule the LDS is handed out in.
+        const int per_cu = move_workgroups_per_cu(p);
+        if (per_cu == 0) return 0;
+        return (size_t(lds_bytes_per_cu() / (per_cu + 1)) + 256) & ~size_t(255);
+    }
     const size_t publish = publish_lds_bytes(p.R, p.E, kThreads);
     const size_t bitmap = count_lds_bytes(p.R, p.E);
     const size_t bases = (size_t(p.R) * p.tab.chunks_padded + kWavesPerBlock) * sizeof(int);
@@ -950,20 +990,6 @@ int64_t dispatch_move_workgroups(const MoveParams& p) {
     const int64_t tiles = p.payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8 ? (p.H + tile * 1024 - 1) / (tile * 1024)
                                                                     : (p.row_bytes + tile * 1024 - 1) / (tile * 1024);
     return (int64_t(p.T) * tiles + kWavesPerBlock - 1) / kWavesPerBlock;
-}
-
-// Compute units of the current device (asked once per device).
-static int compute_units() {
-    constexpr int kMaxDevices = 64;
-    static std::atomic<int> cached[kMaxDevices];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-    int n = cached[dev].load(std::memory_order_relaxed);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev].store(n, std::memory_order_relaxed);
-    }
-    return n;
 }
 
 hipError_t launch_dispatch_move(MoveParams p, hipStream_t stream) {

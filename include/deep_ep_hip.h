@@ -74,8 +74,8 @@ typedef struct {
                                   num_experts <= 512, num_ranks * ceil(num_tokens / 256) <= 1024, num_tokens * num_topk
                                   <= 131072; with do_expand also ceil(num_tokens / 256) * num_experts <= 8192 and
                                   num_tokens * num_topk + num_experts * expert_alignment < 2^18) and it pays (at most
-                                  16384 mover workgroups); 1 = a single launch wherever the shape allows it; 2 = always
-                                  layout kernel + move kernel */
+                                  16384 mover workgroups; with do_expand less than 64 MB of input); 1 = a single launch
+                                  wherever the shape allows it; 2 = always layout kernel + move kernel */
     int32_t cast_pairs;        /* fused FP8 cast: 1024-channel segments per wavefront (1, 2, 4, 7, 8; above 2: two launches) */
     int32_t copy_vecs;         /* pass-through payloads: KB of row per wavefront (1, 2, 4, 7, 8) */
     int32_t plain_loads;       /* 1: payload loads allocate in the caches (for inputs known to be cache resident) */

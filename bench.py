@@ -31,20 +31,20 @@ HBM_PEAK_GBS = 8000.0
 # the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
-    ("C3", "compact", "fp8", "dispatch"): 452144809,
-    ("C3", "compact", "fp8", "combine"): 751990947,
-    ("C3", "expanded", "fp8", "dispatch"): 1863755 + 613017589,
-    ("C3", "expanded", "fp8", "combine"): 1074421479,
-    ("C3", "compact", "bf16", "dispatch"): 1843283 + 755646776,
-    ("C3", "compact", "bf16", "combine"): 751993607,
+    ("C3", "compact", "fp8", "dispatch"): 452335662,
+    ("C3", "compact", "fp8", "combine"): 751992269,
+    ("C3", "expanded", "fp8", "dispatch"): 1863758 + 612972432,
+    ("C3", "expanded", "fp8", "combine"): 1074426643,
+    ("C3", "compact", "bf16", "dispatch"): 1843294 + 755741042,
+    ("C3", "compact", "bf16", "combine"): 751993795,
     # profiles/bench_C4_C2_hbm_counters.md
-    ("C4", "compact", "fp8", "dispatch"): 419952304,
-    ("C4", "compact", "fp8", "combine"): 690499911,
-    ("C2", "compact", "bf16", "dispatch"): 97412245,
-    ("C2", "compact", "bf16", "combine"): 96361869,
+    ("C4", "compact", "fp8", "dispatch"): 420107733,
+    ("C4", "compact", "fp8", "combine"): 690500080,
+    ("C2", "compact", "bf16", "dispatch"): 97436912,
+    ("C2", "compact", "bf16", "combine"): 96362178,
     # profiles/bench_C5_low_latency_hbm_counters.md
-    ("C5", "packed", "fp8", "ll_dispatch"): 23981878,
-    ("C5", "packed", "fp8", "ll_combine"): 30328005,
+    ("C5", "packed", "fp8", "ll_dispatch"): 23981894,
+    ("C5", "packed", "fp8", "ll_combine"): 30328025,
 }
 
 

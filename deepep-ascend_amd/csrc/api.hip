@@ -345,6 +345,7 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
         m.status = status;
         m.cast_pairs = a->tuning.cast_pairs; m.copy_vecs = a->tuning.copy_vecs;
         m.mover_spin_limit = a->tuning.mover_spin_limit > 0 ? unsigned(a->tuning.mover_spin_limit) : (1u << 22);   // seconds
+        m.move_workgroups_per_cu = a->tuning.move_workgroups_per_cu;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 
@@ -632,6 +633,7 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.status = status;
         m.cast_pairs = a->tuning.cast_pairs; m.copy_vecs = a->tuning.copy_vecs;
         m.mover_spin_limit = a->tuning.mover_spin_limit > 0 ? unsigned(a->tuning.mover_spin_limit) : (1u << 22);   // seconds
+        m.move_workgroups_per_cu = a->tuning.move_workgroups_per_cu;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 

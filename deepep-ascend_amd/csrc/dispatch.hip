@@ -911,7 +911,10 @@ static int lds_bytes_per_cu() {
 // eight, 156.5 with six), expanded layout 114.9 / 115.1 / 114.7 / 113.4 / 116.0 - while the BF16 copy does not care down
 // to six and loses 3 us at five.  Launches that would not fill two rounds of eight per CU are left alone.
 static int move_workgroups_per_cu(const MoveParams& p) {
-    if (p.fused || p.payload != DEEP_EP_HIP_PAYLOAD_CAST_FP8) return 0;
+    if (p.fused) return 0;
+    if (p.move_workgroups_per_cu != 0)       // two is the least an LDS share within a workgroup's 64 KB can enforce
+        return p.move_workgroups_per_cu >= 8 ? 0 : (p.move_workgroups_per_cu < 2 ? 2 : p.move_workgroups_per_cu);
+    if (p.payload != DEEP_EP_HIP_PAYLOAD_CAST_FP8) return 0;
     if (int64_t(p.num_movers) < int64_t(compute_units()) * 16) return 0;
     return p.do_expand ? 5 : 6;
 }

@@ -63,6 +63,7 @@ inline deep_ep_hip_tuning& process_tuning() {
         t.ll_two_kernels = env("DEEP_EP_HIP_LL_TWO_KERNELS");
         t.ll_combine_vecs = env("DEEP_EP_HIP_LL_COMBINE_VECS");
         t.mover_spin_limit = env("DEEP_EP_HIP_MOVER_SPIN_LIMIT");
+        t.move_workgroups_per_cu = env("DEEP_EP_HIP_MOVE_WORKGROUPS_PER_CU");
         return t;
     }();
     return tuning;
@@ -81,6 +82,7 @@ inline int32_t* tuning_field(const std::string& name) {
     if (name == "ll_two_kernels") return &t.ll_two_kernels;
     if (name == "ll_combine_vecs") return &t.ll_combine_vecs;
     if (name == "mover_spin_limit") return &t.mover_spin_limit;
+    if (name == "move_workgroups_per_cu") return &t.move_workgroups_per_cu;
     throw EPException("unknown tuning field: " + name);
 }
 

@@ -158,6 +158,7 @@ struct MoveParams {
     uint32_t* gates;         // [kDispatchGates] wrapping counters of the movers that are done reading, kDispatchGateStride words apart
     uint32_t* gates_finished;    // wrapping counter of the gates all of whose movers are done
     unsigned mover_spin_limit;   // reads a mover repeats for a word of the layout before it gives up (set from the tuning block)
+    int move_workgroups_per_cu;  // forced residency of a move kernel on a finished layout, 0 = choose (tuning block)
     uint32_t* generation;        // see WorkspaceLayout
     uint32_t* tagged;            // the tagged tables, tagged_words long: cleared by the launch that uses the last tag
     int tagged_words;

@@ -90,7 +90,10 @@ typedef struct {
                                   DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT (0 = 2^22, seconds; 1 makes the first workgroups of a
                                   launch give up at once: for tests of that path - every kernel still runs to its end and
                                   the workspace stays consistent) */
-    int32_t reserved[5];
+    int32_t move_workgroups_per_cu;  /* dispatch move kernel launched on a finished layout: workgroups a CU holds at a
+                                        time (2..7; 8 and more = as many as fit; 0 = six / five for the compact / expanded
+                                        layout of a large fused-cast call, no limit otherwise) */
+    int32_t reserved[4];
 } deep_ep_hip_tuning;
 
 /* Bytes of workspace needed for dispatches of up to num_max_tokens tokens.  The workspace must

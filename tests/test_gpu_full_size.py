@@ -83,8 +83,12 @@ def test_compact_fp8_dispatch_properties(name):
 
 @pytest.mark.parametrize("name", ["C3", "C4"])
 @pytest.mark.parametrize("do_expand", [False, True])
-def test_bf16_round_trip(name, do_expand):
-    """combine(dispatch(x)) = x summed once per destination row: n equal BF16 values added in fp32, rounded once."""
+@pytest.mark.parametrize("launches", [0, 1], ids=["launches_by_choice", "one_launch"])
+def test_bf16_round_trip(name, do_expand, launches, monkeypatch):
+    """combine(dispatch(x)) = x summed once per destination row: n equal BF16 values added in fp32, rounded once.
+    At this size the library's own choice is two launches for this payload; the single launch is forced as well."""
+    import deep_ep
+    monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", launches)
     case = rc.c3() if name == "C3" else rc.c4()
     E, R = case.E, case.R
     buf = _buffer(case, allow_multiple_reduction=False)

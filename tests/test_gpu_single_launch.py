@@ -83,6 +83,21 @@ def test_launches_of_changing_shape_share_one_workspace(monkeypatch):
     buf.check_device_status()
 
 
+@pytest.mark.parametrize("T", [9000, 16384])
+def test_single_launch_up_to_131072_token_lanes(T, monkeypatch):
+    """Shapes between 65536 and 131072 (token, lane) pairs: the top of what the tagged position table holds.  One and
+    two launches alternate on one workspace, where the position words of a dispatch in two launches share that table
+    with the tagged ones; every call must be exact."""
+    import deep_ep
+    case = rc.small(f"lanes{T}", T, 128, 32, 8, 8, seed=60 + T % 7, masked_ratio=0.05)
+    buf = _buffer(case, rank=3)
+    for i, launches in enumerate((1, 2, 1, 0, 2)):
+        monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", launches)
+        _check(buf, case, do_expand=bool(i % 2) and T <= 9000, payload=("cast_fp8", "bf16")[i % 2], alignment=4 if i % 2 else 1)
+        assert int(_control_words(buf).abs().sum()) == 0
+    buf.check_device_status()
+
+
 def test_many_back_to_back_launches_without_host_sync(monkeypatch):
     """50 single-launch dispatches queued without a host wait in between: the counters of launch n must have wrapped to
     zero and its generation must have advanced before launch n + 1 starts (stream order), whatever the number of

@@ -387,6 +387,7 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     d.packed_recv_src_info, d.packed_recv_layout_range = info.data_ptr(), rng.data_ptr()
     d.lane_rows = lane_rows.data_ptr()
     d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    d.tuning = _abi.Tuning.from_env()
     c = _abi.LLCombineArgs()
     c.num_src_ranks, c.src_rank_begin, c.src_token_stride = R, 0, T
     c.hidden, c.num_topk, c.num_experts, c.expert_begin, c.num_local_experts, c.num_ranks = H, K, E, 0, E_l, R
@@ -395,6 +396,7 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     c.packed_recv_src_info, c.packed_recv_layout_range, c.combined_x = info.data_ptr(), rng.data_ptr(), out.data_ptr()
     c.lane_rows = 0 if os.environ.get("BENCH_LL_SEARCH") else lane_rows.data_ptr()
     c.workspace, c.workspace_bytes = ws.data_ptr(), ws.numel()
+    c.tuning = _abi.Tuning.from_env()
     stream = torch.cuda.current_stream()
     sp = stream.cuda_stream
 

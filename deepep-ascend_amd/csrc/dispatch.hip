@@ -770,8 +770,8 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
 }
 
 // The kernels.  The single-launch forms also hold the counting and publishing code, whose register needs must not cost
-// the movers their occupancy: they are held to six wavefronts per SIMD (80 registers), the number the movers' own code
-// reaches; five resident workgroups per CU are what the move needs to saturate the memory pipeline.
+// the movers their occupancy: they are held to six wavefronts per SIMD (80 registers) - six workgroups per CU, which
+// is also where the move streams fastest (more were slower when tried with a leaner counting step, fewer are slower too).
 template <int kVecs>
 __global__ __launch_bounds__(kThreads) void dispatch_copy_kernel(const MoveParams p) {
     dispatch_copy<kVecs, false>(p);

@@ -346,6 +346,7 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
         m.cast_pairs = a->tuning.cast_pairs; m.copy_vecs = a->tuning.copy_vecs;
         m.mover_spin_limit = a->tuning.mover_spin_limit > 0 ? unsigned(a->tuning.mover_spin_limit) : (1u << 22);   // seconds
         m.move_workgroups_per_cu = a->tuning.move_workgroups_per_cu;
+        m.warm_rounds = a->tuning.warm_rounds;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 
@@ -634,6 +635,7 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.cast_pairs = a->tuning.cast_pairs; m.copy_vecs = a->tuning.copy_vecs;
         m.mover_spin_limit = a->tuning.mover_spin_limit > 0 ? unsigned(a->tuning.mover_spin_limit) : (1u << 22);   // seconds
         m.move_workgroups_per_cu = a->tuning.move_workgroups_per_cu;
+        m.warm_rounds = a->tuning.warm_rounds;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 

@@ -64,6 +64,7 @@ inline deep_ep_hip_tuning& process_tuning() {
         t.ll_combine_vecs = env("DEEP_EP_HIP_LL_COMBINE_VECS");
         t.mover_spin_limit = env("DEEP_EP_HIP_MOVER_SPIN_LIMIT");
         t.move_workgroups_per_cu = env("DEEP_EP_HIP_MOVE_WORKGROUPS_PER_CU");
+        t.warm_rounds = env("DEEP_EP_HIP_WARM_ROUNDS");
         return t;
     }();
     return tuning;
@@ -83,6 +84,7 @@ inline int32_t* tuning_field(const std::string& name) {
     if (name == "ll_combine_vecs") return &t.ll_combine_vecs;
     if (name == "mover_spin_limit") return &t.mover_spin_limit;
     if (name == "move_workgroups_per_cu") return &t.move_workgroups_per_cu;
+    if (name == "warm_rounds") return &t.warm_rounds;
     throw EPException("unknown tuning field: " + name);
 }
 

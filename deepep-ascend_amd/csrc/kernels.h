@@ -140,6 +140,9 @@ struct MoveParams {
     int payload;         // DEEP_EP_HIP_PAYLOAD_*
     int row_bytes;       // input row bytes
     int tiles;           // column tiles per token
+    unsigned warm_lds_offset;   // single-launch cast: byte offset (in the dynamic LDS) of the 4 KB landing area of the
+                                // cache-warming loads, 0 = none
+    unsigned warm_ahead;        // ... and how many work items ahead of its own a wavefront warms
     int xcd_remap;       // give each XCD a contiguous token range
     int plain_loads;     // payload loads without the non-temporal hint
     int cast_pairs;      // forced column tile of the fused cast, 0 = choose
@@ -159,6 +162,7 @@ struct MoveParams {
     uint32_t* gates_finished;    // wrapping counter of the gates all of whose movers are done
     unsigned mover_spin_limit;   // reads a mover repeats for a word of the layout before it gives up (set from the tuning block)
     int move_workgroups_per_cu;  // forced residency of a move kernel on a finished layout, 0 = choose (tuning block)
+    int warm_rounds;             // rounds ahead the first movers of a single launch warm the caches, 0 = choose, < 0 = none (tuning block)
     uint32_t* generation;        // see WorkspaceLayout
     uint32_t* tagged;            // the tagged tables, tagged_words long: cleared by the launch that uses the last tag
     int tagged_words;

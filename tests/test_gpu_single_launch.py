@@ -98,6 +98,21 @@ def test_single_launch_up_to_131072_token_lanes(T, monkeypatch):
     buf.check_device_status()
 
 
+@pytest.mark.parametrize("warm_rounds", [1, 0, -1])
+def test_cache_warming_loads_change_nothing(warm_rounds, monkeypatch):
+    """A launch with more mover workgroups than a GPU holds at a time: the first of them also load, into a piece of LDS
+    nobody reads, tiles of work items further on.  Results are the oracle's whatever the distance."""
+    import deep_ep
+    monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", 1)
+    monkeypatch.setattr(deep_ep.tuning, "warm_rounds", warm_rounds)
+    case = rc.small("warm", 3300, 7168, 64, 8, 8, seed=91, masked_ratio=0.05)       # 3300 mover workgroups
+    buf = _buffer(case, rank=2)
+    for do_expand in (False, True):
+        _check(buf, case, do_expand, "cast_fp8", alignment=4 if do_expand else 1)
+        assert int(_control_words(buf).abs().sum()) == 0
+    buf.check_device_status()
+
+
 def test_many_back_to_back_launches_without_host_sync(monkeypatch):
     """50 single-launch dispatches queued without a host wait in between: the counters of launch n must have wrapped to
     zero and its generation must have advanced before launch n + 1 starts (stream order), whatever the number of

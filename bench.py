@@ -31,15 +31,15 @@ HBM_PEAK_GBS = 8000.0
 # the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
-    ("C3", "compact", "fp8", "dispatch"): 452335662,
-    ("C3", "compact", "fp8", "combine"): 751992269,
+    ("C3", "compact", "fp8", "dispatch"): 459116312,
+    ("C3", "compact", "fp8", "combine"): 751994706,
     ("C3", "expanded", "fp8", "dispatch"): 1863758 + 612972432,
     ("C3", "expanded", "fp8", "combine"): 1074426643,
     ("C3", "compact", "bf16", "dispatch"): 1843294 + 755741042,
     ("C3", "compact", "bf16", "combine"): 751993795,
     # profiles/bench_C4_C2_hbm_counters.md
-    ("C4", "compact", "fp8", "dispatch"): 420107733,
-    ("C4", "compact", "fp8", "combine"): 690500080,
+    ("C4", "compact", "fp8", "dispatch"): 425458977,
+    ("C4", "compact", "fp8", "combine"): 690500098,
     ("C2", "compact", "bf16", "dispatch"): 97436912,
     ("C2", "compact", "bf16", "combine"): 96362178,
     # profiles/bench_C5_low_latency_hbm_counters.md

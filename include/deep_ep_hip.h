@@ -93,7 +93,7 @@ typedef struct {
     int32_t move_workgroups_per_cu;  /* dispatch move kernel launched on a finished layout: workgroups a CU holds at a
                                         time (2..7; 8 and more = as many as fit; 0 = six / five for the compact / expanded
                                         layout of a large fused-cast call, no limit otherwise) */
-    int32_t warm_rounds;       /* single-launch dispatch with the fused cast: the movers that are resident at launch also
+    int32_t warm_rounds;       /* single-launch dispatch: the movers that are resident at launch also
                                   load, into the caches only, the tiles of the work items this many rounds of resident
                                   workgroups ahead of their own (0 = 2; negative = none) */
     int32_t reserved[3];

@@ -108,8 +108,9 @@ def test_cache_warming_loads_change_nothing(warm_rounds, monkeypatch):
     case = rc.small("warm", 3300, 7168, 64, 8, 8, seed=91, masked_ratio=0.05)       # 3300 mover workgroups
     buf = _buffer(case, rank=2)
     for do_expand in (False, True):
-        _check(buf, case, do_expand, "cast_fp8", alignment=4 if do_expand else 1)
-        assert int(_control_words(buf).abs().sum()) == 0
+        for payload in ("cast_fp8", "bf16"):
+            _check(buf, case, do_expand, payload, alignment=4 if do_expand else 1)
+            assert int(_control_words(buf).abs().sum()) == 0
     buf.check_device_status()
 
 

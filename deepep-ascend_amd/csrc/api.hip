@@ -442,6 +442,22 @@ int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* a, void* stream
     return dispatch_with_workspace(a, a->workspace, a->workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+int deep_ep_hip_dispatch_kernel_launches(const deep_ep_hip_dispatch_args* a) {
+    REQUIRE(a != nullptr, "args is NULL");
+    if (int rc = check_routing_shape(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks)) return rc;
+    const bool do_layout = (a->phases & DEEP_EP_HIP_PHASE_LAYOUT) != 0;
+    const bool do_move = (a->phases & DEEP_EP_HIP_PHASE_MOVE) != 0;
+    REQUIRE(do_layout || do_move, "phases selects nothing");
+    REQUIRE(a->payload == DEEP_EP_HIP_PAYLOAD_BF16 || a->payload == DEEP_EP_HIP_PAYLOAD_FP8 ||
+            a->payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8, "unknown payload kind %d", a->payload);
+    if (a->num_tokens == 0) return do_layout ? 1 : 0;      // an empty move launches nothing
+    const int elem_in = a->payload == DEEP_EP_HIP_PAYLOAD_FP8 ? 1 : 2;
+    const LaunchPlan plan = plan_launches(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks, do_layout, do_move,
+                                          a->do_expand != 0, a->expert_alignment, a->payload, a->hidden, a->hidden * elem_in,
+                                          a->tuning);
+    return plan.fused ? 1 : int(do_layout) + int(do_move);
+}
+
 int deep_ep_hip_launch_dispatch_static(const deep_ep_hip_dispatch_args* a, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     REQUIRE(a != nullptr, "args is NULL");

@@ -245,6 +245,7 @@ EXPORTS = {
     "deep_ep_hip_launch_layout": (c_int, [POINTER(LayoutArgs), c_void_p]),
     "deep_ep_hip_launch_dispatch": (c_int, [POINTER(DispatchArgs), c_void_p]),
     "deep_ep_hip_launch_dispatch_static": (c_int, [POINTER(DispatchArgs), c_void_p]),
+    "deep_ep_hip_dispatch_kernel_launches": (c_int, [POINTER(DispatchArgs)]),
     "deep_ep_hip_launch_combine": (c_int, [POINTER(CombineArgs), c_void_p]),
     "deep_ep_hip_launch_intranode_dispatch": (c_int, [POINTER(IntranodeDispatchArgs), c_void_p]),
     "deep_ep_hip_launch_intranode_combine": (c_int, [POINTER(IntranodeCombineArgs), c_void_p]),

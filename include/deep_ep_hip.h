@@ -205,6 +205,13 @@ typedef struct {
 
 int deep_ep_hip_launch_dispatch(const deep_ep_hip_dispatch_args* args, void* stream);
 
+/* How many kernels deep_ep_hip_launch_dispatch would launch for the layout and move phases of these arguments (shape,
+ * phases, payload, do_expand, expert_alignment and tuning are read; no pointer is dereferenced, nothing is launched): 1
+ * where layout and move share a launch, else one per requested phase; 0 for a move of no tokens.  The zero-padding
+ * kernel of an expanded dispatch is not counted.  Negative: an error code.  No counterpart in the reference; for callers
+ * that size graphs or want to know which path a shape takes. */
+int deep_ep_hip_dispatch_kernel_launches(const deep_ep_hip_dispatch_args* args);
+
 /* The same dispatch for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  args->workspace and
  * args->workspace_bytes are ignored: the workspace is a device-resident array built into the library,

@@ -111,6 +111,37 @@ def test_dispatch_rejects_bad_arguments_before_launch(kw, fragment):
     assert fragment in _abi.last_error(), _abi.last_error()
 
 
+def _launches(T=8192, H=7168, K=8, E=256, R=8, payload=None, phases=None, **kw):
+    a = _abi.DispatchArgs()
+    a.phases = _abi.PHASE_LAYOUT | _abi.PHASE_MOVE if phases is None else phases
+    a.payload = _abi.PAYLOAD_CAST_FP8 if payload is None else payload
+    a.num_tokens, a.hidden, a.num_topk, a.num_experts, a.num_ranks = T, H, K, E, R
+    a.num_max_tokens_per_rank, a.expert_alignment = T, 1
+    for k, v in kw.items():
+        if k.startswith("tuning_"):
+            setattr(a.tuning, k[len("tuning_"):], v)
+        else:
+            setattr(a, k, v)
+    return _abi.lib.deep_ep_hip_dispatch_kernel_launches(ctypes.byref(a))
+
+
+def test_launch_plan_of_a_dispatch():
+    """Which shapes share one launch between layout and move (no pointer is read, nothing is launched)."""
+    assert _launches() == 1                                             # the headline shape: fused cast, compact
+    assert _launches(T=16384) == 1 and _launches(T=16385) == 2          # up to 131072 (token, lane) pairs
+    assert _launches(K=9, E=288) == 2 and _launches(E=512, R=8) == 2    # top-k <= 8, ranks + experts <= 512
+    assert _launches(do_expand=1) == 2 and _launches(T=4096, do_expand=1) == 1   # expanded: two launches from 64 MB of input on
+    assert _launches(T=4096, do_expand=1, tuning_dispatch_launches=2) == 2
+    assert _launches(do_expand=1, tuning_dispatch_launches=1) == 1
+    assert _launches(payload=_abi.PAYLOAD_BF16) == 2                    # 28672 mover workgroups: more than the single launch takes
+    assert _launches(payload=_abi.PAYLOAD_BF16, tuning_dispatch_launches=1) == 1
+    assert _launches(T=4096, H=2048, K=6, E=64, payload=_abi.PAYLOAD_BF16) == 1
+    assert _launches(tuning_cast_pairs=4) == 2                          # wide cast tiles have no single-launch kernel
+    assert _launches(phases=_abi.PHASE_LAYOUT) == 1 and _launches(phases=_abi.PHASE_MOVE) == 1
+    assert _launches(T=0) == 1 and _launches(T=0, phases=_abi.PHASE_MOVE) == 0
+    assert _launches(phases=0) == -1 and _launches(payload=9) == -1 and _launches(E=255) == -1
+
+
 def test_workspace_size_contract():
     rc = _abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(_dispatch_args(workspace_bytes=64)), None)
     assert rc == -2 and "needed" in _abi.last_error()

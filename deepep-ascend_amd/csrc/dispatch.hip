@@ -1015,7 +1015,13 @@ void plan_cache_warming(MoveParams& p) {
     p.warm_lds_offset = 0;
     if (!p.fused || p.warm_rounds < 0) return;
     const unsigned first_round = unsigned(p.num_cus) * unsigned(kResidentWorkgroupsPerCu);
-    const unsigned rounds = p.warm_rounds > 0 ? unsigned(p.warm_rounds) : 2u;
+    // By default two rounds ahead; launches of one and a half to two rounds warm their second round (3072 x 7168 fused
+    // cast: 38.2 -> 36.1 us, 3400 tokens 43.8 -> 40.6 us), shorter ones nothing (2048 tokens: 27.9 -> 28.6 us).
+    unsigned rounds = p.warm_rounds > 0 ? unsigned(p.warm_rounds) : 2u;
+    if (p.warm_rounds == 0 && uint64_t(p.num_movers) <= 2ull * first_round) {
+        if (2ull * p.num_movers <= 3ull * first_round) return;
+        rounds = 1u;
+    }
     if (uint64_t(p.num_movers) <= uint64_t(rounds) * first_round) return;
     p.warm_lds_offset = unsigned((move_lds_bytes(p) + 1023) & ~size_t(1023));
     p.warm_ahead = rounds * first_round * unsigned(kWavesPerBlock);

@@ -95,7 +95,8 @@ typedef struct {
                                         layout of a large fused-cast call, no limit otherwise) */
     int32_t warm_rounds;       /* single-launch dispatch: the movers that are resident at launch also
                                   load, into the caches only, the tiles of the work items this many rounds of resident
-                                  workgroups ahead of their own (0 = 2; negative = none) */
+                                  workgroups ahead of their own (0 = 2, or 1 in launches of one and a half to two rounds;
+                                  negative = none) */
     int32_t reserved[3];
 } deep_ep_hip_tuning;
 

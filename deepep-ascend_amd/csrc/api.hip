@@ -386,6 +386,12 @@ size_t deep_ep_hip_workspace_bytes(int num_max_tokens, int num_topk, int num_exp
     return make_workspace_layout(num_max_tokens, num_topk, num_experts, num_ranks).total_bytes;
 }
 
+size_t deep_ep_hip_combine_workspace_bytes(int num_tokens, int num_topk, int num_experts, int num_ranks) {
+    if (num_tokens < 0 || num_topk < 1 || num_experts < 1 || num_ranks < 1) return 0;
+    const size_t tables = make_workspace_layout(num_tokens, num_topk, num_experts, num_ranks).total_bytes;
+    return tables + align_up(size_t(num_tokens > 0 ? num_tokens : 1) * num_topk * 4, 256);
+}
+
 size_t deep_ep_hip_workspace_status_offset(void) { return 0; }
 
 size_t deep_ep_hip_workspace_control_bytes(void) { return make_workspace_layout(1, 1, 1, 1).expert_start; }
@@ -479,14 +485,32 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
     REQUIRE(a->rank_idx >= 0 && a->rank_idx < a->num_ranks, "rank_idx %d outside [0, %d)", a->rank_idx, a->num_ranks);
     REQUIRE(a->num_x_rows >= 0 && a->num_x_rows < (int64_t(1) << 31), "num_x_rows out of range");
     const bool any = a->num_tokens > 0;
-    REQUIRE(!any || (a->topk_idx != nullptr && a->dst_buffer_slot_idx != nullptr && a->psum_num_recv_tokens_per_rank != nullptr),
-            "handle tensors are NULL");
+    REQUIRE(!any || (a->topk_idx != nullptr && a->psum_num_recv_tokens_per_rank != nullptr), "handle tensors are NULL");
     REQUIRE(!any || a->combined_x != nullptr, "combined_x is NULL");
     REQUIRE(!any || a->x != nullptr || a->num_x_rows == 0, "x is NULL");
     REQUIRE(a->num_recv_rows >= 0, "num_recv_rows must be >= 0");
     REQUIRE(!(a->do_expand && any && a->num_recv_rows > 0 && a->recv_src_metadata == nullptr),
             "the expanded layout needs recv_src_metadata");
     REQUIRE(a->workspace != nullptr && a->workspace_bytes >= 256, "workspace is NULL or smaller than 256 bytes");
+    const int32_t* slot = a->dst_buffer_slot_idx;
+    if (slot == nullptr && any) {
+        // The handle came without its token -> row map: rebuild it behind the dispatch tables of the workspace.
+        REQUIRE(a->recv_src_metadata != nullptr || a->num_recv_rows == 0, "without dst_buffer_slot_idx the map is rebuilt from recv_src_metadata, which is NULL");
+        const size_t need = deep_ep_hip_combine_workspace_bytes(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks);
+        if (a->workspace_bytes < need)
+            return fail(DEEP_EP_HIP_ERR_WORKSPACE_TOO_SMALL, "workspace has %llu bytes, %zu needed to rebuild dst_buffer_slot_idx",
+                        (unsigned long long)a->workspace_bytes, need);
+        SlotMapParams q{};
+        q.meta = a->recv_src_metadata;
+        q.num_meta_rows = a->num_recv_rows;
+        q.psum_rank = a->psum_num_recv_tokens_per_rank;
+        q.slot = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a->workspace) +
+                                            make_workspace_layout(a->num_tokens, a->num_topk, a->num_experts, a->num_ranks).total_bytes);
+        q.T = a->num_tokens; q.K = a->num_topk; q.R = a->num_ranks; q.rank_idx = a->rank_idx; q.M = a->num_max_tokens_per_rank;
+        const hipError_t err = launch_rebuild_slot_map(q, static_cast<hipStream_t>(stream));
+        if (err != hipSuccess) return hip_fail(err, "slot map launch");
+        slot = q.slot;
+    }
     CombineParams p{};
     p.x = static_cast<const uint8_t*>(a->x);
     p.num_x_rows = a->num_x_rows;
@@ -494,7 +518,7 @@ int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* a, void* stream) 
     p.bias0 = static_cast<const uint8_t*>(a->bias_0);
     p.bias1 = static_cast<const uint8_t*>(a->bias_1);
     p.topk_idx = a->topk_idx;
-    p.slot = a->dst_buffer_slot_idx;
+    p.slot = slot;
     p.meta = a->recv_src_metadata;
     p.num_meta_rows = a->num_recv_rows;
     p.psum_rank = a->psum_num_recv_tokens_per_rank;

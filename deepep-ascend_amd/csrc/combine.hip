@@ -13,6 +13,8 @@
 // own term, in lane order.
 //
 // One wavefront owns one (token, column tile of kVecs * 512 channels).
+#include <algorithm>
+
 #include "device_utils.h"
 #include "kernels.h"
 #include "../../include/deep_ep_hip.h"
@@ -267,7 +269,47 @@ hipError_t launch(CombineParams p, hipStream_t stream) {
     return launch_layout<kVecs, kExpandedRowsReducedPerRank>(p, blocks, stream);
 }
 
+// ---- the token -> received-row map of a handle, rebuilt from the rows' own records ----
+// A compact receive row r carries (source rank * M + token, source rank * K + master lane) in the first two columns of
+// recv_src_metadata, and the rows of destination rank d are [psum[d - 1], psum[d]): so row r is slot r - psum[d - 1] of
+// the master lane of its token.  Every other entry is -1.
+__global__ __launch_bounds__(kThreads) void fill_slot_map_kernel(int32_t* slot, int64_t n) {
+    for (int64_t i = int64_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += int64_t(gridDim.x) * kThreads) slot[i] = -1;
+}
+
+__global__ __launch_bounds__(kThreads) void scatter_slot_map_kernel(const SlotMapParams p) {
+    extern __shared__ int32_t psum[];      // [R]
+    for (int i = threadIdx.x; i < p.R; i += kThreads) psum[i] = p.psum_rank[i];
+    __syncthreads();
+    const int64_t rows = min(int64_t(psum[p.R - 1]), p.num_meta_rows);
+    for (int64_t r = int64_t(blockIdx.x) * kThreads + threadIdx.x; r < rows; r += int64_t(gridDim.x) * kThreads) {
+        const int token = p.meta[r * (p.K + 2)] - p.rank_idx * p.M;
+        const int lane = p.meta[r * (p.K + 2) + 1] - p.rank_idx * p.K;
+        if (token < 0 || token >= p.T || lane < 0 || lane >= p.K) continue;       // a row of another source rank
+        int lo = 0, hi = p.R - 1;                 // first d with r < psum[d]
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (r < psum[mid]) hi = mid;
+            else lo = mid + 1;
+        }
+        const int first = lo > 0 ? psum[lo - 1] : 0;
+        p.slot[int64_t(token) * p.K + lane] = p.rank_idx * p.M + int(r - first);
+    }
+}
+
 }  // namespace
+
+hipError_t launch_rebuild_slot_map(const SlotMapParams& p, hipStream_t stream) {
+    const int64_t n = int64_t(p.T) * p.K;
+    if (n == 0) return hipSuccess;
+    const unsigned fill_blocks = unsigned(std::min<int64_t>((n + kThreads - 1) / kThreads, 2048));
+    hipLaunchKernelGGL(fill_slot_map_kernel, dim3(fill_blocks), dim3(kThreads), 0, stream, p.slot, n);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess || p.num_meta_rows == 0) return err;
+    const unsigned blocks = unsigned(std::min<int64_t>((p.num_meta_rows + kThreads - 1) / kThreads, 2048));
+    hipLaunchKernelGGL(scatter_slot_map_kernel, dim3(blocks), dim3(kThreads), size_t(p.R) * sizeof(int32_t), stream, p);
+    return hipGetLastError();
+}
 
 hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream) {
     if (p.T == 0) return hipSuccess;

@@ -1,107 +1,17 @@
 // Host side of dispatch / combine for the HIP backend: the class the `deep_ep._C` extension registers as
 // `ElasticBuffer` (the role of csrc/elastic/buffer.hpp:83-1345 on CUDA and csrc/backends/ascend/elastic_buffer.hpp on
 // Ascend).  It checks arguments, allocates the outputs, sequences the launches on the right stream and returns the
-// reference's tuples.  Torch types stop here: below this class everything goes through the C ABI of
-// include/deep_ep_hip.h (plain pointers, sizes and a stream).
+// reference's tuples.
 //
 // One GPU, logical ranks: `num_ranks` only decides which bucket (destination rank) an expert belongs to; every
 // bucket lives in this GPU's HBM.  One call moves the tokens of the logical source rank `rank_idx`.
 #pragma once
 
-#include <c10/hip/HIPFunctions.h>
-#include <pybind11/pybind11.h>
-#include <torch/types.h>
-
-#include <algorithm>
-#include <cstdint>
-#include <cstdlib>
-#include <optional>
-#include <sstream>
-#include <stdexcept>
-#include <string>
-#include <tuple>
-#include <vector>
-
-#include "../../../include/deep_ep_hip.h"
-#include "event.hpp"
+#include "runtime_base.hpp"
 
 namespace deep_ep::hip {
 
-// Host checks raise what the reference's EP_HOST_ASSERT raises: an exception Python sees as RuntimeError
-// (deep_ep/include/deep_ep/common/exception.cuh:11-34).
-class EPException : public std::runtime_error {
-public:
-    using std::runtime_error::runtime_error;
-};
-
-#define EP_HIP_HOST_ASSERT(cond)                                                                      \
-    do {                                                                                              \
-        if (!(cond)) throw ::deep_ep::hip::EPException(std::string("Assertion failed: ") + #cond);    \
-    } while (0)
-
-inline int64_t align_up(int64_t x, int64_t y) { return (x + y - 1) / y * y; }
-
-constexpr int64_t kBufferAlignmentBytes = 2 * 1024 * 1024;   // symmetric::kNumAlignmentBytes (csrc/elastic/buffer.hpp:1363-1365)
-constexpr int64_t kRecordAlignBytes = 32;                    // ptx::kNumTMAAlignBytes, used only by the size calculus
-
-// Launch-shape knobs every call passes down (all zero = the library's own choice); seeded from DEEP_EP_HIP_<NAME>.
-inline deep_ep_hip_tuning& process_tuning() {
-    static deep_ep_hip_tuning tuning = [] {
-        deep_ep_hip_tuning t{};
-        auto env = [](const char* name) {
-            const char* v = std::getenv(name);
-            return v != nullptr ? std::atoi(v) : 0;
-        };
-        t.dispatch_launches = env("DEEP_EP_HIP_DISPATCH_LAUNCHES");
-        t.cast_pairs = env("DEEP_EP_HIP_CAST_PAIRS");
-        t.copy_vecs = env("DEEP_EP_HIP_COPY_VECS");
-        t.plain_loads = env("DEEP_EP_HIP_PLAIN_LOADS");
-        t.xcd_remap = env("DEEP_EP_HIP_XCD_REMAP");
-        t.combine_vecs = env("DEEP_EP_HIP_COMBINE_VECS");
-        t.ll_pairs = env("DEEP_EP_HIP_LL_PAIRS");
-        t.ll_threads = env("DEEP_EP_HIP_LL_THREADS");
-        t.ll_two_kernels = env("DEEP_EP_HIP_LL_TWO_KERNELS");
-        t.ll_combine_vecs = env("DEEP_EP_HIP_LL_COMBINE_VECS");
-        t.mover_spin_limit = env("DEEP_EP_HIP_MOVER_SPIN_LIMIT");
-        t.move_workgroups_per_cu = env("DEEP_EP_HIP_MOVE_WORKGROUPS_PER_CU");
-        t.warm_rounds = env("DEEP_EP_HIP_WARM_ROUNDS");
-        return t;
-    }();
-    return tuning;
-}
-
-inline int32_t* tuning_field(const std::string& name) {
-    deep_ep_hip_tuning& t = process_tuning();
-    if (name == "dispatch_launches") return &t.dispatch_launches;
-    if (name == "cast_pairs") return &t.cast_pairs;
-    if (name == "copy_vecs") return &t.copy_vecs;
-    if (name == "plain_loads") return &t.plain_loads;
-    if (name == "xcd_remap") return &t.xcd_remap;
-    if (name == "combine_vecs") return &t.combine_vecs;
-    if (name == "ll_pairs") return &t.ll_pairs;
-    if (name == "ll_threads") return &t.ll_threads;
-    if (name == "ll_two_kernels") return &t.ll_two_kernels;
-    if (name == "ll_combine_vecs") return &t.ll_combine_vecs;
-    if (name == "mover_spin_limit") return &t.mover_spin_limit;
-    if (name == "move_workgroups_per_cu") return &t.move_workgroups_per_cu;
-    if (name == "warm_rounds") return &t.warm_rounds;
-    throw EPException("unknown tuning field: " + name);
-}
-
-inline void check_abi(int rc, const char* what) {
-    if (rc != 0) {
-        std::ostringstream msg;
-        msg << "DeepEP HIP backend: " << what << " failed (code " << rc << "): " << deep_ep_hip_last_error();
-        throw EPException(msg.str());
-    }
-}
-
-template <class T>
-inline T* ptr_of(const std::optional<torch::Tensor>& t) {
-    return t.has_value() ? static_cast<T*>(t->data_ptr()) : nullptr;
-}
-
-class ElasticBuffer {
+class ElasticBuffer : public HostRuntime {
 public:
     using cpu_comm_t = pybind11::object;      // there is no CPU communicator on one GPU; whatever is passed is ignored
 
@@ -109,30 +19,18 @@ public:
                   int64_t num_cpu_buffer_bytes, bool allow_hybrid_mode, bool allow_multiple_reduction,
                   bool prefer_overlap_with_compute, int /*sl_idx*/, int /*num_allocated_qps*/, int num_cpu_timeout_secs,
                   int /*num_gpu_timeout_secs*/, bool explicitly_destroy)
-        : rank_idx_(rank_idx), num_ranks_(num_ranks), num_buffer_bytes_(num_buffer_bytes),
+        : HostRuntime(rank_idx, num_ranks, explicitly_destroy), num_buffer_bytes_(num_buffer_bytes),
           allow_hybrid_mode_(allow_hybrid_mode), allow_multiple_reduction_(allow_multiple_reduction),
-          prefer_overlap_with_compute_(prefer_overlap_with_compute), num_cpu_timeout_secs_(num_cpu_timeout_secs),
-          explicitly_destroy_(explicitly_destroy), comm_stream_(make_comm_stream()), last_stream_(comm_stream_) {
-        EP_HIP_HOST_ASSERT(0 <= rank_idx and rank_idx < num_ranks);
-        EP_HIP_HOST_ASSERT(num_ranks <= DEEP_EP_HIP_MAX_RANKS);
+          prefer_overlap_with_compute_(prefer_overlap_with_compute), num_cpu_timeout_secs_(num_cpu_timeout_secs) {
         EP_HIP_HOST_ASSERT(num_buffer_bytes > 0 and num_buffer_bytes % kBufferAlignmentBytes == 0);
         EP_HIP_HOST_ASSERT(num_cpu_buffer_bytes == 0);      // CPU buffers are not supported by the HIP backend
-        device_ = torch::Device(torch::kCUDA, comm_stream_.device_index());
     }
 
     // ---- lifetime ----
     void destroy() {
-        EP_HIP_HOST_ASSERT(explicitly_destroy_);
-        EP_HIP_HOST_ASSERT(not destroyed_);
-        c10::hip::device_synchronize();
-        workspace_.reset();
-        status_read_.reset();
-        destroyed_ = true;
+        release();
+        slots_of_handle_.clear();
     }
-
-    bool is_destroyed() const { return destroyed_; }
-
-    c10::Stream get_comm_stream() const { return comm_stream_.unwrap(); }
 
     // (RDMA ranks, load/store-reachable ranks): every logical rank is local
     std::tuple<int, int> get_physical_domain_size() const { return {1, num_ranks_}; }
@@ -175,8 +73,9 @@ public:
     }
 
     // ---- dispatch: argument order and the 16-tuple follow csrc/elastic/buffer.hpp:695-728,1166-1178 ----
-    // `cast_to_fp8` (extension): `x` is BF16 and the FP8 e4m3 cast with per-1x128 fp32 scales is fused into the
-    // scatter; the result equals casting first and dispatching the pair.
+    // The 29 arguments are the reference's, in its order; `cast_to_fp8` is an extension bound as a trailing keyword
+    // with a default: `x` is BF16 and the FP8 e4m3 cast with per-1x128 fp32 scales is fused into the scatter; the
+    // result equals casting first and dispatching the pair.
     std::tuple<torch::Tensor, std::optional<torch::Tensor>, std::optional<torch::Tensor>, std::optional<torch::Tensor>,
                std::optional<torch::Tensor>, int, int, std::vector<int>, torch::Tensor, torch::Tensor, torch::Tensor,
                torch::Tensor, torch::Tensor, std::optional<torch::Tensor>, std::optional<torch::Tensor>,
@@ -383,6 +282,7 @@ public:
         args.recv_capacity = recv_src_metadata.size(0);
         args.expanded_capacity = do_expand ? num_expanded_tokens : 0;
         check_abi(deep_ep_hip_launch_dispatch(&args, stream_ptr), "dispatch");
+        if (not cached_mode) slots_of_handle_.remember(recv_src_metadata, dst_slot);
 
         std::optional<EventHandle> event = scope.finish(
             {x, sf, topk_idx, topk_weights, recv_x, recv_sf, recv_topk_idx, recv_topk_weights,
@@ -394,8 +294,12 @@ public:
     }
 
     // ---- combine: argument order and the 3-tuple follow csrc/elastic/buffer.hpp:1181-1198,1344 ----
-    // `dst_buffer_slot_idx` (the handle's token -> received-row map) is what lets a single GPU gather instead of
-    // routing rows back through a buffer; the Python wrapper passes it.
+    // The 18 arguments are the reference's, in its order.  A single GPU gathers rows through the handle's token ->
+    // received-row map (`dst_buffer_slot_idx`) instead of routing them back through a buffer, and the reference's
+    // signature does not carry that tensor: it may be given as a trailing keyword; otherwise the buffer finds the one
+    // it produced together with this `src_metadata`, and for a handle it has not seen (or whose tensors were cloned)
+    // the library rebuilds the map from `src_metadata[:, 0:2]` and the per-rank prefix, a scatter of one entry per
+    // received row.
     std::tuple<torch::Tensor, std::optional<torch::Tensor>, std::optional<EventHandle>>
     combine(const torch::Tensor& x, const std::optional<torch::Tensor>& topk_weights, const std::optional<torch::Tensor>& bias_0,
             const std::optional<torch::Tensor>& bias_1, const torch::Tensor& src_metadata, const torch::Tensor& combined_topk_idx,
@@ -404,9 +308,11 @@ public:
             const std::optional<torch::Tensor>& /*channel_linked_list*/, int num_experts, int num_max_tokens_per_rank,
             int /*num_sms*/, int /*num_qps*/, const std::optional<EventHandle>& previous_event,
             const std::optional<EventHandle>& previous_event_before_epilogue, bool async_with_compute_stream,
-            bool allocate_on_comm_stream, bool use_expanded_layout, const std::optional<torch::Tensor>& dst_buffer_slot_idx) {
+            bool allocate_on_comm_stream, bool use_expanded_layout, const std::optional<torch::Tensor>& dst_buffer_slot_idx_arg) {
         EP_HIP_HOST_ASSERT(not destroyed_);
-        EP_HIP_HOST_ASSERT(dst_buffer_slot_idx.has_value());
+        EP_HIP_HOST_ASSERT(src_metadata.is_cuda() and src_metadata.is_contiguous() and src_metadata.scalar_type() == torch::kInt32);
+        std::optional<torch::Tensor> dst_buffer_slot_idx = dst_buffer_slot_idx_arg;
+        if (not dst_buffer_slot_idx.has_value()) dst_buffer_slot_idx = slots_of_handle_.find(src_metadata);
         EP_HIP_HOST_ASSERT(x.dim() == 2 and x.is_cuda() and x.is_contiguous());
         EP_HIP_HOST_ASSERT(x.scalar_type() == torch::kBFloat16);
         const int64_t num_x_rows = x.size(0);
@@ -414,7 +320,12 @@ public:
         EP_HIP_HOST_ASSERT((hidden * 2) % 16 == 0);
         EP_HIP_HOST_ASSERT(combined_topk_idx.dim() == 2 and combined_topk_idx.scalar_type() == torch::kInt64 and combined_topk_idx.is_contiguous());
         const int num_tokens = static_cast<int>(combined_topk_idx.size(0)), num_topk = static_cast<int>(combined_topk_idx.size(1));
-        EP_HIP_HOST_ASSERT(dst_buffer_slot_idx->dim() == 2 and dst_buffer_slot_idx->size(0) == num_tokens and dst_buffer_slot_idx->size(1) == num_topk);
+        if (dst_buffer_slot_idx.has_value())
+            EP_HIP_HOST_ASSERT(dst_buffer_slot_idx->dim() == 2 and dst_buffer_slot_idx->size(0) == num_tokens and
+                               dst_buffer_slot_idx->size(1) == num_topk and dst_buffer_slot_idx->scalar_type() == torch::kInt32 and
+                               dst_buffer_slot_idx->is_contiguous());
+        EP_HIP_HOST_ASSERT(psum_num_recv_tokens_per_scaleup_rank.dim() == 1 and psum_num_recv_tokens_per_scaleup_rank.size(0) == num_ranks_ and
+                           psum_num_recv_tokens_per_scaleup_rank.scalar_type() == torch::kInt32);
         EP_HIP_HOST_ASSERT(src_metadata.dim() == 2 and src_metadata.size(1) == num_topk + 2);
         if (topk_weights.has_value()) {
             EP_HIP_HOST_ASSERT(topk_weights->scalar_type() == torch::kFloat32 and topk_weights->is_cuda() and topk_weights->is_contiguous());
@@ -455,7 +366,7 @@ public:
         args.bias_0 = bias_0.has_value() ? bias_0->data_ptr() : nullptr;
         args.bias_1 = bias_1.has_value() ? bias_1->data_ptr() : nullptr;
         args.topk_idx = static_cast<const int64_t*>(combined_topk_idx.data_ptr());
-        args.dst_buffer_slot_idx = static_cast<const int32_t*>(dst_buffer_slot_idx->data_ptr());
+        args.dst_buffer_slot_idx = ptr_of<const int32_t>(dst_buffer_slot_idx);     // NULL: rebuilt in the workspace
         args.recv_src_metadata = static_cast<const int32_t*>(src_metadata.data_ptr());
         args.num_recv_rows = src_metadata.size(0);
         args.psum_num_recv_tokens_per_rank = static_cast<const int32_t*>(psum_num_recv_tokens_per_scaleup_rank.data_ptr());
@@ -472,201 +383,15 @@ public:
         return {combined_x, combined_topk_weights, event};
     }
 
-    // ---- V1 `Buffer.get_dispatch_layout` on this buffer (csrc/legacy/buffer.hpp:337-404) ----
-    std::tuple<torch::Tensor, std::optional<torch::Tensor>, torch::Tensor, torch::Tensor, std::optional<EventHandle>>
-    get_dispatch_layout(const torch::Tensor& topk_idx, int num_experts, const std::optional<EventHandle>& previous_event,
-                        bool async_finish, bool allocate_on_comm_stream) {
-        EP_HIP_HOST_ASSERT(topk_idx.dim() == 2 and topk_idx.is_contiguous() and topk_idx.is_cuda());
-        EP_HIP_HOST_ASSERT(topk_idx.scalar_type() == torch::kInt64);
-        EP_HIP_HOST_ASSERT(num_experts > 0 and num_experts % num_ranks_ == 0);
-        const int num_tokens = static_cast<int>(topk_idx.size(0)), num_topk = static_cast<int>(topk_idx.size(1));
-        StreamScope scope(*this, previous_event, allocate_on_comm_stream, async_finish);
-        const Stream& run = scope.run_stream;
-        torch::Tensor workspace = acquire_workspace(run, num_tokens, num_topk, num_experts);
-        torch::Tensor per_rank, per_expert, in_rank;
-        {
-            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
-            const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(device_);
-            per_rank = torch::empty({num_ranks_}, i32);
-            per_expert = torch::empty({num_experts}, i32);
-            in_rank = torch::empty({num_tokens, num_ranks_}, torch::TensorOptions().dtype(torch::kBool).device(device_));
-        }
-        deep_ep_hip_layout_args args{};
-        args.topk_idx = static_cast<const int64_t*>(topk_idx.data_ptr());
-        args.num_tokens = num_tokens; args.num_topk = num_topk; args.num_experts = num_experts; args.num_ranks = num_ranks_;
-        args.num_tokens_per_rank = static_cast<int32_t*>(per_rank.data_ptr());
-        args.num_tokens_per_expert = static_cast<int32_t*>(per_expert.data_ptr());
-        args.is_token_in_rank = static_cast<uint8_t*>(in_rank.data_ptr());
-        args.workspace = workspace.data_ptr();
-        args.workspace_bytes = static_cast<uint64_t>(workspace.numel());
-        check_abi(deep_ep_hip_launch_layout(&args, run.stream()), "get_dispatch_layout");
-        std::optional<EventHandle> event = scope.finish({topk_idx, per_rank, per_expert, in_rank, workspace});
-        return {per_rank, std::nullopt, per_expert, in_rank, event};
-    }
-
-    // Synchronise and raise if a kernel flagged bad routing input or a row that did not fit the outputs.
-    void check_device_status(const std::string& what) {
-        c10::hip::device_synchronize();
-        if (workspace_.has_value()) read_and_clear_status(*workspace_, what.c_str());
-    }
-
-    // Queues, on the current stream, a copy of the status word into `out` (one int32 in pinned host memory or on the
-    // device), clearing it on the way if asked.  Capturable: a graph that holds it refreshes `out` on every replay.
-    void queue_status_read(const torch::Tensor& out, bool clear) {
-        EP_HIP_HOST_ASSERT(out.scalar_type() == torch::kInt32 and out.numel() >= 1 and (out.is_cuda() or out.is_pinned()));
-        EP_HIP_HOST_ASSERT(workspace_.has_value());                    // a dispatch or combine has run on this buffer
-        const Stream stream = current_stream();
-        if (last_stream_ != stream) stream_wait(stream, last_stream_);
-        check_abi(deep_ep_hip_read_status(workspace_->data_ptr(), out.data_ptr<int32_t>(), clear ? 1 : 0, stream.stream()),
-                  "status read");
-    }
-
-    // The status check of a loop that never waits for the GPU.  A call that finds no read in flight queues one on the
-    // current stream (deep_ep_hip_read_status in its clearing form: a small kernel moves the status word into pinned
-    // host memory and leaves the workspace ready for the next launch) and returns false.  A later call returns false
-    // while that read is still running; once it has finished, the call throws like check_device_status if a kernel had
-    // flagged something since the previous read, and returns true if nothing was flagged.
-    bool poll_device_status(const std::string& what) {
-        if (not workspace_.has_value()) return true;
-        if (not status_read_.has_value()) {
-            if (not status_host_.has_value())
-                status_host_ = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
-            queue_status_read(*status_host_, true);
-            status_read_.emplace(current_stream());
-            return false;
-        }
-        if (not status_read_->event->query()) return false;
-        status_read_.reset();
-        const int status = *status_host_->data_ptr<int32_t>();
-        if (status != 0) throw_status(status, what.c_str());
-        return true;
-    }
-
-    // The status word as the GPU has it now (every launch queued so far has finished): 0 = nothing flagged.
-    int device_status() {
-        c10::hip::device_synchronize();
-        return workspace_.has_value() ? workspace_->slice(0, 0, 4).view(torch::kInt32).item<int>() : 0;
-    }
-
-    // The counters and flags at the head of the workspace (status, launch protocol), copied to the host after a full
-    // synchronisation: between launches everything but the status word (word 0), the two row totals (words 2 and 3) and
-    // the launch generation (word 32) reads zero.
-    torch::Tensor workspace_control_words() {
-        c10::hip::device_synchronize();
-        const int64_t n = static_cast<int64_t>(deep_ep_hip_workspace_counter_bytes());
-        if (not workspace_.has_value()) return torch::zeros({n / 4}, torch::kInt32);
-        return workspace_->slice(0, 0, n).view(torch::kInt32).cpu();
-    }
+    // V1 `get_dispatch_layout` on this buffer is inherited from HostRuntime.
 
 private:
-    // The one communication stream of the buffer, at the default priority.  Fails loudly when there is no GPU.
-    static Stream make_comm_stream() {
-        if (c10::hip::device_count() <= 0) throw EPException("DeepEP HIP backend: no GPU is visible");
-        return c10::hip::getStreamFromPoolMasqueradingAsCUDA(false);
-    }
-
-    // Stream choreography of one call (csrc/elastic/buffer.hpp:528-586).  The reference always runs on its comm
-    // stream; when nothing asks for overlap the same ordering is had, without two cross-stream waits, by running on
-    // the caller's stream.  The destructor restores the current stream whatever happens in between.
-    struct StreamScope {
-        ElasticBuffer& buffer;
-        Stream compute_stream, run_stream;
-        bool allocate_on_comm_stream, async_with_compute_stream, switched = false;
-
-        StreamScope(ElasticBuffer& b, const std::optional<EventHandle>& previous_event, bool allocate_on_comm, bool async)
-            : buffer(b), compute_stream(current_stream()), run_stream(compute_stream), allocate_on_comm_stream(allocate_on_comm),
-              async_with_compute_stream(async) {
-            if (previous_event.has_value()) EP_HIP_HOST_ASSERT(allocate_on_comm_stream);
-            const bool overlap = previous_event.has_value() or allocate_on_comm_stream or async_with_compute_stream;
-            if (not overlap) return;
-            run_stream = buffer.comm_stream_;
-            if (allocate_on_comm_stream) {
-                c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(buffer.comm_stream_);
-                switched = true;
-            }
-            if (previous_event.has_value()) stream_wait(run_stream, *previous_event);
-            else if (run_stream != compute_stream) stream_wait(run_stream, compute_stream);
-        }
-
-        ~StreamScope() {
-            if (switched) c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(compute_stream);
-        }
-
-        std::optional<EventHandle> finish(std::initializer_list<std::optional<torch::Tensor>> tensors) {
-            buffer.last_stream_ = run_stream;
-            std::optional<EventHandle> event;
-            if (run_stream != compute_stream) {
-                if (async_with_compute_stream) {
-                    event = EventHandle(run_stream);
-                    const char* avoid = std::getenv("EP_AVOID_RECORD_STREAM");
-                    if (avoid != nullptr and std::atoi(avoid) != 0) {
-                        for (const auto& t : tensors)
-                            if (t.has_value()) event->tensors_to_record.push_back(t);
-                    } else {
-                        for (const auto& t : tensors) {
-                            if (t.has_value() and t->is_cuda()) {
-                                t->record_stream(compute_stream.unwrap());
-                                t->record_stream(run_stream.unwrap());
-                            }
-                        }
-                    }
-                } else {
-                    stream_wait(compute_stream, run_stream);
-                }
-            } else if (async_with_compute_stream) {
-                event = EventHandle(run_stream);
-            }
-            return event;
-        }
-    };
-
-    // The workspace is shared by every call on this buffer and is not re-entrant: a call that runs on another
-    // stream than the previous one first waits for everything queued there.  It grows geometrically, so that
-    // steady-state calls never allocate; a replaced workspace stays reserved for the stream that last used it.
-    torch::Tensor acquire_workspace(const Stream& run, int num_tokens, int num_topk, int num_experts) {
-        if (last_stream_ != run) stream_wait(run, last_stream_);
-        const int64_t need = static_cast<int64_t>(deep_ep_hip_workspace_bytes(std::max(num_tokens, 1), num_topk, num_experts, num_ranks_));
-        if (not workspace_.has_value() or workspace_->numel() < need) {
-            const int64_t size = std::max(need, 2 * (workspace_.has_value() ? workspace_->numel() : int64_t(0)));
-            if (workspace_.has_value()) workspace_->record_stream(last_stream_.unwrap());
-            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
-            workspace_ = torch::zeros({size}, torch::TensorOptions().dtype(torch::kUInt8).device(device_));
-        }
-        return *workspace_;
-    }
-
-    void read_and_clear_status(const torch::Tensor& workspace, const char* what) {
-        const int status = workspace.slice(0, 0, 4).view(torch::kInt32).item<int>();
-        if (status == 0) return;
-        // also the launch bookkeeping words that follow: a dispatch that gave up has left them mid-protocol
-        workspace.slice(0, 0, static_cast<int64_t>(deep_ep_hip_workspace_control_bytes())).zero_();
-        throw_status(status, what);
-    }
-
-    [[noreturn]] static void throw_status(int status, const char* what) {
-        std::string reasons;
-        auto add = [&](int bit, const char* text) {
-            if (status & bit) reasons += (reasons.empty() ? "" : "; ") + std::string(text);
-        };
-        add(DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE, "topk_idx holds an expert id >= num_experts");
-        add(DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT, "a token selects the same expert twice");
-        add(DEEP_EP_HIP_STATUS_ROW_OVERFLOW, "a received row did not fit the output tensors");
-        add(DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT, "a single-launch dispatch gave up waiting for its counting workgroups (outputs invalid)");
-        throw EPException(std::string("DeepEP HIP backend: ") + what + ": " + reasons);
-    }
-
-    int rank_idx_, num_ranks_;
     int64_t num_buffer_bytes_;
     bool allow_hybrid_mode_, allow_multiple_reduction_, prefer_overlap_with_compute_;
     int num_cpu_timeout_secs_;
-    bool explicitly_destroy_;
-    bool destroyed_ = false;
-    Stream comm_stream_;
-    Stream last_stream_;                     // stream of the last launch that used the workspace
-    torch::Device device_ = torch::Device(torch::kCUDA, 0);
-    std::optional<torch::Tensor> workspace_;
-    std::optional<torch::Tensor> status_host_;        // one pinned int32: where poll_device_status has the status copied
-    std::optional<EventHandle> status_read_;          // recorded after the read in flight
+    // recv_src_metadata of the dispatches of this buffer -> their dst_buffer_slot_idx: the token -> received-row map a
+    // combine gathers through, which the reference's combine signature has no argument for
+    HandleMemory slots_of_handle_;
 };
 
 }  // namespace deep_ep::hip

@@ -241,6 +241,17 @@ struct CombineParams {
 
 hipError_t launch_combine_kernel(CombineParams p, hipStream_t stream);
 
+// dst_buffer_slot_idx of a handle rebuilt from its recv_src_metadata and per-rank prefix (see combine.hip).
+struct SlotMapParams {
+    const int32_t* meta;         // [num_meta_rows, K + 2]
+    int64_t num_meta_rows;
+    const int32_t* psum_rank;    // [R] inclusive
+    int32_t* slot;               // [T, K] out
+    int T, K, R, rank_idx, M;
+};
+
+hipError_t launch_rebuild_slot_map(const SlotMapParams& p, hipStream_t stream);
+
 struct CastParams {
     const uint8_t* x;
     uint8_t* out;

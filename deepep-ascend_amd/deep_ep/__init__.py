@@ -2,8 +2,7 @@
 reference's deep_ep/__init__.py:92-109).  The HIP kernel library is loaded at import; without it
 the import fails (there is no fallback path)."""
 from . import _abi  # noqa: F401  (loads libdeep_ep_hip.so or raises)
-from ._binding import EventHandle, topk_idx_t, tuning
-from ._runtime import Config
+from ._binding import Config, EventHandle, topk_idx_t, tuning
 from .buffers.elastic import ElasticBuffer, EPHandle, LogicalGroup
 from .buffers.legacy import Buffer
 from .utils.event import EventOverlap

@@ -8,7 +8,7 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
 LIB_NAME = "libdeep_ep_hip.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 PHASE_LAYOUT = 1
 PHASE_MOVE = 2
@@ -247,6 +247,7 @@ EXPORTS = {
     "deep_ep_hip_launch_dispatch_static": (c_int, [POINTER(DispatchArgs), c_void_p]),
     "deep_ep_hip_dispatch_kernel_launches": (c_int, [POINTER(DispatchArgs)]),
     "deep_ep_hip_launch_combine": (c_int, [POINTER(CombineArgs), c_void_p]),
+    "deep_ep_hip_combine_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "deep_ep_hip_launch_intranode_dispatch": (c_int, [POINTER(IntranodeDispatchArgs), c_void_p]),
     "deep_ep_hip_launch_intranode_combine": (c_int, [POINTER(IntranodeCombineArgs), c_void_p]),
     "deep_ep_hip_ll_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

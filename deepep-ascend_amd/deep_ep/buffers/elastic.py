@@ -161,8 +161,6 @@ class ElasticBuffer:
 
     def get_comm_stream(self) -> torch.cuda.Stream:
         ts = self.runtime.get_comm_stream()
-        if isinstance(ts, torch.cuda.Stream):
-            return ts
         return torch.cuda.Stream(stream_id=ts.stream_id, device_index=ts.device_index, device_type=ts.device_type)
 
     def get_physical_domain_size(self) -> Tuple[int, int]:
@@ -248,7 +246,7 @@ class ElasticBuffer:
             unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
             async_with_compute_stream, allocate_on_comm_stream,
             do_handle_copy, do_cpu_sync, do_expand, do_zero_padding, use_tma_aligned_col_major_sf,
-            cast_to_fp8)
+            cast_to_fp8=cast_to_fp8)
 
         if handle is None:
             kept_topk_idx = cloned_topk_idx if do_handle_copy else topk_idx      # without a copy the handle aliases the caller's tensor
@@ -292,7 +290,7 @@ class ElasticBuffer:
             handle.channel_linked_list, handle.num_experts, handle.num_max_tokens_per_rank,
             num_sms or handle.num_sms, num_qps, unwrap_event(previous_event), unwrap_event(previous_event_before_epilogue),
             async_with_compute_stream, allocate_on_comm_stream, handle.do_expand,
-            handle.dst_buffer_slot_idx)
+            dst_buffer_slot_idx=handle.dst_buffer_slot_idx)
         return combined_x, combined_topk_weights, EventOverlap(event)
 
     def check_device_status(self) -> None:

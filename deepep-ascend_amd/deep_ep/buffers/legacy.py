@@ -1,7 +1,7 @@
 """`Buffer`: the part of the V1 Python surface that sits on the routing hot path —
 `get_dispatch_layout`, `dispatch` / `combine` inside one scale-up domain, and the low-latency packed
-dispatch / combine (reference deep_ep/buffers/legacy.py:293-455, 553-670; host side
-csrc/legacy/buffer.hpp:337-860, 1463-1715).
+dispatch / combine (reference deep_ep/buffers/legacy.py:293-455, 553-689).  The work is done by the compiled
+host class `deep_ep._C.Buffer` (csrc/host/legacy_buffer.hpp), which takes the reference's positional arguments.
 
 `dispatch` moves the tokens of logical source rank `group.rank()`; the received rows are the concatenation
 over destination ranks d of what d gets from this source, in token order (rows of destination d start at
@@ -17,13 +17,11 @@ rank.  The packed buffers returned by `low_latency_dispatch` are those of destin
     i.e. everything destination rank `group.rank()` would receive in a real R-rank run.
 Rows of one expert are filled by source rank ascending, then token ascending.
 """
-import ctypes
-from typing import Callable, List, Optional, Tuple, Union
+from typing import Optional, Tuple, Union
 
 import torch
 
-from .. import _abi, _binding
-from .. import _runtime as _C
+from .. import _binding as _C
 from ..platform import unwrap_event
 from ..utils.event import EventOverlap
 
@@ -39,11 +37,8 @@ class Buffer:
         # sizes and mode are recorded as given; the rows land in the tensors the calls return, not in these buffers
         self.num_nvl_bytes, self.num_rdma_bytes, self.low_latency_mode = num_nvl_bytes, num_rdma_bytes, low_latency_mode
         self.explicitly_destroy = explicitly_destroy
-        self.runtime = _C.ElasticBuffer(self.rank, self.group_size, 0, [], _C.get_elastic_buffer_alignment(), 0,
-                                        False, True, True, 0, 0, 300, 100, explicitly_destroy)
-        self._ll_workspace: Optional[torch.Tensor] = None
-        self._ll_combine_buffer: Optional[torch.Tensor] = None
-        self._ll_lane_rows = None
+        self.runtime = _C.Buffer(self.rank, self.group_size, num_nvl_bytes, num_rdma_bytes, low_latency_mode,
+                                 explicitly_destroy, enable_shrink, False)
 
     def destroy(self) -> None:
         assert self.explicitly_destroy, 'construct with explicitly_destroy=True to release by hand'
@@ -52,7 +47,7 @@ class Buffer:
 
     @staticmethod
     def capture() -> EventOverlap:
-        return EventOverlap(_binding.EventHandle())
+        return EventOverlap(_C.EventHandle())
 
     @staticmethod
     def is_sm90_compiled() -> bool:
@@ -60,30 +55,28 @@ class Buffer:
         return True
 
     def get_comm_stream(self) -> torch.cuda.Stream:
-        return self.runtime.get_comm_stream()
+        ts = self.runtime.get_comm_stream()
+        return torch.cuda.Stream(stream_id=ts.stream_id, device_index=ts.device_index, device_type=ts.device_type)
+
+    def get_local_buffer_tensor(self, *args, **kwargs):
+        raise NotImplementedError('the HIP backend stages nothing: there is no buffer to look into')
 
     def clean_low_latency_buffer(self, num_max_dispatch_tokens_per_rank: int, hidden: int, num_experts: int) -> None:
         """Nothing is staged between calls on one GPU, so there is nothing to clean
         (deep_ep/buffers/legacy.py:538-551)."""
+        self.runtime.clean_low_latency_buffer(num_max_dispatch_tokens_per_rank, hidden, num_experts)
 
     def internode_dispatch(self, *args, **kwargs):
-        raise NotImplementedError('the HIP backend has one scale-up domain: there are no RDMA ranks to dispatch to')
+        return self.runtime.internode_dispatch(*args, **kwargs)        # raises NotImplementedError
 
     def internode_combine(self, *args, **kwargs):
-        raise NotImplementedError('the HIP backend has one scale-up domain: there are no RDMA ranks to combine from')
+        return self.runtime.internode_combine(*args, **kwargs)         # raises NotImplementedError
 
     @staticmethod
     def get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
                                        num_experts: int) -> int:
         """Bytes the reference would reserve (csrc/legacy/config.hpp:131-188); nothing is staged here."""
-        num_scales = hidden // 128
-        msg = 16 + max(hidden * 2, hidden + num_scales * 4)
-        combine_msg = num_scales * 4 + hidden * 2
-        send = max(num_max_dispatch_tokens_per_rank * msg, num_experts * num_max_dispatch_tokens_per_rank * combine_msg)
-        recv = num_experts * num_max_dispatch_tokens_per_rank * max(msg, combine_msg)
-        signal = num_experts * 4
-        total = 2 * (send + recv + signal)
-        return (total + 127) // 128 * 128
+        return _C.get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts)
 
     def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
                             previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
@@ -182,11 +175,6 @@ class Buffer:
             unwrap_event(previous_event), async_finish, allocate_on_comm_stream)
         return combined_x, combined_topk_weights, EventOverlap(event)
 
-    def _workspace(self, num_bytes: int) -> torch.Tensor:
-        if self._ll_workspace is None or self._ll_workspace.numel() < num_bytes:
-            self._ll_workspace = torch.zeros(max(num_bytes, 4096), dtype=torch.uint8, device=self.runtime.device)
-        return self._ll_workspace
-
     def low_latency_dispatch(self, x: torch.Tensor, topk_idx: torch.Tensor,
                              num_max_dispatch_tokens_per_rank: int, num_experts: int,
                              cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
@@ -209,83 +197,22 @@ class Buffer:
         to powers of two (csrc/kernels/legacy/utils.cuh:481-503) and with `use_ue8m0` returned as exponent bytes
         packed four to an int32: `[E/R, R*M, hidden // 512]`, column-major in the last two dimensions.
         """
-        assert not round_scale or use_fp8, '`round_scale` needs `use_fp8`'
-        assert not use_ue8m0 or round_scale, '`use_ue8m0` needs `round_scale`'
-        assert not (return_recv_hook and async_finish), 'a receive hook and `async_finish` exclude each other'
-        R, M = self.group_size, num_max_dispatch_tokens_per_rank
-        assert x.dtype == torch.bfloat16 and x.is_contiguous() and x.is_cuda
-        assert topk_idx.is_contiguous() and topk_idx.dtype == _C.topk_idx_t
-        assert num_experts % R == 0
-        if x.dim() == 3:
-            S, T, H = x.shape
-            assert S == R and tuple(topk_idx.shape[:2]) == (S, T), 'stacked input must cover all logical source ranks'
-            src_begin = 0
-        else:
-            assert x.dim() == 2 and topk_idx.dim() == 2 and x.shape[0] == topk_idx.shape[0]
-            (T, H), S, src_begin = x.shape, 1, self.rank
-        K = topk_idx.shape[-1]
-        assert T <= M and H % 16 == 0 and (not use_fp8 or H % 128 == 0)
-        assert (R * M) % 4 == 0, 'the number of rows per expert must be a multiple of 4'
-        E_l = num_experts // R
-        dev = x.device
-        rows = R * M
-
-        compute_stream, run_stream = self.runtime._prologue(None, False, async_finish)
-        with torch.cuda.stream(run_stream):
-            packed_recv_x = torch.empty((E_l, rows, H), dtype=torch.float8_e4m3fn if use_fp8 else torch.bfloat16, device=dev)
-            packed_recv_src_info = torch.empty((E_l, rows), dtype=torch.int32, device=dev)
-            # ranges of source ranks that do not send in this call stay (begin 0, count 0)
-            packed_recv_layout_range = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
-            packed_recv_count = torch.empty((E_l,), dtype=torch.int32, device=dev)
-            lane_rows = torch.empty((S * T, K), dtype=torch.int32, device=dev)
-            packed_recv_x_scales = None
-            if use_fp8 and use_ue8m0:
-                assert H % 512 == 0
-                packed_recv_x_scales = torch.empty((E_l, H // 512, rows), dtype=torch.int32, device=dev).transpose(1, 2)
-            elif use_fp8:
-                packed_recv_x_scales = torch.empty((E_l, H // 128, rows), dtype=torch.float32, device=dev).transpose(1, 2)
-            if T > 0:
-                ws = self._workspace(_abi.lib.deep_ep_hip_ll_workspace_bytes(S, T, K, E_l))
-                args = _abi.LLDispatchArgs()
-                args.tuning = _abi.tuning
-                args.use_fp8, args.round_scale, args.use_ue8m0 = int(use_fp8), int(round_scale), int(use_ue8m0)
-                args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
-                args.num_tokens_per_src = 0
-                args.hidden, args.num_topk, args.num_experts = H, K, num_experts
-                args.expert_begin, args.num_local_experts = self.rank * E_l, E_l
-                args.num_ranks, args.num_max_dispatch_tokens_per_rank = R, M
-                args.x, args.topk_idx = _abi.ptr(x), _abi.ptr(topk_idx)
-                args.packed_recv_x = _abi.ptr(packed_recv_x)
-                args.packed_recv_x_scales = _abi.ptr(packed_recv_x_scales)
-                args.packed_recv_count = _abi.ptr(packed_recv_count)
-                args.packed_recv_src_info = _abi.ptr(packed_recv_src_info)
-                args.packed_recv_layout_range = _abi.ptr(packed_recv_layout_range)
-                args.cumulative_local_expert_recv_stats = _abi.ptr(cumulative_local_expert_recv_stats)
-                args.lane_rows = _abi.ptr(lane_rows)
-                args.workspace, args.workspace_bytes = _abi.ptr(ws), ws.numel()
-                _abi.check(_abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(args), run_stream.cuda_stream),
-                           "low_latency_dispatch")
-            else:
-                packed_recv_count.zero_()
+        (packed_recv_x, packed_recv_x_scales, packed_recv_count, packed_recv_src_info, packed_recv_layout_range, event,
+         hook) = self.runtime.low_latency_dispatch(x, topk_idx, cumulative_local_expert_recv_stats,
+                                                   dispatch_wait_recv_cost_stats, num_max_dispatch_tokens_per_rank,
+                                                   num_experts, use_fp8, round_scale, use_ue8m0, async_finish,
+                                                   return_recv_hook)
+        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, x.size(-1), num_experts)
         tensors = (x, topk_idx, packed_recv_x, packed_recv_x_scales, packed_recv_count, packed_recv_src_info,
                    packed_recv_layout_range, cumulative_local_expert_recv_stats)
-        event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
-        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H, num_experts)
-        # The handle keeps the reference's five fields; the packed row of every (token, lane) rides beside it and
-        # lets the combine of this very handle skip its search through src_info.
-        self._ll_lane_rows = (packed_recv_src_info, lane_rows, tuple(topk_idx.shape)) if T > 0 else None
         recv = (packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x
-        hook = (lambda: None) if return_recv_hook else None
         return recv, packed_recv_count, handle, EventOverlap(event, tensors if async_finish else None), hook
 
     def get_next_low_latency_combine_buffer(self, handle: tuple) -> torch.Tensor:
         """`[E/R, R*M, hidden]` BF16 buffer a caller may fill instead of passing `x` to `low_latency_combine`
         (`zero_copy=True`), deep_ep/buffers/legacy.py:673-689."""
-        src_info, layout_range, M, H, num_experts = handle
-        shape = (num_experts // self.group_size, self.group_size * M, H)
-        if self._ll_combine_buffer is None or tuple(self._ll_combine_buffer.shape) != shape:
-            self._ll_combine_buffer = torch.empty(shape, dtype=torch.bfloat16, device=self.runtime.device)
-        return self._ll_combine_buffer
+        src_info, layout_range, num_max_dispatch_tokens_per_rank, hidden, num_experts = handle
+        return self.runtime.get_next_low_latency_combine_buffer(num_max_dispatch_tokens_per_rank, hidden, num_experts)
 
     def low_latency_combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
                             handle: tuple, use_logfmt: bool = False, zero_copy: bool = False,
@@ -304,54 +231,9 @@ class Buffer:
         is not a multiple of 1024) whose 128-channel groups all have amax < 1 come back as 9-bit logarithmic codes,
         the others unchanged.  Needs hidden % 512 == 0 and excludes `zero_copy` (internode_ll.cu:1182).
         """
-        if use_logfmt and zero_copy:
-            raise RuntimeError('Assertion failed: not (zero_copy and use_logfmt)')
-        assert not (return_recv_hook and async_finish), 'a receive hook and `async_finish` exclude each other'
-        src_info, layout_range, M, H, num_experts = handle
-        if zero_copy:
-            assert self._ll_combine_buffer is not None, 'call get_next_low_latency_combine_buffer() first'
-            x = self._ll_combine_buffer
-        R = self.group_size
-        E_l = num_experts // R
-        assert x.dtype == torch.bfloat16 and x.is_contiguous() and tuple(x.shape) == (E_l, R * M, H)
-        assert topk_idx.is_contiguous() and topk_idx.dtype == _C.topk_idx_t
-        assert topk_weights.is_contiguous() and topk_weights.dtype == torch.float32
-        assert topk_idx.shape == topk_weights.shape
-        if topk_idx.dim() == 3:
-            S, T, K = topk_idx.shape
-            assert S == R
-            src_begin, out_shape = 0, (S, T, H)
-        else:
-            T, K = topk_idx.shape
-            S, src_begin, out_shape = 1, self.rank, (T, H)
-        compute_stream, run_stream = self.runtime._prologue(None, False, async_finish)
-        with torch.cuda.stream(run_stream):
-            if out is None:
-                combined_x = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)
-            else:
-                assert tuple(out.shape) == out_shape and out.dtype == torch.bfloat16 and out.is_contiguous()
-                combined_x = out
-            if T > 0:
-                ws = self._workspace(4096)
-                args = _abi.LLCombineArgs()
-                args.tuning = _abi.tuning
-                args.num_src_ranks, args.src_rank_begin, args.src_token_stride = S, src_begin, T
-                args.use_logfmt = int(use_logfmt)
-                args.num_tokens_per_src = 0
-                args.hidden, args.num_topk, args.num_experts = H, K, num_experts
-                args.expert_begin, args.num_local_experts, args.num_ranks = self.rank * E_l, E_l, R
-                args.num_max_dispatch_tokens_per_rank = M
-                args.x, args.topk_idx, args.topk_weights = _abi.ptr(x), _abi.ptr(topk_idx), _abi.ptr(topk_weights)
-                args.packed_recv_src_info = _abi.ptr(src_info)
-                args.packed_recv_layout_range = _abi.ptr(layout_range)
-                cached = self._ll_lane_rows
-                if cached is not None and cached[0] is src_info and cached[2] == tuple(topk_idx.shape):
-                    args.lane_rows = _abi.ptr(cached[1])
-                args.combined_x = _abi.ptr(combined_x)
-                args.workspace, args.workspace_bytes = _abi.ptr(ws), ws.numel()
-                _abi.check(_abi.lib.deep_ep_hip_launch_ll_combine(ctypes.byref(args), run_stream.cuda_stream),
-                           "low_latency_combine")
+        src_info, layout_range, num_max_dispatch_tokens_per_rank, hidden, num_experts = handle
+        combined_x, event, hook = self.runtime.low_latency_combine(
+            x, topk_idx, topk_weights, src_info, layout_range, combine_wait_recv_cost_stats,
+            num_max_dispatch_tokens_per_rank, num_experts, use_logfmt, zero_copy, async_finish, return_recv_hook, out)
         tensors = (x, topk_idx, topk_weights, src_info, layout_range, combined_x)
-        event = self.runtime._epilogue(list(tensors), compute_stream, run_stream, False, async_finish)
-        hook = (lambda: None) if return_recv_hook else None
         return combined_x, EventOverlap(event, tensors if async_finish else None), hook

@@ -2,7 +2,7 @@
 deep_ep/platform.py:9-80, which only knows "cuda" and "ascend")."""
 import torch
 
-from . import _binding, _runtime
+from . import _binding
 
 
 def get_platform() -> str:
@@ -19,7 +19,7 @@ def capture_event():
 
 def unwrap_event(event):
     """EventOverlap or EventHandle or None -> EventHandle or None."""
-    is_handle = isinstance(event, (_binding.EventHandle, _runtime.EventHandle))
+    is_handle = isinstance(event, _binding.EventHandle)
     return getattr(event, "event", event) if event is not None and not is_handle else event
 
 

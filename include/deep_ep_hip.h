@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define DEEP_EP_HIP_ABI_VERSION 3
+#define DEEP_EP_HIP_ABI_VERSION 4
 
 #define DEEP_EP_HIP_OK 0
 #define DEEP_EP_HIP_ERR_INVALID_ARGUMENT (-1)
@@ -240,7 +240,10 @@ typedef struct {
     const void* bias_0;                 /* bf16 [num_tokens, hidden] or NULL */
     const void* bias_1;
     const int64_t* topk_idx;            /* handle: [num_tokens, num_topk] */
-    const int32_t* dst_buffer_slot_idx; /* handle: [num_tokens, num_topk] */
+    const int32_t* dst_buffer_slot_idx; /* handle: [num_tokens, num_topk], or NULL: the call first rebuilds the map from
+                                           recv_src_metadata[:, 0:2] and psum_num_recv_tokens_per_rank (two small
+                                           launches) into the workspace, which must then hold
+                                           deep_ep_hip_combine_workspace_bytes() bytes */
     const int32_t* recv_src_metadata;   /* handle: [num_recv_rows, num_topk + 2] (expanded layout) */
     int64_t num_recv_rows;              /* rows of recv_src_metadata */
     const int32_t* psum_num_recv_tokens_per_rank; /* handle: [num_ranks] */
@@ -252,6 +255,10 @@ typedef struct {
 } deep_ep_hip_combine_args;
 
 int deep_ep_hip_launch_combine(const deep_ep_hip_combine_args* args, void* stream);
+/* Workspace a combine needs when it has to rebuild dst_buffer_slot_idx: the dispatch workspace of the same shape
+ * (deep_ep_hip_workspace_bytes, left untouched, so that dispatch and combine can share one allocation) followed by the
+ * rebuilt map.  A combine that is given dst_buffer_slot_idx needs 256 bytes (the status word). */
+size_t deep_ep_hip_combine_workspace_bytes(int num_tokens, int num_topk, int num_experts, int num_ranks);
 
 /* ------------------------------------------------------------------------------------------
  * V1 `Buffer.dispatch` / `Buffer.combine` inside one scale-up domain (the reference's "intranode" pair),

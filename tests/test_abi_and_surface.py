@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "deep_ep_hip.h")
 
 import deep_ep
-from deep_ep import _C, _abi, _runtime
+from deep_ep import _C, _abi
 
 
 def header_functions():
@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(_abi.lib, name), f"{name} is declared in the header but not exported"
     assert sorted(_abi.EXPORTS) == names, "ctypes binding table and header disagree"
-    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 3
+    assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 4
 
 
 def test_ctypes_structs_match_the_header_layout():
@@ -149,6 +149,8 @@ def test_workspace_size_contract():
     assert need(0, 2, 8, 2) > 0 and need(8192, 8, 256, 8) >= need(4096, 8, 256, 8) >= need(128, 2, 8, 2)
     assert need(8192, 8, 256, 8) % 256 == 0 and need(8192, 8, 256, 8) < (1 << 21)
     assert need(-1, 8, 256, 8) == 0 and _abi.lib.deep_ep_hip_ll_workspace_bytes(8, 128, 8, 32) > 0
+    # a combine that rebuilds the handle's token -> row map keeps it behind the dispatch tables
+    assert _abi.lib.deep_ep_hip_combine_workspace_bytes(8192, 8, 256, 8) == need(8192, 8, 256, 8) + 8192 * 8 * 4
     with pytest.raises(RuntimeError, match="DeepEP HIP backend"):
         _abi.check(-1, "probe")
 
@@ -236,12 +238,22 @@ def test_no_product_module_touches_the_oracle():
 # The reference's binding contract (tests/platform/api_contract.py:1-42): names every platform's `_C` has, and what
 # this platform adds (the Ascend build adds `is_destroyed` in the same way).
 COMMON_MODULE_NAMES = {"get_platform", "topk_idx_t", "EventHandle", "ElasticBuffer", "calculate_elastic_buffer_size"}
+# V1 names of the reference's extension (csrc/legacy/buffer.hpp:1751-1787) and the `Buffer` methods that exist on one
+# GPU; sync / IPC / NVSHMEM handles and the mask-buffer calls of shrink mode have no meaning here and are absent.
+LEGACY_MODULE_NAMES = {"Config", "Buffer", "get_low_latency_rdma_size_hint"}
+LEGACY_BUFFER_METHODS = {"is_available", "get_num_rdma_ranks", "get_rdma_rank", "get_root_rdma_rank", "get_local_device_id",
+                         "get_comm_stream", "destroy", "get_dispatch_layout", "intranode_dispatch", "intranode_combine",
+                         "internode_dispatch", "internode_combine", "clean_low_latency_buffer", "low_latency_dispatch",
+                         "low_latency_combine", "get_next_low_latency_combine_buffer"}
+REFERENCE_LEGACY_METHODS_ABSENT = {"get_local_ipc_handle", "get_local_nvshmem_unique_id", "get_local_buffer_tensor", "sync",
+                                   "low_latency_update_mask_buffer", "low_latency_query_mask_buffer",
+                                   "low_latency_clean_mask_buffer"}
+STATUS_METHODS = {"is_destroyed", "check_device_status", "poll_device_status", "queue_status_read", "device_status",
+                  "workspace_control_words"}
 COMMON_BUFFER_METHODS = {"destroy", "get_comm_stream", "get_physical_domain_size", "get_logical_domain_size", "barrier",
                          "dispatch", "combine"}
 HIP_ONLY_MODULE_NAMES = {"EPException", "get_elastic_buffer_alignment", "set_tuning", "get_tuning", "abi_version"}
-HIP_ONLY_BUFFER_METHODS = {"is_destroyed", "get_dispatch_layout", "check_device_status", "poll_device_status", "queue_status_read",
-                           "device_status",
-                           "workspace_control_words"}
+HIP_ONLY_BUFFER_METHODS = {"get_dispatch_layout"} | STATUS_METHODS
 
 
 def _public(obj):
@@ -254,8 +266,11 @@ def test_compiled_extension_has_exactly_the_contract_names():
     assert _C.__file__.endswith(".so") and deep_ep._binding.name == "pybind" and deep_ep._binding.compiled is _C
     assert _C.get_platform() == "hip" and deep_ep.platform.get_platform() == "hip"
     assert _C.topk_idx_t == torch.int64 == deep_ep.topk_idx_t
-    assert _public(_C) == COMMON_MODULE_NAMES | HIP_ONLY_MODULE_NAMES
+    assert _public(_C) == COMMON_MODULE_NAMES | LEGACY_MODULE_NAMES | HIP_ONLY_MODULE_NAMES
     assert _public(_C.ElasticBuffer) == COMMON_BUFFER_METHODS | HIP_ONLY_BUFFER_METHODS
+    assert _public(_C.Buffer) == LEGACY_BUFFER_METHODS | STATUS_METHODS
+    assert not (_public(_C.Buffer) & REFERENCE_LEGACY_METHODS_ABSENT)
+    assert _public(_C.Config) == {"num_sms", "get_nvl_buffer_size_hint", "get_rdma_buffer_size_hint"}
     assert _public(_C.EventHandle) == {"current_stream_wait"} and hasattr(_C.EventHandle, "__copy__")
     assert _C.abi_version() == _abi.ABI_VERSION
     with pytest.raises(RuntimeError):          # host checks surface as RuntimeError (exception.cuh:11-34)
@@ -269,26 +284,31 @@ def test_compiled_extension_has_exactly_the_contract_names():
         _C.set_tuning("no_such_knob", 1)
 
 
-def test_ctypes_binding_can_be_selected():
-    env = dict(os.environ, DEEP_EP_HIP_BINDING="ctypes", PYTHONPATH=os.path.join(ROOT, "deepep-ascend_amd"))
-    code = "import deep_ep; print(deep_ep._binding.name, deep_ep.EventHandle.__module__)"
-    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True)
-    assert res.returncode == 0 and res.stdout.split() == ["ctypes", "deep_ep._runtime"], res.stderr
+def test_missing_extension_fails_loudly():
+    """There is one host runtime: without the compiled extension the package does not import (no silent second path)."""
+    with tempfile.TemporaryDirectory() as tmp:
+        pkg = os.path.join(tmp, "deep_ep")
+        os.makedirs(os.path.join(pkg, "buffers")); os.makedirs(os.path.join(pkg, "utils"))
+        src = os.path.join(ROOT, "deepep-ascend_amd", "deep_ep")
+        for dirpath, _, files in os.walk(src):
+            for f in files:
+                if f.endswith(".py") or f == _abi.LIB_NAME:
+                    rel = os.path.relpath(os.path.join(dirpath, f), src)
+                    os.symlink(os.path.join(dirpath, f), os.path.join(pkg, rel))
+        res = subprocess.run([sys.executable, "-c", "import deep_ep"], env=dict(os.environ, PYTHONPATH=tmp), capture_output=True, text=True)
+    assert res.returncode != 0 and "ImportError" in res.stderr and "deep_ep._C" in res.stderr and "no fallback" in res.stderr
 
 
 def test_module_surface():
-    for name in ("ElasticBuffer", "EPHandle", "EventOverlap", "EventHandle", "Buffer", "topk_idx_t", "__version__"):
+    for name in ("ElasticBuffer", "EPHandle", "EventOverlap", "EventHandle", "Buffer", "Config", "topk_idx_t", "__version__"):
         assert hasattr(deep_ep, name)
     assert deep_ep.topk_idx_t == torch.int64
-    for runtime in (_C, _runtime):
-        assert COMMON_MODULE_NAMES <= _public(runtime)
-        assert runtime.get_platform() == "hip"
-        assert COMMON_BUFFER_METHODS <= _public(runtime.ElasticBuffer)
-        assert callable(runtime.EventHandle.current_stream_wait) and hasattr(runtime.EventHandle, "__copy__")
-    assert hasattr(_runtime.ElasticBuffer, "cpu_comm_t")
+    assert deep_ep.Config is _C.Config and deep_ep.EventHandle is _C.EventHandle
+    assert callable(_C.EventHandle.current_stream_wait) and hasattr(_C.EventHandle, "__copy__")
+    assert not hasattr(deep_ep, "_runtime")
 
 
-def test_tuning_reaches_both_runtimes():
+def test_tuning_reaches_the_runtime_and_the_raw_abi_block():
     deep_ep.tuning.combine_vecs = 4
     try:
         assert _abi.tuning.combine_vecs == 4 and _C.get_tuning("combine_vecs") == 4 and deep_ep.tuning.combine_vecs == 4
@@ -333,18 +353,50 @@ def test_signatures_are_drop_in():
                                                 "async_finish", "allocate_on_comm_stream"]
     assert _params(deep_ep.Buffer.combine) == ["x", "handle", "topk_weights", "bias", "config", "previous_event",
                                                "async_finish", "allocate_on_comm_stream"]
-    assert len(_params(_runtime.ElasticBuffer.intranode_dispatch)) == 17     # the binding's 16 + cached_send_head
-    assert len(_params(_runtime.ElasticBuffer.intranode_combine)) == 12
     assert deep_ep.Buffer.is_sm90_compiled() and deep_ep.Config(20, 6, 256).num_sms == 20
-    # the Python runtime keeps the positional order of the compiled binding (29 dispatch / 18 combine arguments, then
-    # extensions); pybind prints the compiled signatures into the docstrings
-    R = _runtime.ElasticBuffer
-    assert len(_params(R.dispatch)) == 30 and _params(R.dispatch)[-1] == "cast_to_fp8"
-    assert len(_params(R.combine)) == 19 and _params(R.combine)[-1] == "dst_buffer_slot_idx"
-    assert len(_params(R.__init__)) == 14
-    assert _C.ElasticBuffer.dispatch.__doc__.split("->")[0].count("arg") == 30
-    assert _C.ElasticBuffer.combine.__doc__.split("->")[0].count("arg") == 19
-    assert _C.ElasticBuffer.__init__.__doc__.split("->")[0].count("arg") == 14
+
+
+def _arg_names(method):
+    text = method.__doc__.split(" -> ")[0]
+    return [n for n in re.findall(r"(\w+): ", text) if n != "self"]
+
+
+def test_compiled_signatures_take_the_reference_positional_calls():
+    """The reference calls its extension positionally: 29 arguments for `ElasticBuffer.dispatch`
+    (csrc/elastic/buffer.hpp:704-728, deep_ep/buffers/elastic.py:1517-1549), 18 for `combine` (:1182-1198, :1695-1710),
+    16 / 12 for the V1 pair (csrc/legacy/buffer.hpp:417-432, :719-731), 11 / 13 for the low-latency pair (:1463-1473,
+    :1598-1611), 8 for the `Buffer` constructor (:83-91), 14 for `ElasticBuffer` (csrc/elastic/binding.hpp:24-27).
+    What this backend adds comes after those, as keywords with defaults."""
+    E, B = _C.ElasticBuffer, _C.Buffer
+    d = _arg_names(E.dispatch)
+    assert len(d) == 30 and d[-1] == "cast_to_fp8" and d[28] == "use_tma_aligned_col_major_sf" and d[0:3] == ["x", "sf", "topk_idx"]
+    assert "cast_to_fp8: bool = False" in E.dispatch.__doc__
+    c = _arg_names(E.combine)
+    assert len(c) == 19 and c[-1] == "dst_buffer_slot_idx" and c[17] == "use_expanded_layout"
+    assert re.search(r"dst_buffer_slot_idx: .* = None", E.combine.__doc__)
+    i = _arg_names(B.intranode_dispatch)
+    assert len(i) == 17 and i[-1] == "cached_send_head" and i[15] == "allocate_on_comm_stream"
+    assert re.search(r"cached_send_head: .* = None", B.intranode_dispatch.__doc__)
+    assert B.intranode_combine.__doc__.split(" -> ")[0].count("arg") == 12
+    assert B.low_latency_dispatch.__doc__.split(" -> ")[0].count("arg") == 11
+    l = _arg_names(B.low_latency_combine)
+    assert len(l) == 13 and l[-1] == "out" and re.search(r"out: .* = None", B.low_latency_combine.__doc__)
+    assert B.__init__.__doc__.split(" -> ")[0].count("arg") == 8
+    assert E.__init__.__doc__.split(" -> ")[0].count("arg") == 14
+    assert B.get_dispatch_layout.__doc__.split(" -> ")[0].count("arg") == 5
+    assert B.get_next_low_latency_combine_buffer.__doc__.split(" -> ")[0].count("arg") == 3
+    cfg = _C.Config()
+    assert (cfg.num_sms, _C.Config(24, 6, 256, 6, 128).num_sms) == (20, 24)
+    with pytest.raises(RuntimeError):
+        _C.Config(20, 256, 6, 6, 128)          # send chunk not below receive chunk (csrc/legacy/config.hpp:42-44)
+    # size hints: what the reference would reserve, closed forms of csrc/legacy/config.hpp:53-100,131-188
+    assert cfg.get_rdma_buffer_size_hint(7168 * 2, 8) == 0
+    per_slot = 7168 * 2 + 8 + 128 * 8 + 128 * 4 + 128 * 4
+    assert cfg.get_nvl_buffer_size_hint(7168 * 2, 8) == (10 * 8 * 5 * 4 + 10 * 8 * 256 * per_slot + 127) // 128 * 128
+    msg, cmsg = 16 + 7168 * 2, 56 * 4 + 7168 * 2
+    assert _C.get_low_latency_rdma_size_hint(128, 7168, 8, 256) == \
+        (2 * (max(128 * msg, 256 * 128 * cmsg) + 256 * 128 * max(msg, cmsg) + 256 * 4) + 127) // 128 * 128
+    assert deep_ep.Buffer.get_low_latency_rdma_size_hint(128, 7168, 8, 256) == _C.get_low_latency_rdma_size_hint(128, 7168, 8, 256)
 
 
 def test_handle_fields():
@@ -361,12 +413,12 @@ def test_handle_fields():
 def test_buffer_size_calculus_worked_numbers():
     # T=8192 per rank, H=7168, K=8, R=8 (Appendix A of the reference's calculus): BF16 904 MiB, FP8 max(512, 900) MiB
     mib = 1 << 20
-    for rt in (_C, _runtime):
-        assert rt.calculate_elastic_buffer_size(8, 8192, 7168, 8, False, True, True) == 904 * mib
-        assert rt.calculate_elastic_buffer_size(8, 8192, 7168, 8, True, True, True) == 900 * mib
-        assert rt.calculate_elastic_buffer_size(8, 128, 1024, 0, False, True, True) % rt.get_elastic_buffer_alignment() == 0
-        with pytest.raises(RuntimeError):
-            rt.calculate_elastic_buffer_size(8, 0, 7168, 8, False, True, True)
+    rt = _C
+    assert rt.calculate_elastic_buffer_size(8, 8192, 7168, 8, False, True, True) == 904 * mib
+    assert rt.calculate_elastic_buffer_size(8, 8192, 7168, 8, True, True, True) == 900 * mib
+    assert rt.calculate_elastic_buffer_size(8, 128, 1024, 0, False, True, True) % rt.get_elastic_buffer_alignment() == 0
+    with pytest.raises(RuntimeError):
+        rt.calculate_elastic_buffer_size(8, 0, 7168, 8, False, True, True)
     g = deep_ep.LogicalGroup(3, 8)
     assert (g.rank(), g.size()) == (3, 8)
     assert deep_ep.ElasticBuffer.get_buffer_size_hint(g, 8192, 7168, 8) == 904 * mib

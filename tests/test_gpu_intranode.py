@@ -117,7 +117,7 @@ def test_dispatch_and_combine(name, with_topk, fp8):
             assert_equal(out_w, ref_w, "combined_topk_weights")
         else:
             assert out_w is None
-    buf.runtime._read_and_clear_status("intranode")
+    buf.runtime.check_device_status("intranode")
 
 
 def test_reference_round_trip_property_at_headline_shape():
@@ -137,7 +137,7 @@ def test_reference_round_trip_property_at_headline_shape():
     # n identical bf16 values summed in fp32 and rounded once
     assert torch.equal(out.float(), (x_d.float() * n).to(torch.bfloat16).float())
     assert torch.equal(out_w, w_d)
-    buf.runtime._read_and_clear_status("intranode")
+    buf.runtime.check_device_status("intranode")
 
 
 def test_argument_errors():
@@ -174,7 +174,7 @@ def test_empty_inputs():
         assert int(handle[0].abs().sum()) == 0 and handle[5].shape == (T, R) and bool((handle[5] == -1).all())
         out, out_w, _ = buf.combine(recv_x, handle, topk_weights=recv_w)
         assert out.shape == (T, H) and bool((out == 0).all()) and bool((out_w == 0).all())
-    buf.runtime._read_and_clear_status("intranode")
+    buf.runtime.check_device_status("intranode")
 
 
 def test_per_source_calls_compose_into_the_world():

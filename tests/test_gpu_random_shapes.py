@@ -215,4 +215,4 @@ def test_random_v1_configuration(seed):
     assert_equal(out + 0.0, ref_out + 0.0, "combined_x")
     if with_topk:
         assert_equal(out_w, ref_w, "combined_topk_weights")
-    buf.runtime._read_and_clear_status("intranode")
+    buf.runtime.check_device_status("intranode")

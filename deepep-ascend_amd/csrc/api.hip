@@ -178,10 +178,6 @@ void* g_scratch_ptr[kMaxDevices];          // address of `scratch` on each devic
 bool g_scratch_ready[kMaxDevices];
 std::mutex g_scratch_mutex;
 
-__global__ void clear_words_kernel(uint32_t* words, size_t n) {
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) words[i] = 0u;
-}
-
 // The status word as memory has it (past every cache between the kernels that OR into it and this read), stored so
 // that a host polling pinned memory sees it.  A clearing read swaps the word with zero and, if a single-launch dispatch
 // had given up, zeroes the bookkeeping words that launch left mid-protocol.
@@ -198,9 +194,11 @@ __global__ void read_status_kernel(int32_t* status, int32_t* out, int clear, uin
         for (int i = threadIdx.x; i < control_words; i += blockDim.x) store_agent(reinterpret_cast<int*>(control) + i, 0);
 }
 
-// Device address of `scratch` on the current device.  First use on a device resolves the address and clears the
-// bookkeeping words with a small kernel on `stream` (no memset: the call may be under graph capture).
-int static_workspace(hipStream_t stream, void** out) {
+// Device address of `scratch` on the current device, resolved on first use.  The array needs no clearing: a `__device__`
+// array without an initialiser reads zero when its code object is loaded, which is the state a fresh workspace must
+// have, and nothing is launched here (the first call may be under graph capture: a clearing kernel captured with it
+// would run again on every replay).
+int static_workspace(void** out) {
     int dev = -1;
     hipError_t err = hipGetDevice(&dev);
     if (err != hipSuccess) return hip_fail(err, "hipGetDevice");
@@ -210,10 +208,6 @@ int static_workspace(hipStream_t stream, void** out) {
         void* ptr = nullptr;
         err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (err != hipSuccess || ptr == nullptr) return hip_fail(err, "hipGetSymbolAddress(scratch)");
-        const size_t control_words = make_workspace_layout(1, 1, 1, 1).expert_start / 4;
-        hipLaunchKernelGGL(clear_words_kernel, dim3(16), dim3(256), 0, stream, static_cast<uint32_t*>(ptr), control_words);
-        err = hipGetLastError();
-        if (err != hipSuccess) return hip_fail(err, "clearing the static workspace");
         g_scratch_ptr[dev] = ptr;
         g_scratch_ready[dev] = true;
     }
@@ -402,7 +396,7 @@ int deep_ep_hip_read_status(void* workspace, int32_t* status_out, int clear, voi
     REQUIRE(status_out != nullptr, "status_out is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (workspace == nullptr)
-        if (int rc = static_workspace(s, &workspace)) return rc;
+        if (int rc = static_workspace(&workspace)) return rc;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const WorkspaceLayout w = make_workspace_layout(1, 1, 1, 1);
     hipLaunchKernelGGL(read_status_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<int32_t*>(ws + w.status), status_out,
@@ -474,7 +468,7 @@ int deep_ep_hip_launch_dispatch_static(const deep_ep_hip_dispatch_args* a, void*
                     "this shape needs %zu bytes of workspace, the built-in one has %zu: pass a workspace of your own to "
                     "deep_ep_hip_launch_dispatch", need, kStaticWorkspaceBytes);
     void* ws = nullptr;
-    if (int rc = static_workspace(stream, &ws)) return rc;
+    if (int rc = static_workspace(&ws)) return rc;
     return dispatch_with_workspace(a, ws, kStaticWorkspaceBytes, stream);
 }
 

@@ -334,6 +334,19 @@ __device__ __forceinline__ void await_and_clear_flags(const MoveParams& p, int32
     __syncthreads();
 }
 
+__device__ __forceinline__ void finish_hand_off(const MoveParams& p, bool done, uint32_t tag);
+
+// The publisher of an expanded dispatch has read the launch's tag and stored its tagged words (the expert bases): once
+// every thread's stores are acknowledged it reports as a party of the hand-off.  Without this a publisher that starts
+// late could read the generation after the movers - which wait only for the bases they need, none if no lane is valid -
+// have advanced it, and stamp its words with the next launch's tag; and the clearing of the tables at the end of a tag
+// period could overtake stores of words no mover waits for.  All threads call it.
+__device__ __forceinline__ void publisher_is_done_with_the_tag(const MoveParams& p, uint32_t tag) {
+    wait_for_own_stores();
+    __syncthreads();
+    if (threadIdx.x < kWaveSize) finish_hand_off(p, true, tag);
+}
+
 __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     extern __shared__ uint64_t count_lds[];
     const PublishLds lds = carve_publish_lds(reinterpret_cast<int*>(count_lds), p.R, p.E);
@@ -348,6 +361,7 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
         const bool complete = write_expert_bases_from_registers<kThreads>(tab, p.tagged_expert_counts, tagged_bases, tag, kLayoutSpinLimit,
                                                                           p.R, p.E, p.pub.A, p.count_blocks, lds);
         if (!complete && threadIdx.x == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+        publisher_is_done_with_the_tag(p, tag);
     }
 
     // Everything else waits until the counting workgroups have flagged that their stores are acknowledged.  The expert
@@ -359,6 +373,7 @@ __device__ __forceinline__ void fused_publish_block(const MoveParams& p) {
     if (p.do_expand && !bases_first) {
         __syncthreads();
         write_expert_bases<kThreads, true>(tab, tagged_bases, tag, p.E, p.count_blocks, lds);
+        publisher_is_done_with_the_tag(p, tag);
     }
     __syncthreads();
     scan_rank_counts<kThreads>(p.pub, tab, p.R, lds);
@@ -448,21 +463,25 @@ __device__ __forceinline__ unsigned advance_gate(const MoveParams& p, unsigned m
     return atomicInc(p.gates + gate * kDispatchGateStride, movers_of_gate(p, gate) - 1u);
 }
 
-// First wavefront of a mover workgroup (all its lanes), right before its payload stores - not after them: a wait for the
-// atomic's answer behind the stores would be a wait for their acknowledgements too, with the wavefront and its workgroup's
-// resources held that long (8192 x 7168 FP8, side by side on one GPU: 86.0 -> 85.7 us).  `seen` counts on its first lane.  The mover
-// that was the last of its gate reports the gate; the one that reports the last gate advances the generation: by then
-// every mover has read its tagged words.  The launch that used the last tag clears the tagged tables first, all lanes
-// together (a third of a megabyte: some 15 us once in 16383 launches).
-__device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover, unsigned seen, uint32_t tag) {
+// Parties of a launch's hand-off: the gates in use and, for the expanded layout, the publishing workgroup, which reads
+// the tag and stores tagged words (the expert bases) itself.
+__device__ __forceinline__ unsigned hand_off_parties(const MoveParams& p) {
+    const unsigned gates_in_use = p.num_movers < unsigned(kDispatchGates) ? p.num_movers : unsigned(kDispatchGates);
+    return gates_in_use + (p.do_expand ? 1u : 0u);
+}
+
+// One party of the hand-off is done with this launch's tag (all lanes of one wavefront; `done` is looked at on the first
+// lane): a gate whose movers have all read their tagged words, or the publisher of an expanded dispatch once its tagged
+// stores are acknowledged.  The party that completes the count advances the generation: by then every tagged word of
+// the launch has been read or acknowledged, and nobody will read the generation word for this launch again.  The launch
+// that used the last tag clears the tagged tables first, all lanes together (a third of a megabyte: some 15 us once in
+// 16383 launches).
+__device__ __forceinline__ void finish_hand_off(const MoveParams& p, bool done, uint32_t tag) {
     const int lane = lane_id();
     int last = 0;
-    if (lane == 0) {
-        const unsigned gate = mover % unsigned(kDispatchGates);
-        if (seen == movers_of_gate(p, gate) - 1u) {
-            const unsigned gates_in_use = p.num_movers < unsigned(kDispatchGates) ? p.num_movers : unsigned(kDispatchGates);
-            last = atomicInc(p.gates_finished, gates_in_use - 1u) == gates_in_use - 1u ? 1 : 0;
-        }
+    if (lane == 0 && done) {
+        const unsigned parties = hand_off_parties(p);
+        last = atomicInc(p.gates_finished, parties - 1u) == parties - 1u ? 1 : 0;
     }
     if (__builtin_amdgcn_readfirstlane(last) == 0) return;
     uint32_t next = tag >> kTagShift;                     // generation + 1
@@ -472,6 +491,15 @@ __device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover,
         next = 0;
     }
     if (lane == 0) store_agent(reinterpret_cast<int*>(p.generation), int(next));
+}
+
+// First wavefront of a mover workgroup (all its lanes), right before its payload stores - not after them: a wait for the
+// atomic's answer behind the stores would be a wait for their acknowledgements too, with the wavefront and its workgroup's
+// resources held that long (8192 x 7168 FP8, side by side on one GPU: 86.0 -> 85.7 us).  `seen` counts on its first lane.  The mover
+// that was the last of its gate reports the gate.
+__device__ __forceinline__ void settle_gate(const MoveParams& p, unsigned mover, unsigned seen, uint32_t tag) {
+    const unsigned gate = mover % unsigned(kDispatchGates);
+    finish_hand_off(p, seen == movers_of_gate(p, gate) - 1u, tag);
 }
 
 // A wavefront's wait (bounded) for the tagged words its threads want.  Returns whether this thread still misses one.
@@ -891,13 +919,9 @@ __global__ __launch_bounds__(kThreads) void cast_kernel(const CastParams p) {
     const int elem = tile * 1024 + lane * 16;
     const uint16_t* src = reinterpret_cast<const uint16_t*>(p.x) + int64_t(t) * p.H;
     float f[16];
-    float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        f[i] = (elem + i < p.H) ? __uint_as_float(uint32_t(src[elem + i]) << 16) : 0.f;
-        amax = fmaxf(amax, fabsf(f[i]));
-    }
-    amax = fmaxf(group8_max(amax), 1e-4f);
+    for (int i = 0; i < 16; ++i) f[i] = (elem + i < p.H) ? __uint_as_float(uint32_t(src[elem + i]) << 16) : 0.f;
+    const float amax = group_amax<true>(f);       // a NaN in the group reaches its scale, as in the torch recipe
     const float scale = 448.0f / amax;
     const float scale_inv = amax / 448.0f;
     uint8_t* dst = p.out + int64_t(t) * p.H;

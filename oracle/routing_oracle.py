@@ -113,15 +113,25 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q.view(T, Hp)[:, :H].contiguous(), scales.view(T, Hp // 128)
 
 
+def _amax_dropping_nan(g: torch.Tensor) -> torch.Tensor:
+    """max(|x|) over the last dimension the way the reference's low-latency kernel takes it: a running fmaxf that
+    starts at the 1e-4 floor (csrc/kernels/legacy/internode_ll.cu:223-231).  C's fmaxf returns the other operand when
+    one is NaN, so NaN elements do not take part; an infinity does."""
+    mag = g.abs()
+    mag = torch.where(torch.isnan(mag), torch.zeros_like(mag), mag)
+    return mag.amax(dim=-1).clamp(min=1e-4)
+
+
 def per_token_cast_to_fp8_ll(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """What the reference's low-latency kernel emits without `round_scale` (csrc/kernels/legacy/utils.cuh:477-479,
     499-501; internode_ll.cu:223-243): amax clamped below at 1e-4, payload = e4m3fn(x * (448 / amax)) as in
     per_token_cast_to_fp8, but the stored scale is the fp32 product amax * fp32(1 / 448), not the quotient amax / 448
-    (the two differ in the last bit for many amax values)."""
+    (the two differ in the last bit for many amax values).  The maximum is taken with fmaxf: a NaN element encodes as
+    NaN but leaves its group's scale alone (the torch recipe above lets it spread over the group)."""
     assert x.dim() == 2 and x.shape[1] % 128 == 0
     T, H = x.shape
     g = x.to(torch.float32).view(T, H // 128, 128)
-    amax = g.abs().amax(dim=2).clamp(min=1e-4)
+    amax = _amax_dropping_nan(g)
     q = (g * (torch.tensor(448.0, dtype=torch.float32) / amax).unsqueeze(2)).to(torch.float8_e4m3fn)
     scales = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
     return q.view(T, H).contiguous(), scales
@@ -136,7 +146,7 @@ def per_token_cast_to_fp8_pow2(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Ten
     T, H = x.shape
     assert H % 128 == 0
     g = x.to(torch.float32).view(T, H // 128, 128)
-    amax = g.abs().amax(dim=2).clamp(min=1e-4)
+    amax = _amax_dropping_nan(g)
     ratio = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
     mantissa, exponent = torch.frexp(ratio)                         # ratio = mantissa * 2^exponent, 0.5 <= mantissa < 1
     exponent = torch.where(mantissa == 0.5, exponent - 1, exponent)  # ceil(log2(ratio))

@@ -211,3 +211,52 @@ def test_low_latency_scale_is_the_fp32_product_with_the_reciprocal():
     # the low-latency dispatch uses this rule, and only for the scales
     px, ps, _, _, _ = oracle.ll_dispatch([x[:8]], [torch.zeros((8, 1), dtype=torch.int64)], 8, 1, 1, 0)
     assert torch.equal(ps[0, :8], s[:8]) and torch.equal(px[0, :8].view(torch.uint8), q[:8].view(torch.uint8))
+
+
+def _nonfinite_groups():
+    """Four 128-channel groups: one with a NaN, one with +Inf, one with -Inf, one finite; ordinary values elsewhere."""
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn((1, 512), generator=g) * 2).to(torch.bfloat16)
+    x[0, 5], x[0, 128 + 7], x[0, 256 + 9] = float("nan"), float("inf"), float("-inf")
+    return x
+
+
+def test_non_finite_inputs_of_the_torch_recipe():
+    """deep_ep/utils/math.py:37-38 takes the maximum with torch's amax and clamp, which hand a NaN on (a NaN compares
+    false with everything, so a maximum built from comparisons would drop it - the C restatement above does, and is
+    therefore only used on finite inputs).  What follows is plain IEEE arithmetic: 448 / NaN = NaN, x * NaN = NaN;
+    448 / Inf = 0, finite * 0 = +-0, Inf * 0 = NaN, Inf / 448 = Inf."""
+    x = _nonfinite_groups()
+    q, s = oracle.per_token_cast_to_fp8(x)
+    qb = q.view(torch.uint8).view(4, 128)
+    nan_code = (qb & 0x7f) == 0x7f
+    assert torch.isnan(s[0, 0]) and nan_code[0].all()                         # the NaN spreads over its group
+    for grp, pos in ((1, 7), (2, 9)):
+        assert torch.isinf(s[0, grp]) and s[0, grp] > 0
+        assert nan_code[grp, pos] and int(nan_code[grp].sum()) == 1           # only the infinity itself is NaN
+        others = torch.cat([qb[grp, :pos], qb[grp, pos + 1:]])
+        signs = torch.cat([x[0, grp * 128:grp * 128 + pos], x[0, grp * 128 + pos + 1:(grp + 1) * 128]]).float() < 0
+        assert torch.equal(others, torch.where(signs, 0x80, 0).to(torch.uint8))      # signed zeros
+    assert torch.isfinite(s[0, 3]) and not nan_code[3].any()
+
+
+def test_non_finite_inputs_of_the_low_latency_recipe():
+    """csrc/kernels/legacy/internode_ll.cu:223-231 takes the maximum with fmaxf, which returns the other operand when
+    one is NaN (C99 7.12.12.2; numpy's fmax is that function): a NaN element leaves its group's scale alone and only
+    encodes as NaN itself.  Infinities behave as in the torch recipe."""
+    x = _nonfinite_groups()
+    for cast in (oracle.per_token_cast_to_fp8_ll, oracle.per_token_cast_to_fp8_pow2):
+        q, s = cast(x[:, :128])                                               # the group with the NaN
+        qb = q.view(torch.uint8)[0]
+        amax = np.fmax.reduce(np.abs(x[0, :128].float().numpy()))
+        assert np.isfinite(amax) and amax >= 1e-4
+        if cast is oracle.per_token_cast_to_fp8_ll:
+            assert float(s[0, 0]) == float(np.float32(amax) * np.float32(1.0 / 448.0))
+            finite_ref, _ = oracle.per_token_cast_to_fp8(torch.where(torch.isnan(x[:, :128]), torch.zeros_like(x[:, :128]), x[:, :128]))
+            mask = torch.ones(128, dtype=torch.bool); mask[5] = False
+            assert torch.equal(qb[mask], finite_ref.view(torch.uint8)[0][mask])      # the others as if the NaN were not there
+        else:
+            assert float(s[0, 0]) == 2.0 ** int(np.ceil(np.log2(float(np.float32(amax) * np.float32(1.0 / 448.0)))))
+        assert (int(qb[5]) & 0x7f) == 0x7f and int(((qb & 0x7f) == 0x7f).sum()) == 1
+    q, s = oracle.per_token_cast_to_fp8_ll(x[:, 128:384])                     # the groups with the infinities
+    assert torch.isinf(s).all() and int(((q.view(torch.uint8) & 0x7f) == 0x7f).sum()) == 2

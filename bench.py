@@ -9,8 +9,13 @@ case so no host synchronisation sits inside a step.  Calls go straight through t
 
 Prints one JSON line: whole-step achieved HBM GB/s (algorithmic bytes / time), per-op us/call,
 a roofline object for the dominant kernel (combine), one for the dispatch call, and a CPU baseline (the
-torch-CPU oracle timed on the same workload, all tokens, a few passes).  --workload C5 prints the same for the
-low-latency pair of kernels.
+torch-CPU oracle timed on the same workload, all tokens, a few passes).  The default run adds two blocks that take a
+few seconds more: `other_workloads` (C4, the expanded layout and the BF16 payload at the headline shape, C2 and the
+low-latency C5: us per dispatch / combine, algorithmic bytes, fraction of peak) and `us_per_api_call` (what a caller of
+`deep_ep.ElasticBuffer.dispatch` / `.combine` and of `deep_ep.Buffer.low_latency_dispatch` / `low_latency_combine` pays
+per call through the Python wrapper and the compiled extension, outputs allocated inside the call, by the host clock;
+the low-latency step also as a replayed HIP graph).  --brief leaves them out; --workload C5 prints the headline objects
+for the low-latency pair of kernels; --overlap times dispatch and combine under a GPU-filling compute stream.
 """
 import argparse
 import ctypes
@@ -63,6 +68,274 @@ def algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=True, expanded=False):
     return {"layout": layout, "dispatch": dispatch, "combine": combine}
 
 
+class RoutingCalls:
+    """Buffers (worst-case sized, allocated once) and argument blocks of a dispatch + combine pair on one workload,
+    launched straight through the C ABI."""
+
+    def __init__(self, torch, _abi, dev, case, fp8, expanded, launches=0):
+        self.torch, self._abi = torch, _abi
+        T, H, K, E, R, M = case.T, case.H, case.K, case.E, case.R, case.M
+        self.T, self.H, self.K, self.E, self.R, self.M = T, H, K, E, R, M
+        self.x, idx, w = case.x.to(dev), case.topk_idx.to(dev), case.topk_weights.to(dev)
+        x = self.x
+        # realised routing statistics (for the algorithmic bytes)
+        valid = case.topk_idx >= 0
+        self.N_e = N_e = int(valid.sum())
+        dst = torch.where(valid, case.topk_idx // (E // R), torch.full_like(case.topk_idx, -1))
+        self.N_r = N_r = int(sum(int((dst == r).any(dim=1).sum()) for r in range(R)))
+        self.ab = algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=fp8, expanded=expanded)
+
+        i32 = dict(dtype=torch.int32, device=dev)
+        cap = M * R
+        ecap = M * min(K, E)
+        rows = ecap if expanded else cap
+        ws_bytes = _abi.lib.deep_ep_hip_workspace_bytes(T, K, E, R)
+        self.workspace = workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+        psum_rank, psum_expert, unaligned = torch.empty(R, **i32), torch.empty(E, **i32), torch.empty(E, **i32)
+        slot = torch.empty((T, K), **i32)
+        meta = torch.empty((cap, K + 2), **i32)
+        recv_x = torch.empty((rows, H), dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16, device=dev)
+        recv_sf = torch.empty((rows, H // 128), dtype=torch.float32, device=dev) if fp8 else None
+        recv_idx = torch.empty((cap, K), dtype=torch.int64, device=dev) if not expanded else None
+        recv_w = torch.empty((rows,) if expanded else (cap, K), dtype=torch.float32, device=dev)
+        y = torch.randn((rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)   # "expert outputs"
+        out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+        out_w = torch.empty((T, K), dtype=torch.float32, device=dev)
+        self.keep = (idx, w, psum_rank, psum_expert, unaligned, slot, meta, recv_x, recv_sf, recv_idx, recv_w, y, out, out_w)
+
+        d = self.d = _abi.DispatchArgs()
+        d.payload = _abi.PAYLOAD_CAST_FP8 if fp8 else _abi.PAYLOAD_BF16
+        d.do_expand = int(expanded)
+        d.num_tokens, d.hidden, d.num_topk, d.num_experts, d.num_ranks = T, H, K, E, R
+        d.rank_idx, d.num_max_tokens_per_rank, d.expert_alignment = 0, M, 1
+        d.x, d.topk_idx, d.topk_weights = x.data_ptr(), idx.data_ptr(), w.data_ptr()
+        d.num_sf_packs = H // 128 if fp8 else 0
+        d.psum_num_recv_tokens_per_rank = psum_rank.data_ptr()
+        d.psum_num_recv_tokens_per_expert = psum_expert.data_ptr()
+        d.num_unaligned_recv_tokens_per_expert = unaligned.data_ptr()
+        d.dst_buffer_slot_idx, d.recv_src_metadata = slot.data_ptr(), meta.data_ptr()
+        d.recv_x = recv_x.data_ptr()
+        d.recv_sf = recv_sf.data_ptr() if fp8 else 0
+        d.recv_sf_token_stride, d.recv_sf_hidden_stride = (H // 128, 1) if fp8 else (0, 0)
+        d.recv_topk_idx = recv_idx.data_ptr() if recv_idx is not None else 0
+        d.recv_topk_weights = recv_w.data_ptr()
+        d.recv_capacity, d.expanded_capacity = cap, (ecap if expanded else 0)
+        d.workspace, d.workspace_bytes = workspace.data_ptr(), ws_bytes
+        d.tuning = _abi.Tuning.from_env()
+        d.tuning.dispatch_launches = launches
+
+        c = self.c = _abi.CombineArgs()
+        c.tuning = _abi.Tuning.from_env()
+        c.do_expand, c.allow_multiple_reduction = int(expanded), 1
+        c.num_tokens, c.hidden, c.num_topk, c.num_experts, c.num_ranks = T, H, K, E, R
+        c.rank_idx, c.num_max_tokens_per_rank = 0, M
+        c.x, c.num_x_rows = y.data_ptr(), rows
+        c.topk_weights = recv_w.data_ptr()
+        c.topk_idx, c.dst_buffer_slot_idx = idx.data_ptr(), slot.data_ptr()
+        c.recv_src_metadata, c.num_recv_rows = meta.data_ptr(), cap
+        c.psum_num_recv_tokens_per_rank = psum_rank.data_ptr()
+        c.combined_x, c.combined_topk_weights = out.data_ptr(), out_w.data_ptr()
+        c.workspace, c.workspace_bytes = workspace.data_ptr(), ws_bytes
+
+        self.stream = torch.cuda.current_stream()
+        self.sp = self.stream.cuda_stream
+
+    def on_stream(self, stream):
+        """Launch on `stream` from now on (it must be ordered behind everything launched so far)."""
+        self.stream, self.sp = stream, stream.cuda_stream
+
+    def dispatch(self, phases=None):
+        self.d.phases = (self._abi.PHASE_LAYOUT | self._abi.PHASE_MOVE) if phases is None else phases
+        self._abi.check(self._abi.lib.deep_ep_hip_launch_dispatch(ctypes.byref(self.d), self.sp), "dispatch")
+
+    def combine(self):
+        self._abi.check(self._abi.lib.deep_ep_hip_launch_combine(ctypes.byref(self.c), self.sp), "combine")
+
+    def step(self):
+        self.dispatch()
+        self.combine()
+
+    def launches(self):
+        self.d.phases = self._abi.PHASE_LAYOUT | self._abi.PHASE_MOVE
+        return self._abi.lib.deep_ep_hip_dispatch_kernel_launches(ctypes.byref(self.d))
+
+    def status(self):
+        return int(self.workspace[:4].view(self.torch.int32).item())
+
+    def loop_us(self, fn, iters):
+        """Average duration in us of fn over iters back-to-back launches, by HIP events on the launch stream."""
+        torch = self.torch
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(self.stream)
+        for _ in range(iters):
+            fn()
+        e1.record(self.stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def _quantiles(samples):
+    samples = sorted(samples)
+    pick = lambda q: samples[min(len(samples) - 1, int(q * len(samples)))]
+    return {"min": round(samples[0], 2), "p50": round(pick(0.5), 2), "p95": round(pick(0.95), 2)}
+
+
+def host_timed(torch, fn, calls=60, warm=5):
+    """What a caller pays per call, by the host clock.  `waited`: each call between two device synchronisations (host
+    work of the call + launch + kernels + the wait for the result); `issue`: the same calls back to back, the time until
+    the call returns to the caller (device work only shows if the queue fills up)."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    waited, issue = [], []
+    for _ in range(calls):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        waited.append((t2 - t0) * 1e6)
+        issue.append((t1 - t0) * 1e6)
+    return {"waited_us": _quantiles(waited), "issue_us": _quantiles(issue)}
+
+
+def routing_api_figures(torch, dev, case, kernel_us):
+    """us per call of `deep_ep.ElasticBuffer.dispatch` / `.combine` (Python wrapper -> compiled extension -> C ABI, outputs
+    allocated inside the call) at the headline shape, against the kernel time of the same operation."""
+    import deep_ep
+    T, H, K, E, R, M = case.T, case.H, case.K, case.E, case.R, case.M
+    x, idx, w = case.x.to(dev), case.topk_idx.to(dev), case.topk_weights.to(dev)
+    buf = deep_ep.ElasticBuffer(deep_ep.LogicalGroup(0, R), num_max_tokens_per_rank=M, hidden=H, num_topk=K)
+    out = {"binding": deep_ep._binding.name, "calls": 60}
+    no_sync = lambda: buf.dispatch(x, idx, w, num_experts=E, do_cpu_sync=False, cast_to_fp8=True)
+    out["dispatch_no_cpu_sync"] = host_timed(torch, no_sync)
+    out["dispatch_cpu_sync"] = host_timed(torch, lambda: buf.dispatch(x, idx, w, num_experts=E, cast_to_fp8=True))
+    (recv_x, recv_sf), recv_idx, recv_w, handle, _ = no_sync()
+    y = torch.randn((recv_x.shape[0], H), dtype=torch.float32, device=dev).to(torch.bfloat16)
+    out["combine"] = host_timed(torch, lambda: buf.combine(y, handle, topk_weights=recv_w))
+    buf.check_device_status()
+    d_us, c_us = kernel_us
+    out["kernel_us"] = {"dispatch": round(d_us, 2), "combine": round(c_us, 2)}
+    out["host_overhead_us"] = {"dispatch_no_cpu_sync": round(out["dispatch_no_cpu_sync"]["waited_us"]["p50"] - d_us, 2),
+                               "dispatch_cpu_sync": round(out["dispatch_cpu_sync"]["waited_us"]["p50"] - d_us, 2),
+                               "combine": round(out["combine"]["waited_us"]["p50"] - c_us, 2)}
+    return out
+
+
+def low_latency_api_figures(torch, ll, kernel_us):
+    """us per call of `deep_ep.Buffer.low_latency_dispatch` / `low_latency_combine` at the C5 shape, eager and as a
+    replayed HIP graph of one dispatch + combine step, against the kernel time."""
+    import deep_ep
+    x, idx, w = ll.inputs
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(0, ll.R), low_latency_mode=True)
+    out = {"binding": deep_ep._binding.name, "calls": 60}
+    dispatch = lambda: buf.low_latency_dispatch(x, idx, ll.M, ll.E, use_fp8=True)
+    out["low_latency_dispatch"] = host_timed(torch, dispatch)
+    recv, count, handle, _, _ = dispatch()
+    combine = lambda: buf.low_latency_combine(ll.y, idx, w, handle)
+    out["low_latency_combine"] = host_timed(torch, combine)
+
+    def step():
+        recv, count, handle, _, _ = dispatch()
+        return buf.low_latency_combine(ll.y, idx, w, handle)
+
+    out["step_eager"] = host_timed(torch, step)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()                                   # the buffer's workspaces exist and were last used on this stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            captured = step()
+    torch.cuda.current_stream().wait_stream(side)
+    out["step_graph_replay"] = host_timed(torch, graph.replay)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream()
+    e0.record(stream)
+    for _ in range(30):
+        graph.replay()
+    e1.record(stream)
+    e1.synchronize()
+    out["step_graph_replay"]["device_us_back_to_back"] = round(e0.elapsed_time(e1) * 1e3 / 30, 2)
+    d_us, c_us = kernel_us
+    out["kernel_us"] = {"low_latency_dispatch": round(d_us, 2), "low_latency_combine": round(c_us, 2), "step": round(d_us + c_us, 2)}
+    out["host_overhead_us"] = {"low_latency_dispatch": round(out["low_latency_dispatch"]["waited_us"]["p50"] - d_us, 2),
+                               "low_latency_combine": round(out["low_latency_combine"]["waited_us"]["p50"] - c_us, 2),
+                               "step_eager": round(out["step_eager"]["waited_us"]["p50"] - d_us - c_us, 2),
+                               "step_graph_replay": round(out["step_graph_replay"]["waited_us"]["p50"] - d_us - c_us, 2)}
+    del captured
+    return out
+
+
+def other_workloads(torch, rc, _abi, dev, c3_case, iters=12):
+    """The other benchmark configurations in brief: us per dispatch / combine in a hot loop (HIP events on the launch
+    stream, straight through the C ABI), their algorithmic bytes and the fraction of the 8 TB/s peak."""
+    out = {}
+    specs = (("C4", rc.c4, True, False), ("C3_expanded", lambda: c3_case, True, True), ("C3_bf16", lambda: c3_case, False, False),
+             ("C2", rc.c2, False, False))
+    for name, make, fp8, expanded in specs:
+        case = make()
+        rt = RoutingCalls(torch, _abi, dev, case, fp8, expanded)
+        for _ in range(3):
+            rt.step()
+        torch.cuda.synchronize()
+        d_us, c_us = rt.loop_us(rt.dispatch, iters), rt.loop_us(rt.combine, iters)
+        d_bytes, c_bytes = rt.ab["layout"] + rt.ab["dispatch"], rt.ab["combine"]
+        out[name] = {"workload": f"{case.name}: T={rt.T} H={rt.H} E={rt.E} R={rt.R} K={rt.K}, "
+                                 f"{'FP8 (fused cast)' if fp8 else 'BF16'} dispatch, {'expanded' if expanded else 'compact'} layout, "
+                                 f"N_r={rt.N_r}, N_e={rt.N_e}",
+                     "dispatch_us": round(d_us, 2), "combine_us": round(c_us, 2), "dispatch_kernel_launches": rt.launches(),
+                     "dispatch_bytes": d_bytes, "combine_bytes": c_bytes,
+                     "dispatch_frac": round(d_bytes / d_us * 1e-3 / HBM_PEAK_GBS, 4),
+                     "combine_frac": round(c_bytes / c_us * 1e-3 / HBM_PEAK_GBS, 4), "device_status": rt.status()}
+        del rt
+        torch.cuda.empty_cache()
+    ll = LowLatencyCalls(torch, rc, _abi, dev)
+    for _ in range(5):
+        ll.step()
+    torch.cuda.synchronize()
+    d_us, c_us = ll.loop_us(ll.dispatch, 30), ll.loop_us(ll.combine, 30)
+    out["C5"] = {"workload": f"C5 low latency: R={ll.R} T={ll.T} H={ll.H} E={ll.E} K={ll.K} M={ll.M}, rows on rank 0: {ll.n_e}",
+                 "dispatch_us": round(d_us, 2), "combine_us": round(c_us, 2), "dispatch_bytes": ll.dispatch_bytes,
+                 "combine_bytes": ll.combine_bytes, "dispatch_frac": round(ll.dispatch_bytes / d_us * 1e-3 / HBM_PEAK_GBS, 4),
+                 "combine_frac": round(ll.combine_bytes / c_us * 1e-3 / HBM_PEAK_GBS, 4)}
+    api = low_latency_api_figures(torch, ll, kernel_us=(d_us, c_us))
+    del ll
+    torch.cuda.empty_cache()
+    return out, api
+
+
+def under_compute_load(torch, dev, rt, iters=20):
+    """us per dispatch / combine on a communication stream of their own while a chain of 8192^3 BF16 matrix products
+    keeps the GPU busy on another stream (what overlapping the routing with a neighbouring micro-batch's GEMMs looks
+    like), and the same without the load."""
+    comm, load = torch.cuda.Stream(), torch.cuda.Stream()
+    a = torch.randn((8192, 8192), device=dev, dtype=torch.bfloat16)
+    c = torch.empty_like(a)
+    torch.cuda.synchronize()
+    rt.on_stream(comm)
+    out = {}
+    for name, fn in (("dispatch", rt.dispatch), ("combine", rt.combine)):
+        fn()
+        torch.cuda.synchronize()
+        quiet = rt.loop_us(fn, iters)
+        done = torch.cuda.Event()
+        with torch.cuda.stream(load):
+            for _ in range(40):
+                torch.mm(a, a, out=c)
+            done.record(load)
+        time.sleep(0.002)                                  # the products are running
+        busy = rt.loop_us(fn, iters)
+        out[name] = {"alone_us": round(quiet, 2), "under_load_us": round(busy, 2), "load_outlasted_the_measurement": not done.query()}
+        torch.cuda.synchronize()
+    out["device_status"] = rt.status()
+    rt.on_stream(torch.cuda.current_stream())
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +357,9 @@ def main():
     ap.add_argument("--fresh-input", action="store_true",
                     help="per-kernel timings: rewrite x with a copy kernel right before every (untimed) call, as a producer would")
     ap.add_argument("--l2-flush", action="store_true", help="zero a 256 MB buffer between per-kernel timings")
+    ap.add_argument("--overlap", action="store_true",
+                    help="also time dispatch and combine on a stream of their own while matrix products fill the GPU on another")
+    ap.add_argument("--brief", action="store_true", help="only the headline workload: no other workloads, no API-level figures")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (logical ranks share its HBM); use --gpus 1", file=sys.stderr)
@@ -103,88 +379,16 @@ def main():
         print(json.dumps(bench_low_latency(args, torch, rc, _abi, dev)))
         return
     case = {"C2": rc.c2, "C3": rc.c3, "C4": rc.c4}[args.workload]()
-    T, H, K, E, R, M = case.T, case.H, case.K, case.E, case.R, case.M
     if args.routing == "sequential":
-        E_l = E // R
-        base = torch.tensor([0, E_l, 2 * E_l, 3 * E_l, 4 * E_l, 1, E_l + 1, 2 * E_l + 1][:K], dtype=torch.int64)
-        case.topk_idx = base.unsqueeze(0).repeat(T, 1).contiguous()
+        E_l = case.E // case.R
+        base = torch.tensor([0, E_l, 2 * E_l, 3 * E_l, 4 * E_l, 1, E_l + 1, 2 * E_l + 1][:case.K], dtype=torch.int64)
+        case.topk_idx = base.unsqueeze(0).repeat(case.T, 1).contiguous()
     fp8 = not args.bf16
     expanded = args.expanded
-    x, idx, w = case.x.to(dev), case.topk_idx.to(dev), case.topk_weights.to(dev)
-
-    # realised routing statistics (for the algorithmic bytes)
-    valid = case.topk_idx >= 0
-    N_e = int(valid.sum())
-    dst = torch.where(valid, case.topk_idx // (E // R), torch.full_like(case.topk_idx, -1))
-    N_r = int(sum(int((dst == r).any(dim=1).sum()) for r in range(R)))
-    ab = algorithmic_bytes(T, H, K, E, R, N_r, N_e, fp8=fp8, expanded=expanded)
-
-    # ---- buffers (worst-case sized, allocated once) ----
-    i32 = dict(dtype=torch.int32, device=dev)
-    cap = M * R
-    ecap = M * min(K, E)
-    rows = ecap if expanded else cap
-    ws_bytes = _abi.lib.deep_ep_hip_workspace_bytes(T, K, E, R)
-    workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-    psum_rank, psum_expert, unaligned = torch.empty(R, **i32), torch.empty(E, **i32), torch.empty(E, **i32)
-    slot = torch.empty((T, K), **i32)
-    meta = torch.empty((cap, K + 2), **i32)
-    recv_x = torch.empty((rows, H), dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16, device=dev)
-    recv_sf = torch.empty((rows, H // 128), dtype=torch.float32, device=dev) if fp8 else None
-    recv_idx = torch.empty((cap, K), dtype=torch.int64, device=dev) if not expanded else None
-    recv_w = torch.empty((rows,) if expanded else (cap, K), dtype=torch.float32, device=dev)
-    y = torch.randn((rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)   # "expert outputs"
-    out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
-    out_w = torch.empty((T, K), dtype=torch.float32, device=dev)
-
-    d = _abi.DispatchArgs()
-    d.payload = _abi.PAYLOAD_CAST_FP8 if fp8 else _abi.PAYLOAD_BF16
-    d.do_expand = int(expanded)
-    d.num_tokens, d.hidden, d.num_topk, d.num_experts, d.num_ranks = T, H, K, E, R
-    d.rank_idx, d.num_max_tokens_per_rank, d.expert_alignment = 0, M, 1
-    d.x, d.topk_idx, d.topk_weights = x.data_ptr(), idx.data_ptr(), w.data_ptr()
-    d.num_sf_packs = H // 128 if fp8 else 0
-    d.psum_num_recv_tokens_per_rank = psum_rank.data_ptr()
-    d.psum_num_recv_tokens_per_expert = psum_expert.data_ptr()
-    d.num_unaligned_recv_tokens_per_expert = unaligned.data_ptr()
-    d.dst_buffer_slot_idx, d.recv_src_metadata = slot.data_ptr(), meta.data_ptr()
-    d.recv_x = recv_x.data_ptr()
-    d.recv_sf = recv_sf.data_ptr() if fp8 else 0
-    d.recv_sf_token_stride, d.recv_sf_hidden_stride = (H // 128, 1) if fp8 else (0, 0)
-    d.recv_topk_idx = recv_idx.data_ptr() if recv_idx is not None else 0
-    d.recv_topk_weights = recv_w.data_ptr()
-    d.recv_capacity, d.expanded_capacity = cap, (ecap if expanded else 0)
-    d.workspace, d.workspace_bytes = workspace.data_ptr(), ws_bytes
-    d.tuning = _abi.Tuning.from_env()
-    d.tuning.dispatch_launches = args.launches
-
-    c = _abi.CombineArgs()
-    c.tuning = _abi.Tuning.from_env()
-    c.do_expand, c.allow_multiple_reduction = int(expanded), 1
-    c.num_tokens, c.hidden, c.num_topk, c.num_experts, c.num_ranks = T, H, K, E, R
-    c.rank_idx, c.num_max_tokens_per_rank = 0, M
-    c.x, c.num_x_rows = y.data_ptr(), rows
-    c.topk_weights = recv_w.data_ptr()
-    c.topk_idx, c.dst_buffer_slot_idx = idx.data_ptr(), slot.data_ptr()
-    c.recv_src_metadata, c.num_recv_rows = meta.data_ptr(), cap
-    c.psum_num_recv_tokens_per_rank = psum_rank.data_ptr()
-    c.combined_x, c.combined_topk_weights = out.data_ptr(), out_w.data_ptr()
-    c.workspace, c.workspace_bytes = workspace.data_ptr(), ws_bytes
-
-    stream = torch.cuda.current_stream()
-    sp = stream.cuda_stream
-    lib = _abi.lib
-
-    def dispatch(phases):
-        d.phases = phases
-        _abi.check(lib.deep_ep_hip_launch_dispatch(ctypes.byref(d), sp), "dispatch")
-
-    def combine():
-        _abi.check(lib.deep_ep_hip_launch_combine(ctypes.byref(c), sp), "combine")
-
-    def step():
-        dispatch(_abi.PHASE_LAYOUT | _abi.PHASE_MOVE)
-        combine()
+    rt = RoutingCalls(torch, _abi, dev, case, fp8, expanded, args.launches)
+    T, H, K, E, R, M = rt.T, rt.H, rt.K, rt.E, rt.R, rt.M
+    N_r, N_e, ab, x, workspace, stream = rt.N_r, rt.N_e, rt.ab, rt.x, rt.workspace, rt.stream
+    dispatch, combine, step = rt.dispatch, rt.combine, rt.step
 
     flush_buf = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev) if args.l2_flush else None
     x_master = x.clone() if args.fresh_input else None
@@ -313,6 +517,15 @@ def main():
     if args.stream_yardsticks:
         result["stream_yardsticks_gbs"] = stream_yardsticks(torch, dev)
 
+    if args.overlap:
+        result["under_compute_load"] = under_compute_load(torch, dev, rt)
+
+    headline = args.workload == "C3" and fp8 and not expanded and args.routing == "case" and not args.l2_flush and not args.fresh_input
+    if headline and not args.brief:
+        result["us_per_api_call"] = {"C3": routing_api_figures(torch, dev, case, kernel_us=(dispatch_us, combine_us))}
+        torch.cuda.empty_cache()
+        result["other_workloads"], result["us_per_api_call"]["C5"] = other_workloads(torch, rc, _abi, dev, case)
+
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens, fp8, expanded)
     print(json.dumps(result))
@@ -361,67 +574,84 @@ def stream_yardsticks(torch, dev, iters=10):
     return out
 
 
-def bench_low_latency(args, torch, rc, _abi, dev):
+class LowLatencyCalls:
     """C5: low-latency decode.  Destination rank 0 of 8 receives from all 8 logical source ranks (128 tokens each,
-    hidden 7168, top-8 of 256): FP8 dispatch into [32, 1024, 7168] packed buffers, weighted BF16 combine back."""
+    hidden 7168, top-8 of 256): FP8 dispatch into [32, 1024, 7168] packed buffers, weighted BF16 combine back.
+    Buffers allocated once, launches straight through the C ABI."""
     R, T, H, E, K, M = 8, 128, 7168, 256, 8, 128
-    E_l, rows = E // R, R * M
-    x_cpu, idx_cpu, w_cpu = rc.c5_sources(seed=0, R=R, T=T, H=H, E=E, K=K)
-    x, idx, w = x_cpu.to(dev), idx_cpu.to(dev), w_cpu.to(dev)
-    n_e = int(((idx_cpu >= 0) & (idx_cpu < E_l)).sum())            # (token, lane) pairs that land on rank 0
-    px = torch.empty((E_l, rows, H), dtype=torch.float8_e4m3fn, device=dev)
-    ps = torch.empty((E_l, H // 128, rows), dtype=torch.float32, device=dev)
-    cnt = torch.empty(E_l, dtype=torch.int32, device=dev)
-    info = torch.empty((E_l, rows), dtype=torch.int32, device=dev)
-    rng = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
-    lane_rows = torch.empty((R * T, K), dtype=torch.int32, device=dev)    # what Buffer keeps beside the handle
-    y = torch.randn((E_l, rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)
-    out = torch.empty((R, T, H), dtype=torch.bfloat16, device=dev)
-    ws = torch.zeros(max(_abi.lib.deep_ep_hip_ll_workspace_bytes(R, T, K, E_l), 4096), dtype=torch.uint8, device=dev)
-    d = _abi.LLDispatchArgs()
-    d.use_fp8, d.num_src_ranks, d.src_rank_begin, d.src_token_stride = 1, R, 0, T
-    d.hidden, d.num_topk, d.num_experts, d.expert_begin, d.num_local_experts = H, K, E, 0, E_l
-    d.num_ranks, d.num_max_dispatch_tokens_per_rank = R, M
-    d.x, d.topk_idx = x.data_ptr(), idx.data_ptr()
-    d.packed_recv_x, d.packed_recv_x_scales, d.packed_recv_count = px.data_ptr(), ps.data_ptr(), cnt.data_ptr()
-    d.packed_recv_src_info, d.packed_recv_layout_range = info.data_ptr(), rng.data_ptr()
-    d.lane_rows = lane_rows.data_ptr()
-    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
-    d.tuning = _abi.Tuning.from_env()
-    c = _abi.LLCombineArgs()
-    c.num_src_ranks, c.src_rank_begin, c.src_token_stride = R, 0, T
-    c.hidden, c.num_topk, c.num_experts, c.expert_begin, c.num_local_experts, c.num_ranks = H, K, E, 0, E_l, R
-    c.num_max_dispatch_tokens_per_rank = M
-    c.x, c.topk_idx, c.topk_weights = y.data_ptr(), idx.data_ptr(), w.data_ptr()
-    c.packed_recv_src_info, c.packed_recv_layout_range, c.combined_x = info.data_ptr(), rng.data_ptr(), out.data_ptr()
-    c.lane_rows = 0 if os.environ.get("BENCH_LL_SEARCH") else lane_rows.data_ptr()
-    c.workspace, c.workspace_bytes = ws.data_ptr(), ws.numel()
-    c.tuning = _abi.Tuning.from_env()
-    stream = torch.cuda.current_stream()
-    sp = stream.cuda_stream
 
-    def dispatch():
-        _abi.check(_abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(d), sp), "ll dispatch")
+    def __init__(self, torch, rc, _abi, dev):
+        self.torch, self._abi = torch, _abi
+        R, T, H, E, K, M = self.R, self.T, self.H, self.E, self.K, self.M
+        E_l, rows = E // R, R * M
+        self.cpu_inputs = x_cpu, idx_cpu, w_cpu = rc.c5_sources(seed=0, R=R, T=T, H=H, E=E, K=K)
+        x, idx, w = x_cpu.to(dev), idx_cpu.to(dev), w_cpu.to(dev)
+        self.inputs = (x, idx, w)
+        self.n_e = n_e = int(((idx_cpu >= 0) & (idx_cpu < E_l)).sum())            # (token, lane) pairs that land on rank 0
+        px = torch.empty((E_l, rows, H), dtype=torch.float8_e4m3fn, device=dev)
+        ps = torch.empty((E_l, H // 128, rows), dtype=torch.float32, device=dev)
+        cnt = torch.empty(E_l, dtype=torch.int32, device=dev)
+        info = torch.empty((E_l, rows), dtype=torch.int32, device=dev)
+        rng = torch.zeros((E_l, R), dtype=torch.int64, device=dev)
+        lane_rows = torch.empty((R * T, K), dtype=torch.int32, device=dev)    # what Buffer keeps beside the handle
+        self.y = y = torch.randn((E_l, rows, H), dtype=torch.float32, device=dev).to(torch.bfloat16)
+        out = torch.empty((R, T, H), dtype=torch.bfloat16, device=dev)
+        ws = torch.zeros(max(_abi.lib.deep_ep_hip_ll_workspace_bytes(R, T, K, E_l), 4096), dtype=torch.uint8, device=dev)
+        self.keep = (px, ps, cnt, info, rng, lane_rows, out, ws)
+        d = self.d = _abi.LLDispatchArgs()
+        d.use_fp8, d.num_src_ranks, d.src_rank_begin, d.src_token_stride = 1, R, 0, T
+        d.hidden, d.num_topk, d.num_experts, d.expert_begin, d.num_local_experts = H, K, E, 0, E_l
+        d.num_ranks, d.num_max_dispatch_tokens_per_rank = R, M
+        d.x, d.topk_idx = x.data_ptr(), idx.data_ptr()
+        d.packed_recv_x, d.packed_recv_x_scales, d.packed_recv_count = px.data_ptr(), ps.data_ptr(), cnt.data_ptr()
+        d.packed_recv_src_info, d.packed_recv_layout_range = info.data_ptr(), rng.data_ptr()
+        d.lane_rows = lane_rows.data_ptr()
+        d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+        d.tuning = _abi.Tuning.from_env()
+        c = self.c = _abi.LLCombineArgs()
+        c.num_src_ranks, c.src_rank_begin, c.src_token_stride = R, 0, T
+        c.hidden, c.num_topk, c.num_experts, c.expert_begin, c.num_local_experts, c.num_ranks = H, K, E, 0, E_l, R
+        c.num_max_dispatch_tokens_per_rank = M
+        c.x, c.topk_idx, c.topk_weights = y.data_ptr(), idx.data_ptr(), w.data_ptr()
+        c.packed_recv_src_info, c.packed_recv_layout_range, c.combined_x = info.data_ptr(), rng.data_ptr(), out.data_ptr()
+        c.lane_rows = 0 if os.environ.get("BENCH_LL_SEARCH") else lane_rows.data_ptr()
+        c.workspace, c.workspace_bytes = ws.data_ptr(), ws.numel()
+        c.tuning = _abi.Tuning.from_env()
+        self.stream = torch.cuda.current_stream()
+        self.sp = self.stream.cuda_stream
+        self.dispatch_bytes = R * T * H * 2 + R * T * K * 8 + n_e * (H + (H // 128) * 4 + 4) + E_l * (4 + R * 8)
+        self.combine_bytes = n_e * H * 2 + R * T * K * 12 + R * T * H * 2
 
-    def combine():
-        _abi.check(_abi.lib.deep_ep_hip_launch_ll_combine(ctypes.byref(c), sp), "ll combine")
+    def dispatch(self):
+        self._abi.check(self._abi.lib.deep_ep_hip_launch_ll_dispatch(ctypes.byref(self.d), self.sp), "ll dispatch")
 
-    def timed(fn, iters):
+    def combine(self):
+        self._abi.check(self._abi.lib.deep_ep_hip_launch_ll_combine(ctypes.byref(self.c), self.sp), "ll combine")
+
+    def step(self):
+        self.dispatch()
+        self.combine()
+
+    def loop_us(self, fn, iters):
+        torch = self.torch
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
+        e0.record(self.stream)
         for _ in range(iters):
             fn()
-        e1.record(stream)
+        e1.record(self.stream)
         e1.synchronize()
         return e0.elapsed_time(e1) * 1e3 / iters
 
+
+def bench_low_latency(args, torch, rc, _abi, dev):
+    ll = LowLatencyCalls(torch, rc, _abi, dev)
+    R, T, H, E, K, M, n_e = ll.R, ll.T, ll.H, ll.E, ll.K, ll.M, ll.n_e
     for _ in range(args.warmup):
-        dispatch(); combine()
+        ll.step()
     torch.cuda.synchronize()
-    step_us = timed(lambda: (dispatch(), combine()), args.steps)
-    d_us, c_us = timed(dispatch, max(args.steps, 20)), timed(combine, max(args.steps, 20))
-    d_bytes = R * T * H * 2 + R * T * K * 8 + n_e * (H + (H // 128) * 4 + 4) + E_l * (4 + R * 8)
-    c_bytes = n_e * H * 2 + R * T * K * 12 + R * T * H * 2
+    step_us = ll.loop_us(ll.step, args.steps)
+    d_us, c_us = ll.loop_us(ll.dispatch, max(args.steps, 20)), ll.loop_us(ll.combine, max(args.steps, 20))
+    d_bytes, c_bytes = ll.dispatch_bytes, ll.combine_bytes
     if args.calibration_copy:
         calibration_copy(torch, dev)
     result = {"metric": "low-latency dispatch+combine us/call, 8 sources x 128 tokens x 7168, top-8 of 256, destination rank 0",
@@ -438,8 +668,9 @@ def bench_low_latency(args, torch, rc, _abi, dev):
             "roofline_combine": {"kernel": "ll_combine_kernel", "bound": "hbm", "achieved": round(c_bytes / c_us * 1e-3, 1),
                                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(c_bytes / c_us * 1e-3 / HBM_PEAK_GBS, 4),
                                  "traffic": MEASURED_TRAFFIC_BYTES.get(("C5", "packed", "fp8", "ll_combine"))}}
+    result["us_per_api_call"] = low_latency_api_figures(torch, ll, kernel_us=(d_us, c_us))
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline_low_latency(x_cpu, idx_cpu, w_cpu, R, M, E)
+        result["cpu_baseline"] = cpu_baseline_low_latency(*ll.cpu_inputs, R, M, E)
     return result
 
 

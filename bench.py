@@ -359,6 +359,8 @@ def main():
     ap.add_argument("--l2-flush", action="store_true", help="zero a 256 MB buffer between per-kernel timings")
     ap.add_argument("--overlap", action="store_true",
                     help="also time dispatch and combine on a stream of their own while matrix products fill the GPU on another")
+    ap.add_argument("--persistent-movers", type=int, default=0,
+                    help="dispatch move phase as a persistent kernel with this many workgroups per compute unit (implies two launches)")
     ap.add_argument("--brief", action="store_true", help="only the headline workload: no other workloads, no API-level figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -386,6 +388,7 @@ def main():
     fp8 = not args.bf16
     expanded = args.expanded
     rt = RoutingCalls(torch, _abi, dev, case, fp8, expanded, args.launches)
+    rt.d.tuning.persistent_movers = args.persistent_movers
     T, H, K, E, R, M = rt.T, rt.H, rt.K, rt.E, rt.R, rt.M
     N_r, N_e, ab, x, workspace, stream = rt.N_r, rt.N_e, rt.ab, rt.x, rt.workspace, rt.stream
     dispatch, combine, step = rt.dispatch, rt.combine, rt.step
@@ -488,7 +491,7 @@ def main():
         "config": {"workload": f"{case.name}: T={T} H={H} E={E} R={R} K={K} "
                                f"{'expanded' if expanded else 'compact'} layout, N_r={N_r}, N_e={N_e}",
                    "l2_flush": bool(args.l2_flush), "fresh_input": bool(args.fresh_input),
-                   "dispatch_launches": args.launches},
+                   "dispatch_launches": args.launches, "persistent_movers": args.persistent_movers},
         "us_per_single_launch": dist,
         "us_per_call": {"dispatch": round(dispatch_us, 2), "dispatch_layout": round(layout_us, 2),
                         "dispatch_move": round(move_us, 2), "combine": round(combine_us, 2)},
@@ -520,7 +523,8 @@ def main():
     if args.overlap:
         result["under_compute_load"] = under_compute_load(torch, dev, rt)
 
-    headline = args.workload == "C3" and fp8 and not expanded and args.routing == "case" and not args.l2_flush and not args.fresh_input
+    headline = (args.workload == "C3" and fp8 and not expanded and args.routing == "case" and not args.l2_flush and
+                not args.fresh_input and args.persistent_movers == 0)
     if headline and not args.brief:
         result["us_per_api_call"] = {"C3": routing_api_figures(torch, dev, case, kernel_us=(dispatch_us, combine_us))}
         torch.cuda.empty_cache()

@@ -63,7 +63,8 @@ LaunchPlan plan_launches(int T, int K, int E, int R, bool do_layout, bool do_mov
     q.chunks = T > 0 ? (T + kLayoutChunk - 1) / kLayoutChunk : 1;
     q.chunks_padded = (q.chunks + 3) / 4 * 4;
     q.fused = do_layout && do_move && T > 0 && K <= 8 && (R + E) <= 512 && R * q.chunks_padded <= kTaggedRankWords &&
-              int64_t(T) * K <= kTaggedPosWords && tuning.dispatch_launches != 2;
+              int64_t(T) * K <= kTaggedPosWords && tuning.dispatch_launches != 2 &&
+              !(tuning.persistent_movers > 0 && payload == DEEP_EP_HIP_PAYLOAD_CAST_FP8);      // the persistent move runs on a finished layout
     if (q.fused && do_expand) {
         // the tagged expert bases: the table must fit, and a row number must fit under the tag
         const int64_t experts_padded = (int64_t(E) + 31) / 32 * 32;
@@ -341,6 +342,7 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
         m.mover_spin_limit = a->tuning.mover_spin_limit > 0 ? unsigned(a->tuning.mover_spin_limit) : (1u << 22);   // seconds
         m.move_workgroups_per_cu = a->tuning.move_workgroups_per_cu;
         m.warm_rounds = a->tuning.warm_rounds;
+        m.persistent_movers = a->tuning.persistent_movers;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 
@@ -670,6 +672,7 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.mover_spin_limit = a->tuning.mover_spin_limit > 0 ? unsigned(a->tuning.mover_spin_limit) : (1u << 22);   // seconds
         m.move_workgroups_per_cu = a->tuning.move_workgroups_per_cu;
         m.warm_rounds = a->tuning.warm_rounds;
+        m.persistent_movers = a->tuning.persistent_movers;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 

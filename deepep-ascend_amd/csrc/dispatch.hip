@@ -866,6 +866,96 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
     }
 }
 
+// ---- the same move as a persistent kernel (tuning.persistent_movers) ----
+// A few workgroups per compute unit stay resident and their wavefronts loop over the work items (wavefront w takes items
+// w, w + W, w + 2W, ...), with the loads of the next item - payload tile, top-k ids, weights, position words - issued
+// before the current item is converted and stored.  Kept as a measured alternative, not a default: on MI355X it is
+// slower than one short-lived wavefront per work item (8192 x 7168 FP8, move phase on a finished layout: 96 / 103 / 96 us
+// with four / six / eight workgroups per compute unit against 82 us).  A likely reason: one counter orders a wavefront's
+// loads and stores, so a looping wavefront waits for the acknowledgement of the stores of item i before it can use the
+// loads of item i + 1 that were issued behind them, while a short-lived wavefront hands its stores to the memory system
+// and leaves, and the next one starts with an empty queue.
+template <int kPairs>
+struct CastItem {
+    vec16 in[kPairs][2];
+    RouteInputs route_in;
+    uint32_t word;
+};
+
+template <int kPairs>
+__device__ __forceinline__ void load_cast_item(const MoveParams& p, unsigned work, int lane, CastItem<kPairs>& item) {
+    const int t = int(work / unsigned(p.tiles));
+    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
+    const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
+#pragma unroll
+    for (int q = 0; q < kPairs; ++q) {
+        const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+        item.in[q][0] = vec16{0, 0, 0, 0};
+        item.in[q][1] = vec16{0, 0, 0, 0};
+        if (elem < p.H) {
+            item.in[q][0] = load16_stream(src + int64_t(elem) * 2);
+            item.in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+        }
+    }
+    item.route_in = load_route_inputs(p, t, lane);
+    item.word = load_position_word(p, t, lane);
+}
+
+template <int kPairs>
+__device__ __forceinline__ void finish_cast_item(const MoveParams& p, unsigned work, int lane, const CastItem<kPairs>& item) {
+    const int t = int(work / unsigned(p.tiles));
+    const int tile = int(work - unsigned(t) * unsigned(p.tiles));
+    const Route r = resolve_route<false>(p, item.route_in, item.word, nullptr, 0, t, lane, tile == 0);
+    if (tile == 0) write_token_metadata(p, r, t, lane);
+    vec16 out[kPairs];
+    float my_scale = 0.f;
+#pragma unroll
+    for (int q = 0; q < kPairs; ++q) {
+        const float scale_inv = cast_16_channels(item.in[q][0], item.in[q][1], out[q]);
+        const float gathered = __shfl(scale_inv, (lane & 7) * 8, kWaveSize);
+        if ((lane >> 3) == q) my_scale = gathered;
+    }
+    const int group = tile * kPairs * 8 + lane;
+    const bool owns_scale = lane < kPairs * 8 && group * 128 < p.H;
+    int row_of_lane;
+    uint64_t dests = destination_lanes(p, r, row_of_lane);
+    while (dests) {
+        const int j = __builtin_ctzll(dests);
+        dests &= dests - 1;
+        const int row = read_lane(row_of_lane, j);
+        uint8_t* dst = p.recv_x + int64_t(row) * p.H;
+#pragma unroll
+        for (int q = 0; q < kPairs; ++q) {
+            const int elem = (tile * kPairs + q) * 1024 + lane * 16;
+            if (elem < p.H) store16_stream(dst + elem, out[q]);
+        }
+        if (owns_scale) p.recv_sf[int64_t(row) * p.rsf_ts + int64_t(group) * p.rsf_hs] = __float_as_uint(my_scale);
+    }
+}
+
+template <int kPairs>
+__global__ __launch_bounds__(kThreads) void dispatch_cast_persistent_kernel(const MoveParams p) {
+    const int lane = threadIdx.x & 63;
+    const unsigned total = unsigned(p.T) * unsigned(p.tiles);
+    const unsigned stride = gridDim.x * unsigned(kWavesPerBlock);
+    unsigned work = wave_work_index(blockIdx.x, kWavesPerBlock);
+    if (work >= total) return;
+    CastItem<kPairs> a, b;
+    load_cast_item<kPairs>(p, work, lane, a);
+    for (;;) {                                         // every wavefront leaves through one of the two breaks
+        unsigned next = work + stride;
+        if (next < total) load_cast_item<kPairs>(p, next, lane, b);
+        finish_cast_item<kPairs>(p, work, lane, a);
+        if (next >= total) break;
+        work = next;
+        next = work + stride;
+        if (next < total) load_cast_item<kPairs>(p, next, lane, a);
+        finish_cast_item<kPairs>(p, work, lane, b);
+        if (next >= total) break;
+        work = next;
+    }
+}
+
 // The kernels.  The single-launch forms also hold the counting and publishing code, whose register needs must not cost
 // the movers their occupancy: they are held to six wavefronts per SIMD (80 registers) - six workgroups per CU, which
 // is also where the move streams fastest (more were slower when tried with a leaner counting step, fewer are slower too).
@@ -1073,6 +1163,13 @@ hipError_t launch_cast(MoveParams p, hipStream_t stream) {
         }
     }
     if (p.fused) return hipErrorInvalidConfiguration;      // the launch plan keeps wider tiles out of the single launch
+    if constexpr (kPairs <= 2) {
+        if (p.persistent_movers > 0) {
+            const unsigned resident = unsigned(compute_units()) * unsigned(p.persistent_movers > 8 ? 8 : p.persistent_movers);
+            hipLaunchKernelGGL((dispatch_cast_persistent_kernel<kPairs>), dim3(resident < blocks ? resident : blocks), dim3(kThreads), 0, stream, p);
+            return hipGetLastError();
+        }
+    }
     hipLaunchKernelGGL((dispatch_cast_kernel<kPairs>), dim3(blocks), dim3(kThreads), move_lds_bytes(p), stream, p);
     return hipGetLastError();
 }

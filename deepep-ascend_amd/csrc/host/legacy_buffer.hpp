@@ -396,10 +396,15 @@ public:
         c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
         const auto dev = torch::TensorOptions().device(device_);
         torch::Tensor packed_recv_x = torch::empty({E_l, rows, H}, dev.dtype(use_fp8 ? torch::kFloat8_e4m3fn : torch::kBFloat16));
-        torch::Tensor packed_recv_src_info = torch::empty({E_l, rows}, dev.dtype(torch::kInt32));
-        torch::Tensor packed_recv_layout_range = torch::zeros({E_l, R}, dev.dtype(torch::kInt64));
-        torch::Tensor packed_recv_count = torch::empty({E_l}, dev.dtype(torch::kInt32));
-        torch::Tensor lane_rows = torch::empty({int64_t(S) * T, K}, dev.dtype(torch::kInt32));
+        // The small outputs share one allocation (each torch allocation costs the host about a microsecond, which
+        // counts in a call of twenty): ranges first, for their 8-byte alignment.  The kernel writes every range,
+        // (begin 0, count 0) for source ranks that do not send in this call.
+        const int64_t n_range = int64_t(E_l) * R, n_info = int64_t(E_l) * rows, n_lane = int64_t(S) * T * K;
+        torch::Tensor small = torch::empty({2 * n_range + n_info + E_l + n_lane}, dev.dtype(torch::kInt32));
+        torch::Tensor packed_recv_layout_range = small.slice(0, 0, 2 * n_range).view(torch::kInt64).view({E_l, R});
+        torch::Tensor packed_recv_src_info = small.slice(0, 2 * n_range, 2 * n_range + n_info).view({E_l, rows});
+        torch::Tensor packed_recv_count = small.slice(0, 2 * n_range + n_info, 2 * n_range + n_info + E_l);
+        torch::Tensor lane_rows = small.slice(0, 2 * n_range + n_info + E_l, 2 * n_range + n_info + E_l + n_lane).view({int64_t(S) * T, K});
         std::optional<torch::Tensor> packed_recv_x_scales;
         if (use_fp8 and use_ue8m0) packed_recv_x_scales = torch::empty({E_l, H / 512, rows}, dev.dtype(torch::kInt32)).transpose(1, 2);
         else if (use_fp8) packed_recv_x_scales = torch::empty({E_l, H / 128, rows}, dev.dtype(torch::kFloat32)).transpose(1, 2);
@@ -428,6 +433,7 @@ public:
             // its search through src_info
             lane_rows_of_handle_.remember(packed_recv_src_info, lane_rows);
         } else {
+            packed_recv_layout_range.zero_();
             packed_recv_count.zero_();
         }
         ll_last_stream_ = run;

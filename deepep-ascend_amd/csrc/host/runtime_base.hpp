@@ -66,6 +66,7 @@ inline deep_ep_hip_tuning& process_tuning() {
         t.mover_spin_limit = env("DEEP_EP_HIP_MOVER_SPIN_LIMIT");
         t.move_workgroups_per_cu = env("DEEP_EP_HIP_MOVE_WORKGROUPS_PER_CU");
         t.warm_rounds = env("DEEP_EP_HIP_WARM_ROUNDS");
+        t.persistent_movers = env("DEEP_EP_HIP_PERSISTENT_MOVERS");
         return t;
     }();
     return tuning;
@@ -86,6 +87,7 @@ inline int32_t* tuning_field(const std::string& name) {
     if (name == "mover_spin_limit") return &t.mover_spin_limit;
     if (name == "move_workgroups_per_cu") return &t.move_workgroups_per_cu;
     if (name == "warm_rounds") return &t.warm_rounds;
+    if (name == "persistent_movers") return &t.persistent_movers;
     throw EPException("unknown tuning field: " + name);
 }
 

@@ -163,6 +163,7 @@ struct MoveParams {
     unsigned mover_spin_limit;   // reads a mover repeats for a word of the layout before it gives up (set from the tuning block)
     int move_workgroups_per_cu;  // forced residency of a move kernel on a finished layout, 0 = choose (tuning block)
     int warm_rounds;             // rounds ahead the first movers of a single launch warm the caches, 0 = choose, < 0 = none (tuning block)
+    int persistent_movers;       // fused-cast move kernel on a finished layout as a persistent kernel with this many workgroups per CU, 0 = off (tuning block)
     uint32_t* generation;        // see WorkspaceLayout
     uint32_t* tagged;            // the tagged tables, tagged_words long: cleared by the launch that uses the last tag
     int tagged_words;

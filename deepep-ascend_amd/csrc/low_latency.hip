@@ -116,6 +116,9 @@ __global__ __launch_bounds__(kThreads) void ll_count_kernel(const LLDispatchPara
         }
         p.packed_count[j] = running;
         if (p.cumulative_stats != nullptr) p.cumulative_stats[j] += running;
+        // source ranks that do not send in this call: (begin 0, count 0)
+        for (int r = 0; r < p.R; ++r)
+            if (r < p.src_rank_begin || r >= p.src_rank_begin + p.S) p.packed_layout_range[int64_t(j) * p.R + r] = 0;
     }
     if (tid == 0) *p.done_counter = 0u;
 }
@@ -262,6 +265,9 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     const bool live = has_work && t < tokens_of_source(p, s);
     vec16 in[kPairs][2];
     if (live) ll_load_tile<kPairs>(p, g, tile, lane, in);
+    // ... and so does the read of this token's own selections: behind the routing pass it would be one more trip to
+    // the L2 on the critical path
+    const int64_t own_raw = (live && lane < p.K) ? p.topk_idx[g * p.K + lane] : int64_t(-1);
 
     for (int i = tid; i < p.E_l * words; i += kFusedThreads) bits[i] = 0ull;
     __syncthreads();
@@ -325,6 +331,9 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
             }
             p.packed_count[le] = running;
             if (p.cumulative_stats != nullptr) p.cumulative_stats[le] += running;
+            // source ranks that do not send in this call: (begin 0, count 0)
+            for (int r = 0; r < p.R; ++r)
+                if (r < p.src_rank_begin || r >= p.src_rank_begin + p.S) p.packed_layout_range[int64_t(le) * p.R + r] = 0;
         }
         return;
     }
@@ -340,7 +349,7 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     };
     int le = -1, slot = -1, flags = 0;
     if (lane < p.K) {
-        const int64_t raw = p.topk_idx[g * p.K + lane];
+        const int64_t raw = own_raw;
         if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
         if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) {
             le = int(raw) - p.expert_begin;
@@ -494,13 +503,13 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
         for (int c = 0; c < 8; ++c) acc[i][c] = 0.f;
 
     uint64_t srcs = __ballot(row_of_lane >= 0);
-    while (srcs) {
-        const int j = __builtin_ctzll(srcs);
-        srcs &= srcs - 1;
-        const int64_t row = int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j);
-        const float wj = read_lane(w, j);
-        const uint8_t* src = p.x + row * row_bytes;
-        if constexpr (kLogFmt) {
+    if constexpr (kLogFmt) {
+        while (srcs) {
+            const int j = __builtin_ctzll(srcs);
+            srcs &= srcs - 1;
+            const int64_t row = int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j);
+            const float wj = read_lane(w, j);
+            const uint8_t* src = p.x + row * row_bytes;
             // hidden % (kVecs * 512) == 0: every lane of the tile holds channels of the row
             float val[kVecs][8], mag[kVecs][8];
             LogFmtGroup group[kVecs];
@@ -522,16 +531,46 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
 #pragma unroll
                 for (int c = 0; c < 8; ++c) acc[i][c] += val[i][c] * wj;
             }
-        } else {
+        }
+    } else {
+        // Rows go in rounds of up to four: the loads of a round are all issued before its first multiply-add, so a
+        // token with many local lanes pays one trip to memory per four rows, not one per row.  The sum keeps lane order.
+        constexpr int kRound = 4;
+        while (srcs) {
+            const uint8_t* src[kRound];
+            float wj[kRound];
 #pragma unroll
-            for (int i = 0; i < kVecs; ++i) {
-                const int off = (tile * kVecs + i) * 1024 + lane * 16;
-                if (off < row_bytes) {
-                    const vec16 v = load16_stream(src + off);
-                    acc[i][0] += bf16_lo(v.x) * wj; acc[i][1] += bf16_hi(v.x) * wj;
-                    acc[i][2] += bf16_lo(v.y) * wj; acc[i][3] += bf16_hi(v.y) * wj;
-                    acc[i][4] += bf16_lo(v.z) * wj; acc[i][5] += bf16_hi(v.z) * wj;
-                    acc[i][6] += bf16_lo(v.w) * wj; acc[i][7] += bf16_hi(v.w) * wj;
+            for (int b = 0; b < kRound; ++b) {
+                src[b] = nullptr;
+                wj[b] = 0.f;
+                if (srcs) {
+                    const int j = __builtin_ctzll(srcs);
+                    srcs &= srcs - 1;
+                    src[b] = p.x + (int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j)) * row_bytes;
+                    wj[b] = read_lane(w, j);
+                }
+            }
+            vec16 v[kRound][kVecs];
+#pragma unroll
+            for (int b = 0; b < kRound; ++b)
+#pragma unroll
+                for (int i = 0; i < kVecs; ++i) {
+                    const int off = (tile * kVecs + i) * 1024 + lane * 16;
+                    v[b][i] = vec16{0, 0, 0, 0};
+                    if (src[b] != nullptr && off < row_bytes) v[b][i] = load16_stream(src[b] + off);
+                }
+#pragma unroll
+            for (int b = 0; b < kRound; ++b) {
+                if (src[b] == nullptr) continue;           // wave-uniform: an absent row adds nothing, not 0 * weight
+#pragma unroll
+                for (int i = 0; i < kVecs; ++i) {
+                    const int off = (tile * kVecs + i) * 1024 + lane * 16;
+                    if (off < row_bytes) {
+                        acc[i][0] += bf16_lo(v[b][i].x) * wj[b]; acc[i][1] += bf16_hi(v[b][i].x) * wj[b];
+                        acc[i][2] += bf16_lo(v[b][i].y) * wj[b]; acc[i][3] += bf16_hi(v[b][i].y) * wj[b];
+                        acc[i][4] += bf16_lo(v[b][i].z) * wj[b]; acc[i][5] += bf16_hi(v[b][i].z) * wj[b];
+                        acc[i][6] += bf16_lo(v[b][i].w) * wj[b]; acc[i][7] += bf16_hi(v[b][i].w) * wj[b];
+                    }
                 }
             }
         }

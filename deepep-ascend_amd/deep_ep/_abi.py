@@ -35,7 +35,7 @@ class Tuning(Structure):
         ("dispatch_launches", c_int32), ("cast_pairs", c_int32), ("copy_vecs", c_int32), ("plain_loads", c_int32),
         ("xcd_remap", c_int32), ("combine_vecs", c_int32), ("ll_pairs", c_int32), ("ll_threads", c_int32),
         ("ll_two_kernels", c_int32), ("ll_combine_vecs", c_int32), ("mover_spin_limit", c_int32),
-        ("move_workgroups_per_cu", c_int32), ("warm_rounds", c_int32), ("reserved", c_int32 * 3),
+        ("move_workgroups_per_cu", c_int32), ("warm_rounds", c_int32), ("persistent_movers", c_int32), ("reserved", c_int32 * 2),
     ]
 
     @classmethod

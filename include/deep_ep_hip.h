@@ -97,7 +97,11 @@ typedef struct {
                                   load, into the caches only, the tiles of the work items this many rounds of resident
                                   workgroups ahead of their own (0 = 2, or 1 in launches of one and a half to two rounds;
                                   negative = none) */
-    int32_t reserved[3];
+    int32_t persistent_movers; /* fused-cast dispatch: > 0 = the move phase as a persistent kernel, this many workgroups per
+                                  compute unit (1..8), whose wavefronts loop over the work items with the next item's loads
+                                  issued before the current item's stores; implies layout kernel + move kernel.  A measured
+                                  alternative (slower on MI355X), not a default */
+    int32_t reserved[2];
 } deep_ep_hip_tuning;
 
 /* Bytes of workspace needed for dispatches of up to num_max_tokens tokens.  The workspace must
@@ -368,7 +372,8 @@ typedef struct {
                                            use_ue8m0: byte (e, row, g) at ((e*G/4 + g/4)*rows + row)*4 + g%4 */
     int32_t* packed_recv_count;         /* [num_local_experts] out */
     int32_t* packed_recv_src_info;      /* [num_local_experts, rows] out */
-    int64_t* packed_recv_layout_range;  /* [num_local_experts, num_ranks] out: (begin<<32)|count */
+    int64_t* packed_recv_layout_range;  /* [num_local_experts, num_ranks] out: (begin<<32)|count; columns of ranks
+                                           that do not send in this call are written as 0 */
     int32_t* cumulative_local_expert_recv_stats; /* [num_local_experts] += counts, or NULL */
     int32_t* lane_rows;                 /* optional out [num_src_ranks * src_token_stride, num_topk]: e * rows + slot of
                                            the packed row each (token, lane) went to, -1 if none.  Not part of the

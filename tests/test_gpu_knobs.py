@@ -15,6 +15,7 @@ KNOBS = [
     ("cast_pairs", 1), ("cast_pairs", 4), ("cast_pairs", 7), ("cast_pairs", 8), ("copy_vecs", 1), ("copy_vecs", 2),
     ("copy_vecs", 7), ("copy_vecs", 8), ("combine_vecs", 1), ("combine_vecs", 4),
     ("move_workgroups_per_cu", 3), ("move_workgroups_per_cu", 8), ("warm_rounds", -1), ("warm_rounds", 1),
+    ("persistent_movers", 1), ("persistent_movers", 6),
 ]
 
 

@@ -283,6 +283,7 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
     pub.num_unaligned = a->num_unaligned_recv_tokens_per_expert;
     pub.cumulative_stats = a->cumulative_local_expert_recv_stats;
     pub.host_counts = a->host_counts;
+    pub.status = status;
     pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
 
@@ -602,6 +603,7 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
     pub.psum_rank = a->psum_num_recv_tokens_per_rank;
     pub.num_unaligned = with_topk ? a->num_recv_tokens_per_expert : nullptr;
     pub.host_counts = a->host_counts;
+    pub.status = status;
     pub.expert_start = reinterpret_cast<int32_t*>(ws + w.expert_start);
     pub.totals_out = reinterpret_cast<int32_t*>(ws + w.totals);
 

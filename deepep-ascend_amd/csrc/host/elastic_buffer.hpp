@@ -223,23 +223,23 @@ public:
             num_expanded_tokens = *cached_num_expanded_tokens;
             per_expert_list = *cached_num_recv_tokens_per_expert_list;
         } else if (do_cpu_sync) {
+            // layout launch, then the host waits for the counts in its mailbox (no copy, no device synchronisation)
+            int32_t* box = fresh_mailbox(R + num_experts + 1);
             args.phases = DEEP_EP_HIP_PHASE_LAYOUT;
+            args.host_counts = box;
             check_abi(deep_ep_hip_launch_dispatch(&args, stream_ptr), "dispatch layout");
-            torch::Tensor host;
-            {
+            args.host_counts = nullptr;
+            if (not await_mailbox(box, R + num_experts + 1, num_cpu_timeout_secs_))
+                throw EPException("DeepEP HIP backend: dispatch: timed out waiting for the layout counts");
+            if (box[R + num_experts] != 0) {
                 c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
-                host = counts.cpu();                               // waits for the layout kernel
+                read_and_clear_status(workspace, "dispatch");          // raises, and leaves the workspace ready again
             }
-            read_and_clear_status(workspace, "dispatch");
-            const int32_t* h = host.data_ptr<int32_t>();
-            num_recv_tokens = h[R - 1];
+            num_recv_tokens = 0;
+            for (int r = 0; r < R; ++r) num_recv_tokens += box[r];
             num_expanded_tokens = 0;
-            per_expert_list.resize(num_experts);
-            for (int e = 0; e < num_experts; ++e) {
-                const int aligned = (h[R + num_experts + e] + expert_alignment - 1) / expert_alignment * expert_alignment;
-                per_expert_list[e] = aligned;
-                num_expanded_tokens += aligned;
-            }
+            per_expert_list.assign(box + R, box + R + num_experts);         // aligned counts
+            for (int e = 0; e < num_experts; ++e) num_expanded_tokens += per_expert_list[e];
         } else {
             num_recv_tokens = num_max_tokens_per_rank * R;
             num_expanded_tokens = num_max_tokens_per_rank * std::min(num_topk, num_experts) + (expert_alignment - 1) * num_experts;

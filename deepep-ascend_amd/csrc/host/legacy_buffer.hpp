@@ -240,21 +240,30 @@ public:
                 args.phases = DEEP_EP_HIP_PHASE_LAYOUT | DEEP_EP_HIP_PHASE_MOVE;
                 args.fill_unused_topk_idx = 1;
             } else {
-                // the reference spins on host-mapped counters here (csrc/legacy/buffer.hpp:580-600)
+                // The host waits for the counts of the layout launch, as the reference does on its host-mapped counters
+                // (csrc/legacy/buffer.hpp:580-600).  With top-k tensors they arrive in the pinned mailbox; without,
+                // the per-expert counts are the caller's tensor and are copied back with the per-rank ones.
                 args.phases = DEEP_EP_HIP_PHASE_LAYOUT;
-                check_abi(deep_ep_hip_launch_intranode_dispatch(&args, stream_ptr), "intranode dispatch layout");
-                torch::Tensor host;
-                if (topk_idx.has_value()) {
-                    host = counts.cpu();
-                    read_and_clear_status(workspace, "dispatch");
-                } else {
-                    host = torch::cat({counts.slice(0, 0, R), *num_tokens_per_expert}).cpu();
-                }
-                const int32_t* h = host.data_ptr<int32_t>();
-                num_recv_tokens = h[R - 1];
                 per_expert_list.resize(num_experts);
-                for (int e = 0; e < num_experts; ++e)
-                    per_expert_list[e] = (h[R + e] + expert_alignment - 1) / expert_alignment * expert_alignment;
+                if (topk_idx.has_value()) {
+                    int32_t* box = fresh_mailbox(R + num_experts + 1);
+                    args.host_counts = box;
+                    check_abi(deep_ep_hip_launch_intranode_dispatch(&args, stream_ptr), "intranode dispatch layout");
+                    args.host_counts = nullptr;
+                    if (not await_mailbox(box, R + num_experts + 1, 300))
+                        throw EPException("DeepEP HIP backend: dispatch: timed out waiting for the layout counts");
+                    if (box[R + num_experts] != 0) read_and_clear_status(workspace, "dispatch");      // raises
+                    num_recv_tokens = 0;
+                    for (int r = 0; r < R; ++r) num_recv_tokens += box[r];
+                    std::copy(box + R, box + R + num_experts, per_expert_list.begin());               // aligned counts
+                } else {
+                    check_abi(deep_ep_hip_launch_intranode_dispatch(&args, stream_ptr), "intranode dispatch layout");
+                    const torch::Tensor host = torch::cat({counts.slice(0, 0, R), *num_tokens_per_expert}).cpu();
+                    const int32_t* h = host.data_ptr<int32_t>();
+                    num_recv_tokens = h[R - 1];
+                    for (int e = 0; e < num_experts; ++e)
+                        per_expert_list[e] = (h[R + e] + expert_alignment - 1) / expert_alignment * expert_alignment;
+                }
                 args.phases = DEEP_EP_HIP_PHASE_MOVE;
             }
         }

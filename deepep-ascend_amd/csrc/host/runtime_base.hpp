@@ -12,6 +12,7 @@
 #include <torch/types.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cstdint>
 #include <cstdlib>
 #include <deque>
@@ -334,6 +335,35 @@ protected:
                                                                                                num_experts, num_ranks_)));
     }
 
+    // The mailbox through which a layout launch tells the host its counts (deep_ep_hip_dispatch_args::host_counts): pinned
+    // host memory the kernel writes directly, zeroed here, so that sizing the outputs takes no device-to-host copy and no
+    // device synchronisation (the reference's host-mapped counters, csrc/elastic/buffer.hpp:1019-1066).
+    int32_t* fresh_mailbox(int entries) {
+        if (not mailbox_.has_value())
+            mailbox_ = torch::zeros({DEEP_EP_HIP_MAX_RANKS + DEEP_EP_HIP_MAX_EXPERTS + 1},
+                                    torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
+        EP_HIP_HOST_ASSERT(entries <= mailbox_->numel());
+        int32_t* box = mailbox_->data_ptr<int32_t>();
+        std::fill(box, box + entries, 0);
+        return box;
+    }
+
+    // Waits (bounded by the buffer's CPU timeout) until the kernel has published all `entries` values; decodes them in
+    // place.  Returns false on a timeout.
+    static bool await_mailbox(int32_t* box, int entries, int timeout_secs) {
+        const auto deadline = std::chrono::steady_clock::now() + std::chrono::seconds(timeout_secs > 0 ? timeout_secs : 300);
+        volatile int32_t* watched = box;
+        uint32_t spins = 0;
+        for (int i = 0; i < entries; ++i) {
+            while (watched[i] >= 0) {
+                if ((++spins & 0xfffu) == 0 and std::chrono::steady_clock::now() > deadline) return false;
+                __builtin_ia32_pause();
+            }
+            box[i] = -watched[i] - 1;
+        }
+        return true;
+    }
+
     void read_and_clear_status(const torch::Tensor& workspace, const char* what) {
         const int status = workspace.slice(0, 0, 4).view(torch::kInt32).item<int>();
         if (status == 0) return;
@@ -361,6 +391,7 @@ protected:
     Stream last_stream_;                     // stream of the last launch that used the workspace
     torch::Device device_ = torch::Device(torch::kCUDA, 0);
     std::optional<torch::Tensor> workspace_;
+    std::optional<torch::Tensor> mailbox_;            // pinned: counts of a layout launch for a call that waits for them
     std::optional<torch::Tensor> status_host_;        // one pinned int32: where poll_device_status has the status copied
     std::optional<EventHandle> status_read_;          // recorded after the read in flight
 };

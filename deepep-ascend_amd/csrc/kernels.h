@@ -87,7 +87,8 @@ struct PublishParams {
     int32_t* psum_expert;
     int32_t* num_unaligned;
     int32_t* cumulative_stats;
-    int32_t* host_counts;            // host-mapped
+    int32_t* host_counts;            // host-mapped: [R] rank counts, [E] aligned expert counts, then the status word; v as -v-1
+    const int32_t* status;           // the device status word (read for host_counts)
     int32_t* expert_start;           // workspace
     int32_t* totals_out;             // workspace: total compact rows, total expanded rows
 };

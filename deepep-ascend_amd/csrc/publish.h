@@ -183,7 +183,12 @@ __device__ void publish_experts(const PublishParams& q, const PublishLds& s) {
         if (q.psum_expert != nullptr) q.psum_expert[j] = q.do_expand ? start + s.totals[q.R + j] : s.aligned_incl[j];
     }
     if (threadIdx.x == 0 && q.totals_out != nullptr) q.totals_out[1] = q.E > 0 ? s.aligned_incl[q.E - 1] : 0;
-    if (q.host_counts != nullptr) __threadfence_system();
+    if (q.host_counts != nullptr) {
+        // The status word as the counting workgroups left it (they are all done when a workgroup publishes): a host that
+        // sizes its outputs from this mailbox learns about bad routing input without a second trip to the device.
+        if (threadIdx.x == 0) q.host_counts[q.R + q.E] = -(q.status != nullptr ? load_agent(q.status) : 0) - 1;
+        __threadfence_system();
+    }
 }
 
 // table[c][e] = start of expert e's region + sum of expert_counts[0..c)[e], each word ORed with `tag`.

@@ -189,8 +189,11 @@ typedef struct {
     int32_t* psum_num_recv_tokens_per_expert;   /* [num_experts] */
     int32_t* num_unaligned_recv_tokens_per_expert; /* [num_experts] */
     int32_t* cumulative_local_expert_recv_stats;   /* [num_experts] += actual counts, or NULL */
-    int32_t* host_counts;           /* host-mapped [num_ranks + num_experts] or NULL: per-rank counts
-                                       then aligned per-expert counts, value v published as -v-1 */
+    int32_t* host_counts;           /* NULL, or host memory the GPU can write (hipHostMalloc), [num_ranks + num_experts + 1],
+                                       zeroed by the caller before the call: per-rank counts, aligned per-expert counts,
+                                       then the status word as the layout phase left it, each value v published as
+                                       -v-1 (an entry is there once it reads negative: a host that polls needs no
+                                       device synchronisation to size its outputs) */
     int32_t* dst_buffer_slot_idx;   /* [num_tokens, num_topk]: written by phase 2 (input when cached) */
     int32_t* recv_src_metadata;     /* [recv_capacity, num_topk + 2]: written by phase 2 (input when cached) */
 
@@ -306,7 +309,8 @@ typedef struct {
     int32_t* recv_channel_prefix_matrix;    /* [num_ranks, num_channels] out (phase 1), may be NULL */
     int32_t* psum_num_recv_tokens_per_rank; /* [num_ranks] inclusive, out of phase 1, read by phase 2 */
     int32_t* num_recv_tokens_per_expert;    /* [num_experts] counts before alignment, out of phase 1, or NULL */
-    int32_t* host_counts;                   /* host-mapped [num_ranks + num_experts] or NULL (see dispatch) */
+    int32_t* host_counts;                   /* host memory [num_ranks + max(num_experts, num_ranks) + 1] or NULL (see dispatch;
+                                               without top-k tensors the "experts" are the ranks) */
     int32_t* send_head;                     /* [num_tokens, num_ranks]: out of phase 2 (input when cached) */
     int32_t* recv_src_idx;                  /* [recv_capacity] out of phase 2, or NULL */
 

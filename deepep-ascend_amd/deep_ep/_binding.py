@@ -3,6 +3,8 @@ pybind module, csrc/python_api.cpp:37-54).  There is no second host path: if the
 package import fails and says how to build it."""
 import importlib
 
+import torch  # noqa: F401  (the extension's argument converters need torch's Python module loaded first)
+
 from . import _abi
 
 try:

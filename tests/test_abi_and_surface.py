@@ -443,3 +443,14 @@ def test_event_overlap_hooks_without_gpu():
 def test_runtime_fails_loudly_without_gpu():
     with pytest.raises(RuntimeError, match="no GPU"):
         deep_ep.ElasticBuffer(deep_ep.LogicalGroup(0, 2), num_max_tokens_per_rank=16, hidden=256, num_topk=2)
+
+
+def test_package_imports_in_a_fresh_interpreter_before_torch():
+    """`import deep_ep` as the first import of a process: the compiled extension needs torch's Python module, and the
+    package loads it itself."""
+    import subprocess
+    import sys
+    code = "import sys; sys.path.insert(0, %r); import deep_ep; print(deep_ep.ElasticBuffer.__name__)" % os.path.join(ROOT, "deepep-ascend_amd")
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-600:]
+    assert res.stdout.strip() == "ElasticBuffer"

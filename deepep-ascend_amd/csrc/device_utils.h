@@ -101,11 +101,33 @@ __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float
 #endif
 }
 
-// Maximum over each aligned group of 8 consecutive lanes (butterfly over lane xor 1, 2, 4).
+// Lane exchanges inside a row of 16 lanes as DPP operand modifiers (no LDS traffic, no address arithmetic).  All lanes
+// of the wavefront must be active.
+constexpr int kDppSwapNeighbours = 0xB1;     // quad_perm [1,0,3,2]: lane ^ 1
+constexpr int kDppSwapPairs = 0x4E;          // quad_perm [2,3,0,1]: lane ^ 2
+constexpr int kDppHalfMirror = 0x141;        // row_half_mirror: lane i of an aligned group of 8 reads lane 7 - i
+constexpr int kDppMirror = 0x140;            // row_mirror: lane i of a row of 16 reads lane 15 - i
+
+template <int kCtrl>
+__device__ __forceinline__ int dpp_read(int v) {
+    return __builtin_amdgcn_update_dpp(v, v, kCtrl, 0xf, 0xf, false);
+}
+
+// Maximum over each aligned group of 8 consecutive lanes: neighbours, pairs, then the two quads (whose lanes all hold
+// their quad's maximum by then) against each other.
 __device__ __forceinline__ float group8_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 1, kWaveSize));
-    v = fmaxf(v, __shfl_xor(v, 2, kWaveSize));
-    v = fmaxf(v, __shfl_xor(v, 4, kWaveSize));
+    v = fmaxf(v, __int_as_float(dpp_read<kDppSwapNeighbours>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_read<kDppSwapPairs>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_read<kDppHalfMirror>(__float_as_int(v))));
+    return v;
+}
+
+// Sum over each row of 16 lanes, left in every lane of the row.
+__device__ __forceinline__ int row16_sum(int v) {
+    v += dpp_read<kDppSwapNeighbours>(v);
+    v += dpp_read<kDppSwapPairs>(v);
+    v += dpp_read<kDppHalfMirror>(v);
+    v += dpp_read<kDppMirror>(v);
     return v;
 }
 

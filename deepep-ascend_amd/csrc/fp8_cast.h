@@ -31,9 +31,9 @@ enum class ScaleRule {
 __device__ __forceinline__ uint32_t magnitude_bits(float f) { return __float_as_uint(f) & 0x7fffffffu; }
 
 __device__ __forceinline__ uint32_t group8_max_bits(uint32_t v) {
-    v = max(v, uint32_t(__shfl_xor(int(v), 1, kWaveSize)));
-    v = max(v, uint32_t(__shfl_xor(int(v), 2, kWaveSize)));
-    v = max(v, uint32_t(__shfl_xor(int(v), 4, kWaveSize)));
+    v = max(v, uint32_t(dpp_read<kDppSwapNeighbours>(int(v))));
+    v = max(v, uint32_t(dpp_read<kDppSwapPairs>(int(v))));
+    v = max(v, uint32_t(dpp_read<kDppHalfMirror>(int(v))));
     return v;
 }
 

@@ -126,19 +126,27 @@ __global__ __launch_bounds__(kThreads) void ll_count_kernel(const LLDispatchPara
 constexpr int kMoveThreads = 256;
 constexpr int kMoveWaves = kMoveThreads / kWaveSize;
 
-// Loads one column tile (kPairs * 1024 channels) of token g: lane owns 16 consecutive channels per pair.
-template <int kPairs>
-__device__ __forceinline__ void ll_load_tile(const LLDispatchParams& p, int64_t g, int tile, int lane,
+// Loads one column tile (kPairs * 1024 channels) of token g: lane owns 16 consecutive channels per pair.  kClamped:
+// a pair past the end of the row loads the row's last 32 bytes instead of being skipped (no branch around the load;
+// what it brings is never stored).
+template <int kPairs, bool kClamped = false>
+__device__ __forceinline__ void ll_load_tile(const uint8_t* x, int hidden, int64_t g, int tile, int lane,
                                              vec16 (&in)[kPairs][2]) {
-    const uint8_t* src = p.x + g * (int64_t(p.H) * 2);
+    const uint8_t* src = x + g * (int64_t(hidden) * 2);
 #pragma unroll
     for (int q = 0; q < kPairs; ++q) {
         const int elem = (tile * kPairs + q) * 1024 + lane * 16;
-        in[q][0] = vec16{0, 0, 0, 0};
-        in[q][1] = vec16{0, 0, 0, 0};
-        if (elem < p.H) {
-            in[q][0] = load16_stream(src + int64_t(elem) * 2);
-            in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+        if constexpr (kClamped) {
+            const int at = min(elem, hidden - 16);
+            in[q][0] = load16_stream(src + int64_t(at) * 2);
+            in[q][1] = load16_stream(src + int64_t(at) * 2 + 16);
+        } else {
+            in[q][0] = vec16{0, 0, 0, 0};
+            in[q][1] = vec16{0, 0, 0, 0};
+            if (elem < hidden) {
+                in[q][0] = load16_stream(src + int64_t(elem) * 2);
+                in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
+            }
         }
     }
 }
@@ -157,6 +165,9 @@ __device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int64_t
     // optional shortcut for combine: the packed row of every (token, lane)
     if (tile == 0 && p.lane_slot != nullptr && lane < p.K) p.lane_slot[g * p.K + lane] = slot >= 0 ? le * rows_per_expert + slot : -1;
 
+    uint64_t dests = __ballot(slot >= 0);
+    if (dests == 0ull) return;              // nothing of this token stays on this rank: no cast either
+
     vec16 out[kPairs];
     float my_scale = 0.f;
     if constexpr (kFp8) {
@@ -172,7 +183,6 @@ __device__ __forceinline__ void ll_store_tile(const LLDispatchParams& p, int64_t
     const int num_groups = p.H / 128;
     const bool owns_scale = kFp8 && lane < kPairs * 8 && group < num_groups;
 
-    uint64_t dests = __ballot(slot >= 0);
     while (dests) {
         const int j = __builtin_ctzll(dests);
         dests &= dests - 1;
@@ -226,7 +236,7 @@ __global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchP
     if (t >= tokens_of_source(p, s)) return;
 
     vec16 in[kPairs][2];
-    ll_load_tile<kPairs>(p, g, tile, lane, in);
+    ll_load_tile<kPairs>(p.x, p.H, g, tile, lane, in);
 
     const int chunks_per_src = (p.src_token_stride + kLayoutChunk - 1) / kLayoutChunk;
     const int64_t chunk = int64_t(s) * chunks_per_src + t / kLayoutChunk;
@@ -241,11 +251,27 @@ __global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchP
     ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
 }
 
+// Sum over the wavefront of a small non-negative per-lane value (below 2^kBits): one ballot per bit, so the sum is
+// built in scalar registers with no cross-lane data movement.
+template <int kBits>
+__device__ __forceinline__ int wave_sum_small(int v) {
+    int total = 0;
+#pragma unroll
+    for (int b = 0; b < kBits; ++b) total += __popcll(__ballot((v >> b) & 1)) << b;
+    return total;
+}
+
 // Single-kernel path for decode-sized calls.  Every workgroup first rebuilds the complete routing picture in
 // LDS - one bit per (local expert, token), set from its own pass over all topk_idx rows (tens of KB, L2
 // resident) - so slots are prefix popcounts and no workgroup waits for another: no second launch, no ticket,
 // no global scan.  Workgroup 0 only publishes counts and per-source ranges; the wavefronts of the other
 // workgroups each move one (token, column tile).
+//
+// The kernel is bound by what a compute unit can issue, not by memory: the routing pass costs every workgroup a
+// dozen instructions per index entry.  So the index loads are the first thing on the memory pipeline (the pass can
+// start as soon as they are back), the payload loads queue up behind them and land while the pass runs, and the
+// pass itself is kept short: token ids advance by addition (no division per entry), 32-bit LDS atomics, range and
+// duplicate checks left to the wavefront that later moves the token.
 template <int kPairs, bool kFp8, int kFusedThreads>
 __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatchParams p, const int tiles) {
     constexpr int kFusedWaves = kFusedThreads / kWaveSize;
@@ -254,7 +280,7 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     const int total_tokens = p.S * p.src_token_stride;
     const int words = (total_tokens + 63) / 64;
 
-    // This wavefront's work item; its payload loads go out before the routing pass.
+    // This wavefront's work item.
     const unsigned work = blockIdx.x == 0 ? ~0u : wave_work_index(blockIdx.x - 1, kFusedWaves);
     const bool has_work = work < unsigned(total_tokens) * unsigned(tiles);
     const unsigned gu = has_work ? work / unsigned(tiles) : 0u;
@@ -263,51 +289,91 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     const int s = int(gu / unsigned(p.src_token_stride));
     const int t = int(gu - unsigned(s) * unsigned(p.src_token_stride));
     const bool live = has_work && t < tokens_of_source(p, s);
-    vec16 in[kPairs][2];
-    if (live) ll_load_tile<kPairs>(p, g, tile, lane, in);
-    // ... and so does the read of this token's own selections: behind the routing pass it would be one more trip to
-    // the L2 on the critical path
-    const int64_t own_raw = (live && lane < p.K) ? p.topk_idx[g * p.K + lane] : int64_t(-1);
 
-    for (int i = tid; i < p.E_l * words; i += kFusedThreads) bits[i] = 0ull;
-    __syncthreads();
-    // Pass over the whole index table: 16-byte loads (two entries), fully coalesced, all of a thread's loads
-    // in flight at once (addresses are clamped instead of predicated, so no load waits for another).  With
-    // random routing some lane of the wavefront holds a local expert in almost every step, so the "taken" side
-    // below runs every time: it is kept to a dozen instructions (no division, no returning atomic; range and
-    // duplicate checks are left to the wavefront that later moves the token).
+    // Pass over the whole index table: 16-byte loads (two entries), fully coalesced, a batch of a thread's loads in
+    // flight at once (addresses are clamped instead of predicated, so no load waits for another).  The first batch -
+    // for decode sizes the only one - goes out here, ahead of everything else.
+    // Everything up to the pass is straight-line code without a branch around any load: where control flow merges the
+    // compiler can no longer tell how many loads are younger than the one it waits for and waits for all of them - the
+    // pass would sit there until the payload had arrived.  So addresses are clamped instead of predicated (the launcher
+    // sends only calls with an aligned table of at least two entries here), and wavefronts without a work item load
+    // the tile of token 0 and drop it.
     const int total_entries = total_tokens * p.K;
-    const float rcp_k = 1.0f / float(p.K), rcp_stride = 1.0f / float(p.src_token_stride);
-    const bool ragged = p.num_tokens_per_src != nullptr;
-    auto note = [&](int f, uint32_t lo, uint32_t hi) {
-        const uint32_t le = lo - uint32_t(p.expert_begin);
-        if (hi != 0u || le >= uint32_t(p.E_l) || lo >= uint32_t(p.E)) return;   // no selection / another rank's expert
-        const int gg = small_div(f, rcp_k);
-        if (ragged) {
-            const int ss = small_div(gg, rcp_stride);
-            if (gg - ss * p.src_token_stride >= tokens_of_source(p, ss)) return;
-        }
-        atomicOr(reinterpret_cast<unsigned long long*>(&bits[int(le) * words + (gg >> 6)]), 1ull << (gg & 63));
-    };
-    const bool aligned16 = (reinterpret_cast<uintptr_t>(p.topk_idx) & 15) == 0;
-    const int pairs_total = aligned16 ? total_entries / 2 : 0;
+    const int pairs_total = total_entries / 2;
     const vec16* idx2 = reinterpret_cast<const vec16*>(p.topk_idx);
     constexpr int kBatch = 8;
+    for (int i = tid; i < p.E_l * words; i += kFusedThreads) bits[i] = 0ull;
+    __syncthreads();            // here, where no wavefront is held up by the memory pipeline yet: they arrive together
+    vec16 v[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) v[u] = idx2[min(tid + u * kFusedThreads, pairs_total - 1)];
+    // this token's own selections: behind the routing pass they would be one more trip to the L2 on the critical path
+    const int64_t own_loaded = p.topk_idx[g * p.K + min(lane, p.K - 1)];
+    // the payload tile: queued behind the index loads, in flight while the routing pass runs
+    vec16 in[kPairs][2];
+    ll_load_tile<kPairs, true>(p.x, p.H, g, tile, lane, in);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // An entry sets a bit iff it names a local expert: a negative or oversized id has a non-zero upper half or a lower
+    // half beyond every local id.  The atomic is not predicated: a lane without a hit ORs into a word of its own
+    // behind the table, which is cheaper than branching around a handful of instructions sixteen times.  Tokens past
+    // the end of a ragged source are masked out of the table afterwards.
+    const uint32_t row_bytes32 = uint32_t(words) * 8u;
+    const uint32_t spare = uint32_t(p.E_l) * row_bytes32 + uint32_t(lane) * 4u;     // byte offset of the lane's spare word
+    auto note = [&](uint32_t word_off, uint32_t bit, uint32_t lo, uint32_t hi) {
+        const uint32_t le = lo - uint32_t(p.expert_begin);
+        const bool hit = le < uint32_t(p.E_l) && hi == 0u;
+        const uint32_t off = hit ? __umul24(le, row_bytes32) + word_off : spare;
+        atomicOr(reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(bits) + off), bit);
+    };
+    const float rcp_k = 1.0f / float(p.K);
+    const bool even_k = (p.K & 1) == 0;
+    const float rcp_half_k = 2.0f / float(p.K);
     for (int q0 = tid; q0 < pairs_total; q0 += kFusedThreads * kBatch) {
-        vec16 v[kBatch];
+        if (q0 != tid) {
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) v[u] = idx2[min(q0 + u * kFusedThreads, pairs_total - 1)];
+            for (int u = 0; u < kBatch; ++u) v[u] = idx2[min(q0 + u * kFusedThreads, pairs_total - 1)];
+        }
+        if (even_k) {
+            // both entries of a pair belong to one token
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const int q = q0 + u * kFusedThreads;
-            const uint32_t dead = q < pairs_total ? 0u : 0xffffffffu;      // entries past the end read as "none"
-            note(2 * q, v[u].x, v[u].y | dead);
-            note(2 * q + 1, v[u].z, v[u].w | dead);
+            for (int u = 0; u < kBatch; ++u) {
+                const int q = q0 + u * kFusedThreads;
+                const int tok = small_div(q, rcp_half_k);
+                const uint32_t word_off = (uint32_t(tok) >> 3) & ~3u;
+                const uint32_t bit = q < pairs_total ? 1u << (tok & 31) : 0u;     // pairs past the end set nothing
+                note(word_off, bit, v[u].x, v[u].y);
+                note(word_off, bit, v[u].z, v[u].w);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int q = q0 + u * kFusedThreads;
+                const int tok0 = small_div(2 * q, rcp_k), tok1 = small_div(2 * q + 1, rcp_k);
+                const uint32_t live_pair = q < pairs_total ? 1u : 0u;
+                note((uint32_t(tok0) >> 3) & ~3u, live_pair << (tok0 & 31), v[u].x, v[u].y);
+                note((uint32_t(tok1) >> 3) & ~3u, live_pair << (tok1 & 31), v[u].z, v[u].w);
+            }
         }
     }
     for (int f = 2 * pairs_total + tid; f < total_entries; f += kFusedThreads) {
         const uint64_t raw = uint64_t(p.topk_idx[f]);
-        note(f, uint32_t(raw), uint32_t(raw >> 32));
+        const int tok = small_div(f, rcp_k);
+        note((uint32_t(tok) >> 3) & ~3u, 1u << (tok & 31), uint32_t(raw), uint32_t(raw >> 32));
+    }
+    if (p.num_tokens_per_src != nullptr) {
+        // ragged sources: clear the bits of the tokens a source does not have
+        __syncthreads();
+        for (int i = tid; i < p.E_l * words; i += kFusedThreads) {
+            const int first = (i % words) * 64, last = min(first + 64, total_tokens);
+            uint64_t keep = 0ull;
+            for (int ss = first / p.src_token_stride; ss * p.src_token_stride < last; ++ss) {
+                const int from = max(ss * p.src_token_stride, first) - first;
+                const int to = min(ss * p.src_token_stride + tokens_of_source(p, ss), last) - first;      // bits [from, to)
+                if (to > from) keep |= (to == 64 ? ~0ull : (1ull << to) - 1ull) & ~((1ull << from) - 1ull);
+            }
+            bits[i] &= keep;
+        }
     }
     __syncthreads();
 
@@ -321,9 +387,9 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
                 while (pos < end_pos) {
                     const int word = pos >> 6, lo = pos & 63;
                     const int take = min(64 - lo, end_pos - pos);
-                    uint64_t v = row[word] >> lo;
-                    if (take < 64) v &= (1ull << take) - 1ull;
-                    running += __popcll(v);
+                    uint64_t wv = row[word] >> lo;
+                    if (take < 64) wv &= (1ull << take) - 1ull;
+                    running += __popcll(wv);
                     pos += take;
                 }
                 p.packed_layout_range[int64_t(le) * p.R + p.src_rank_begin + ss] =
@@ -339,28 +405,31 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     }
     if (!live) return;
 
-    // rows of expert le that come from tokens [0, g): prefix popcount
-    auto rows_before = [&](int le, int gpos) {
-        const uint64_t* row = bits + le * words;
-        int n = 0;
-        for (int wd = 0; wd < (gpos >> 6); ++wd) n += __popcll(row[wd]);
-        if (gpos & 63) n += __popcll(row[gpos >> 6] & ((1ull << (gpos & 63)) - 1ull));
-        return n;
-    };
     int le = -1, slot = -1, flags = 0;
     if (lane < p.K) {
-        const int64_t raw = own_raw;
-        if (raw >= p.E) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
-        if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) {
-            le = int(raw) - p.expert_begin;
-            slot = rows_before(le, int(g));
-        }
+        const uint32_t lo = uint32_t(own_loaded), hi = uint32_t(uint64_t(own_loaded) >> 32);
+        if (int32_t(hi) > 0 || (hi == 0u && lo >= uint32_t(p.E))) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+        if (hi == 0u && lo - uint32_t(p.expert_begin) < uint32_t(p.E_l)) le = int(lo) - p.expert_begin;
     }
-    if (tile == 0) {
-        for (int j = 0; j < p.K; ++j) {
-            const int other = read_lane(le, j);
-            if (lane != j && le >= 0 && le == other) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
-        }
+    // Slot of a selection = rows of its expert that come from tokens [0, g): a prefix popcount over the expert's
+    // words, taken by the whole wavefront for one selection at a time (lane i looks at word i; at most 32 words, so
+    // the sum sits in the first two rows of 16 lanes).
+    const int own_word = int(g) >> 6;
+    const uint64_t own_below = lanes_below(int(g) & 63);
+    uint64_t pending = __ballot(le >= 0);
+    while (pending) {
+        const int j = __builtin_ctzll(pending);
+        pending &= pending - 1;
+        const int expert = read_lane(le, j);
+        const uint64_t* row = bits + expert * words;
+        uint64_t wv = lane <= own_word ? row[lane] : 0ull;
+        if (lane == own_word) wv &= own_below;
+        const int sums = row16_sum(__popcll(wv));
+        const int before = read_lane(sums, 0) + read_lane(sums, 16);
+        if (lane == j) slot = before;
+        if (__popcll(__ballot(le == expert)) > 1) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+    }
+    if (tile == 0 && __ballot(flags != 0) != 0ull) {
         if (flags != 0) atomicOr(p.status, flags);
     }
     ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
@@ -435,14 +504,14 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
     const int rows_per_expert = p.R * p.M;
     const int row_bytes = p.H * 2;
 
-    int le = -1, recorded = -1;
-    float w = 0.f;
-    if (lane < p.K) {
-        const int64_t raw = p.topk_idx[g * p.K + lane];
-        if (p.lane_slot != nullptr) recorded = p.lane_slot[g * p.K + lane];    // issued together with the index load
-        w = p.topk_weights[g * p.K + lane];
-        if (raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) le = int(raw) - p.expert_begin;
-    }
+    // Every lane loads (lanes past the top-k repeat the last selection): no branch around the three loads, which go
+    // out together.
+    const int64_t entry = g * p.K + min(lane, p.K - 1);
+    const int64_t raw = p.topk_idx[entry];
+    const int recorded = p.lane_slot != nullptr ? p.lane_slot[entry] : -1;
+    const float w = p.topk_weights[entry];
+    int le = -1;
+    if (lane < p.K && raw >= p.expert_begin && raw < p.expert_begin + p.E_l && raw < p.E) le = int(raw) - p.expert_begin;
 
     int row_of_lane = -1;
     if (p.lane_slot != nullptr) {
@@ -534,43 +603,45 @@ __global__ __launch_bounds__(kMoveThreads) void ll_combine_kernel(const LLCombin
         }
     } else {
         // Rows go in rounds of up to four: the loads of a round are all issued before its first multiply-add, so a
-        // token with many local lanes pays one trip to memory per four rows, not one per row.  The sum keeps lane order.
+        // token with many local lanes pays one trip to memory per four rows, not one per row (eight at a time would
+        // need registers that cost the residency decode-sized calls depend on).  The sum keeps lane order.
         constexpr int kRound = 4;
         while (srcs) {
-            const uint8_t* src[kRound];
+            int64_t row_off[kRound];
             float wj[kRound];
+            bool have[kRound];
 #pragma unroll
             for (int b = 0; b < kRound; ++b) {
-                src[b] = nullptr;
+                have[b] = srcs != 0ull;
+                row_off[b] = 0;
                 wj[b] = 0.f;
-                if (srcs) {
+                if (have[b]) {
                     const int j = __builtin_ctzll(srcs);
                     srcs &= srcs - 1;
-                    src[b] = p.x + (int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j)) * row_bytes;
+                    row_off[b] = (int64_t(read_lane(le, j)) * rows_per_expert + read_lane(row_of_lane, j)) * row_bytes;
                     wj[b] = read_lane(w, j);
                 }
             }
             vec16 v[kRound][kVecs];
 #pragma unroll
-            for (int b = 0; b < kRound; ++b)
+            for (int b = 0; b < kRound; ++b) {
+                if (!have[b]) continue;                    // wave-uniform
 #pragma unroll
                 for (int i = 0; i < kVecs; ++i) {
-                    const int off = (tile * kVecs + i) * 1024 + lane * 16;
-                    v[b][i] = vec16{0, 0, 0, 0};
-                    if (src[b] != nullptr && off < row_bytes) v[b][i] = load16_stream(src[b] + off);
+                    // a column past the end of the row reads the row's last 16 bytes instead (never accumulated)
+                    const int off = min((tile * kVecs + i) * 1024 + lane * 16, row_bytes - 16);
+                    v[b][i] = load16_stream(p.x + row_off[b] + off);
                 }
+            }
 #pragma unroll
             for (int b = 0; b < kRound; ++b) {
-                if (src[b] == nullptr) continue;           // wave-uniform: an absent row adds nothing, not 0 * weight
+                if (!have[b]) continue;                    // an absent row adds nothing, not 0 * weight
 #pragma unroll
                 for (int i = 0; i < kVecs; ++i) {
-                    const int off = (tile * kVecs + i) * 1024 + lane * 16;
-                    if (off < row_bytes) {
-                        acc[i][0] += bf16_lo(v[b][i].x) * wj[b]; acc[i][1] += bf16_hi(v[b][i].x) * wj[b];
-                        acc[i][2] += bf16_lo(v[b][i].y) * wj[b]; acc[i][3] += bf16_hi(v[b][i].y) * wj[b];
-                        acc[i][4] += bf16_lo(v[b][i].z) * wj[b]; acc[i][5] += bf16_hi(v[b][i].z) * wj[b];
-                        acc[i][6] += bf16_lo(v[b][i].w) * wj[b]; acc[i][7] += bf16_hi(v[b][i].w) * wj[b];
-                    }
+                    acc[i][0] += bf16_lo(v[b][i].x) * wj[b]; acc[i][1] += bf16_hi(v[b][i].x) * wj[b];
+                    acc[i][2] += bf16_lo(v[b][i].y) * wj[b]; acc[i][3] += bf16_hi(v[b][i].y) * wj[b];
+                    acc[i][4] += bf16_lo(v[b][i].z) * wj[b]; acc[i][5] += bf16_hi(v[b][i].z) * wj[b];
+                    acc[i][6] += bf16_lo(v[b][i].w) * wj[b]; acc[i][7] += bf16_hi(v[b][i].w) * wj[b];
                 }
             }
         }
@@ -633,8 +704,10 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
     if (p.S <= 0 || p.src_token_stride <= 0) return hipSuccess;
     // Decode-sized calls: one kernel, every workgroup derives the slots itself.
     const int64_t total_tokens = int64_t(p.S) * p.src_token_stride;
-    const size_t fused_lds = size_t(p.E_l) * ((total_tokens + 63) / 64) * sizeof(uint64_t);
-    if (total_tokens <= 2048 && fused_lds <= 32 * 1024 && !p.two_kernels) {
+    // the routing table of the single-kernel path, plus one spare 32-bit word per lane
+    const size_t fused_lds = size_t(p.E_l) * ((total_tokens + 63) / 64) * sizeof(uint64_t) + kWaveSize * sizeof(uint32_t);
+    const bool table_fits = (reinterpret_cast<uintptr_t>(p.topk_idx) & 15) == 0 && total_tokens * p.K >= 2 && p.H >= 16;
+    if (total_tokens <= 2048 && fused_lds <= 33 * 1024 && table_fits && !p.two_kernels) {
         const int threads = p.threads != 0 ? p.threads : 512;
         if (threads == 256) return launch_fused_by_width<256>(p, stream, fused_lds);
         if (threads == 1024) return launch_fused_by_width<1024>(p, stream, fused_lds);
@@ -656,8 +729,13 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
 hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream) {
     if (p.S <= 0 || p.src_token_stride <= 0) return hipSuccess;
     int vecs = p.vecs;
-    if (vecs != 1 && vecs != 2 && vecs != 4)
-        vecs = (p.H * 2 <= 1024 || int64_t(p.S) * p.src_token_stride <= 4096) ? 1 : 4;   // decode sizes: many small wavefronts
+    if (vecs != 1 && vecs != 2 && vecs != 4 && vecs != 7) {
+        // Decode-sized calls are over before a second round of workgroups could start: 2 KB per wavefront is the widest
+        // tile whose whole grid is resident at once (measured at 1024 tokens x 7168: 1 KB 8.4 us, 2 KB 7.9, 4 KB 9.2,
+        // 7 KB 9.3).  Large batches stream with 4 KB tiles.
+        const int64_t tokens = int64_t(p.S) * p.src_token_stride;
+        vecs = p.H * 2 <= 1024 ? 1 : tokens <= 4096 ? 2 : 4;
+    }
     if (p.use_logfmt) vecs = p.H % 1024 == 0 ? 2 : 1;                                     // one codec chunk per wavefront
     const int tiles = (p.H * 2 + vecs * 1024 - 1) / (vecs * 1024);
     const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
@@ -669,7 +747,8 @@ hipError_t launch_ll_combine(const LLCombineParams& p, hipStream_t stream) {
     }
     if (vecs == 1) hipLaunchKernelGGL(ll_combine_kernel<1>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
     else if (vecs == 2) hipLaunchKernelGGL(ll_combine_kernel<2>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
-    else hipLaunchKernelGGL(ll_combine_kernel<4>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    else if (vecs == 4) hipLaunchKernelGGL(ll_combine_kernel<4>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
+    else hipLaunchKernelGGL(ll_combine_kernel<7>, dim3(blocks), dim3(kMoveThreads), 0, stream, p, tiles);
     return hipGetLastError();
 }
 

@@ -84,7 +84,7 @@ typedef struct {
     int32_t ll_pairs;          /* low-latency dispatch: 1024-channel segments per wavefront (1, 2, 4) */
     int32_t ll_threads;        /* low-latency dispatch, single-kernel path: workgroup size (256, 512, 1024) */
     int32_t ll_two_kernels;    /* 1: low-latency dispatch always as count kernel + move kernel */
-    int32_t ll_combine_vecs;   /* low-latency combine: KB of row per wavefront (1, 2, 4) */
+    int32_t ll_combine_vecs;   /* low-latency combine: KB of row per wavefront (1, 2, 4, 7) */
     int32_t mover_spin_limit;  /* single-launch dispatch: how often a mover workgroup repeats a read of the layout its own
                                   launch is still computing before it gives up, stores nothing and sets
                                   DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT (0 = 2^22, seconds; 1 makes the first workgroups of a

@@ -59,7 +59,7 @@ def test_dispatch_and_combine_under_knob(knob):
 
 
 LL_KNOBS = [("ll_threads", 256), ("ll_threads", 1024), ("ll_pairs", 1), ("ll_pairs", 2), ("ll_two_kernels", 1),
-            ("ll_combine_vecs", 2), ("ll_combine_vecs", 4)]
+            ("ll_combine_vecs", 1), ("ll_combine_vecs", 2), ("ll_combine_vecs", 4), ("ll_combine_vecs", 7)]
 
 
 @pytest.mark.parametrize("knob", LL_KNOBS, indirect=True, ids=[f"{n}={v}" for n, v in LL_KNOBS])

@@ -164,7 +164,7 @@ public:
         const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(device_);
         torch::Tensor workspace = acquire_workspace(run, num_tokens, num_topk, num_experts);
 
-        torch::Tensor counts, psum_rank, psum_expert, num_unaligned, dst_slot;
+        torch::Tensor psum_rank, psum_expert, num_unaligned, dst_slot;
         std::optional<torch::Tensor> copied_topk_idx;
         {
             c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);      // allocations below belong to the run stream
@@ -179,12 +179,19 @@ public:
                 EP_HIP_HOST_ASSERT(dst_slot.dim() == 2 and dst_slot.size(0) == num_tokens and dst_slot.size(1) == num_topk and
                                    dst_slot.scalar_type() == torch::kInt32 and dst_slot.is_contiguous());
             } else {
-                counts = torch::empty({R + 2 * int64_t(num_experts)}, i32);     // one allocation, one D2H copy when syncing
-                psum_rank = counts.slice(0, 0, R);
-                psum_expert = counts.slice(0, R, R + num_experts);
-                num_unaligned = counts.slice(0, R + num_experts, R + 2 * int64_t(num_experts));
-                dst_slot = torch::empty({num_tokens, num_topk}, i32);
-                if (do_handle_copy) copied_topk_idx = torch::empty_like(topk_idx);
+                // what the handle keeps, in one allocation
+                TensorPack pack(device_);
+                const int i_rank = pack.add(torch::kInt32, {R});
+                const int i_expert = pack.add(torch::kInt32, {num_experts});
+                const int i_unaligned = pack.add(torch::kInt32, {num_experts});
+                const int i_slot = pack.add(torch::kInt32, {num_tokens, num_topk});
+                const int i_copy = do_handle_copy ? pack.add(torch::kInt64, {num_tokens, num_topk}) : -1;
+                pack.allocate();
+                psum_rank = pack.get(i_rank);
+                psum_expert = pack.get(i_expert);
+                num_unaligned = pack.get(i_unaligned);
+                dst_slot = pack.get(i_slot);
+                if (do_handle_copy) copied_topk_idx = pack.get(i_copy);
             }
         }
 
@@ -254,20 +261,25 @@ public:
             c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
             recv_x = torch::empty({num_allocated, hidden}, torch::TensorOptions().dtype(out_dtype).device(device_));
             recv_src_metadata = cached_mode ? *cached_recv_src_metadata : torch::empty({num_recv_tokens, num_topk + 2}, i32);
+            // what travels beside the payload (scales, indices, weights), in one allocation; the payload and the
+            // handle's metadata stay on their own, because callers keep them for different spans
+            TensorPack beside(device_);
+            int i_sf = -1, i_idx = -1, i_w = -1;
             if (sf_dtype.has_value()) {
                 if (not use_tma_aligned_col_major_sf) {
                     rsf_ts = num_sf_packs; rsf_hs = 1;
                 } else {
                     rsf_ts = 1; rsf_hs = align_up(num_allocated, 4);        // column-major, rows padded to 4 (csrc/elastic/buffer.hpp:1092-1101)
                 }
-                recv_sf = torch::empty_strided({num_allocated, num_sf_packs}, {rsf_ts, rsf_hs},
-                                               torch::TensorOptions().dtype(*sf_dtype).device(device_));
+                i_sf = beside.add(*sf_dtype, {num_allocated, num_sf_packs}, {rsf_ts, rsf_hs});
             }
-            if (not do_expand) recv_topk_idx = torch::empty({num_allocated, num_topk}, topk_idx.options());
-            if (topk_weights.has_value()) {
-                const auto f32 = torch::TensorOptions().dtype(torch::kFloat32).device(device_);
-                recv_topk_weights = do_expand ? torch::empty({num_allocated}, f32) : torch::empty({num_allocated, num_topk}, f32);
-            }
+            if (not do_expand) i_idx = beside.add(torch::kInt64, {num_allocated, num_topk});
+            if (topk_weights.has_value())
+                i_w = do_expand ? beside.add(torch::kFloat32, {num_allocated}) : beside.add(torch::kFloat32, {num_allocated, num_topk});
+            if (i_sf >= 0 or i_idx >= 0 or i_w >= 0) beside.allocate();
+            if (i_sf >= 0) recv_sf = beside.get(i_sf);
+            if (i_idx >= 0) recv_topk_idx = beside.get(i_idx);
+            if (i_w >= 0) recv_topk_weights = beside.get(i_w);
         }
 
         if (previous_event_before_epilogue.has_value()) stream_wait(run, *previous_event_before_epilogue);

@@ -404,19 +404,26 @@ public:
         if (ll_last_stream_ != run) stream_wait(run, ll_last_stream_);       // the low-latency workspace is shared too
         c10::hip::HIPStreamGuardMasqueradingAsCUDA on_run(run);
         const auto dev = torch::TensorOptions().device(device_);
-        torch::Tensor packed_recv_x = torch::empty({E_l, rows, H}, dev.dtype(use_fp8 ? torch::kFloat8_e4m3fn : torch::kBFloat16));
-        // The small outputs share one allocation (each torch allocation costs the host about a microsecond, which
-        // counts in a call of twenty): ranges first, for their 8-byte alignment.  The kernel writes every range,
-        // (begin 0, count 0) for source ranks that do not send in this call.
-        const int64_t n_range = int64_t(E_l) * R, n_info = int64_t(E_l) * rows, n_lane = int64_t(S) * T * K;
-        torch::Tensor small = torch::empty({2 * n_range + n_info + E_l + n_lane}, dev.dtype(torch::kInt32));
-        torch::Tensor packed_recv_layout_range = small.slice(0, 0, 2 * n_range).view(torch::kInt64).view({E_l, R});
-        torch::Tensor packed_recv_src_info = small.slice(0, 2 * n_range, 2 * n_range + n_info).view({E_l, rows});
-        torch::Tensor packed_recv_count = small.slice(0, 2 * n_range + n_info, 2 * n_range + n_info + E_l);
-        torch::Tensor lane_rows = small.slice(0, 2 * n_range + n_info + E_l, 2 * n_range + n_info + E_l + n_lane).view({int64_t(S) * T, K});
+        // Two allocations: the payload with its scales, and the small outputs (ranges first, for their 8-byte
+        // alignment).  The kernel writes every range, (begin 0, count 0) for source ranks that do not send in this call.
+        TensorPack payload(device_), small(device_);
+        const int i_x = payload.add(use_fp8 ? torch::kFloat8_e4m3fn : torch::kBFloat16, {E_l, rows, H});
+        int i_scales = -1;                                              // [E_l, rows, groups], column-major in the last two
+        if (use_fp8 and use_ue8m0) i_scales = payload.add(torch::kInt32, {E_l, rows, H / 512}, {int64_t(H / 512) * rows, 1, rows});
+        else if (use_fp8) i_scales = payload.add(torch::kFloat32, {E_l, rows, H / 128}, {int64_t(H / 128) * rows, 1, rows});
+        const int i_range = small.add(torch::kInt64, {E_l, R});
+        const int i_info = small.add(torch::kInt32, {E_l, rows});
+        const int i_count = small.add(torch::kInt32, {E_l});
+        const int i_lane = small.add(torch::kInt32, {int64_t(S) * T, K});
+        payload.allocate();
+        small.allocate();
+        torch::Tensor packed_recv_x = payload.get(i_x);
         std::optional<torch::Tensor> packed_recv_x_scales;
-        if (use_fp8 and use_ue8m0) packed_recv_x_scales = torch::empty({E_l, H / 512, rows}, dev.dtype(torch::kInt32)).transpose(1, 2);
-        else if (use_fp8) packed_recv_x_scales = torch::empty({E_l, H / 128, rows}, dev.dtype(torch::kFloat32)).transpose(1, 2);
+        if (i_scales >= 0) packed_recv_x_scales = payload.get(i_scales);
+        torch::Tensor packed_recv_layout_range = small.get(i_range);
+        torch::Tensor packed_recv_src_info = small.get(i_info);
+        torch::Tensor packed_recv_count = small.get(i_count);
+        torch::Tensor lane_rows = small.get(i_lane);
         if (T > 0) {
             const int64_t need = static_cast<int64_t>(deep_ep_hip_ll_workspace_bytes(S, T, K, E_l));
             if (not ll_workspace_.has_value() or ll_workspace_->numel() < need)

@@ -105,6 +105,61 @@ inline T* ptr_of(const std::optional<torch::Tensor>& t) {
     return t.has_value() ? static_cast<T*>(t->data_ptr()) : nullptr;
 }
 
+
+// Several output tensors of one call in one device allocation.  Every torch allocation costs the host about a
+// microsecond and every view that goes through the dispatcher a third of one, which counts in calls of ten to twenty:
+// the tensors are declared first, allocated together (each one 256-byte aligned), and then built directly on the shared
+// storage.  Tensors of one pack keep each other's memory alive, so a pack holds what lives and dies together.
+class TensorPack {
+public:
+    explicit TensorPack(const c10::Device& device) : device_(device) {}
+
+    // Declares a tensor (contiguous unless strides are given); returns its index for get().
+    int add(c10::ScalarType dtype, std::vector<int64_t> sizes, std::vector<int64_t> strides = {}) {
+        if (strides.empty()) {
+            strides.resize(sizes.size());
+            int64_t running = 1;
+            for (int i = static_cast<int>(sizes.size()) - 1; i >= 0; --i) {
+                strides[i] = running;
+                running *= std::max<int64_t>(sizes[i], 1);
+            }
+        }
+        int64_t span = 1;                                   // elements from the first to one past the last
+        for (size_t i = 0; i < sizes.size(); ++i) {
+            if (sizes[i] == 0) { span = 0; break; }
+            span += (sizes[i] - 1) * strides[i];
+        }
+        const int64_t bytes = span * static_cast<int64_t>(c10::elementSize(dtype));
+        entries_.push_back({dtype, std::move(sizes), std::move(strides), total_bytes_});
+        total_bytes_ = align_up(total_bytes_ + bytes, 256);
+        return static_cast<int>(entries_.size()) - 1;
+    }
+
+    // One allocation for everything declared so far (on the current stream of the caching allocator).
+    void allocate() {
+        blob_ = torch::empty({std::max<int64_t>(total_bytes_, 1)}, torch::TensorOptions().dtype(torch::kUInt8).device(device_));
+    }
+
+    torch::Tensor get(int index) const {
+        const Entry& e = entries_[static_cast<size_t>(index)];
+        auto impl = c10::make_intrusive<c10::TensorImpl>(c10::Storage(blob_.storage()), blob_.key_set(), c10::scalarTypeToTypeMeta(e.dtype));
+        impl->set_storage_offset((blob_.storage_offset() + e.byte_offset) / static_cast<int64_t>(c10::elementSize(e.dtype)));
+        impl->set_sizes_and_strides(e.sizes, e.strides);
+        return torch::Tensor(std::move(impl));
+    }
+
+private:
+    struct Entry {
+        c10::ScalarType dtype;
+        std::vector<int64_t> sizes, strides;
+        int64_t byte_offset;
+    };
+    c10::Device device_;
+    std::vector<Entry> entries_;
+    int64_t total_bytes_ = 0;
+    torch::Tensor blob_;
+};
+
 // A few (key tensor -> companion tensor) pairs a buffer remembers about handles it has produced.  The key is held
 // weakly and compared by identity, so an entry can only be found through the very tensor object the buffer returned:
 // a clone, a view or another tensor that happens to reuse the freed memory misses, and the caller falls back to

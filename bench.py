@@ -36,20 +36,20 @@ HBM_PEAK_GBS = 8000.0
 # the whole call (one kernel where the single launch applies, layout kernel + move kernel otherwise).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/bench_C3_hbm_counters.md
-    ("C3", "compact", "fp8", "dispatch"): 459112087,
-    ("C3", "compact", "fp8", "combine"): 751991270,
-    ("C3", "expanded", "fp8", "dispatch"): 1862350 + 613209199,
-    ("C3", "expanded", "fp8", "combine"): 1074424810,
-    ("C3", "compact", "bf16", "dispatch"): 1844575 + 755751935,
-    ("C3", "compact", "bf16", "combine"): 751995276,
+    ("C3", "compact", "fp8", "dispatch"): 459281822,
+    ("C3", "compact", "fp8", "combine"): 751991366,
+    ("C3", "expanded", "fp8", "dispatch"): 1862368 + 613156339,
+    ("C3", "expanded", "fp8", "combine"): 1074426190,
+    ("C3", "compact", "bf16", "dispatch"): 1844575 + 755717968,
+    ("C3", "compact", "bf16", "combine"): 751994813,
     # profiles/bench_C4_C2_hbm_counters.md
-    ("C4", "compact", "fp8", "dispatch"): 425536715,
-    ("C4", "compact", "fp8", "combine"): 690500049,
-    ("C2", "compact", "bf16", "dispatch"): 97408588,
-    ("C2", "compact", "bf16", "combine"): 96362183,
+    ("C4", "compact", "fp8", "dispatch"): 425752286,
+    ("C4", "compact", "fp8", "combine"): 690500110,
+    ("C2", "compact", "bf16", "dispatch"): 97414801,
+    ("C2", "compact", "bf16", "combine"): 96362205,
     # profiles/bench_C5_low_latency_hbm_counters.md
-    ("C5", "packed", "fp8", "ll_dispatch"): 23985225,
-    ("C5", "packed", "fp8", "ll_combine"): 30346393,
+    ("C5", "packed", "fp8", "ll_dispatch"): 23986102,
+    ("C5", "packed", "fp8", "ll_combine"): 30097556,
 }
 
 

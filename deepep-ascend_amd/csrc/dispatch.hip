@@ -1078,11 +1078,6 @@ static int device_attribute(hipDeviceAttribute_t attribute, std::atomic<int>* ca
     return n;
 }
 
-static int compute_units() {
-    static std::atomic<int> cached[64];
-    return device_attribute(hipDeviceAttributeMultiprocessorCount, cached, 256);
-}
-
 static int lds_bytes_per_cu() {
     static std::atomic<int> cached[64];
     return device_attribute(hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, cached, 160 * 1024);
@@ -1175,6 +1170,11 @@ hipError_t launch_cast(MoveParams p, hipStream_t stream) {
 }
 
 }  // namespace
+
+int compute_units() {
+    static std::atomic<int> cached[64];
+    return device_attribute(hipDeviceAttributeMultiprocessorCount, cached, 256);
+}
 
 // Column tile of a move launch: 1024-channel segments per wavefront for the fused cast, KB of row per wavefront for
 // the pass-through payloads.

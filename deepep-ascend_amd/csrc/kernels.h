@@ -288,6 +288,9 @@ struct LLDispatchParams {
     int pairs, threads, two_kernels;
 };
 
+// Compute units of the current device (asked once per device).
+int compute_units();
+
 hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream);
 
 struct LLCombineParams {

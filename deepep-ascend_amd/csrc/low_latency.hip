@@ -7,6 +7,8 @@
 // With every logical source resident in local HBM the send/receive phases and the RDMA staging
 // buffers disappear; slots come from a scan, so the fill order is deterministic: source rank
 // ascending, then token ascending (the reference fills in arrival order).
+#include <algorithm>
+
 #include "device_utils.h"
 #include "fp8_cast.h"
 #include "kernels.h"
@@ -272,23 +274,37 @@ __device__ __forceinline__ int wave_sum_small(int v) {
 // start as soon as they are back), the payload loads queue up behind them and land while the pass runs, and the
 // pass itself is kept short: token ids advance by addition (no division per entry), 32-bit LDS atomics, range and
 // duplicate checks left to the wavefront that later moves the token.
-template <int kPairs, bool kFp8, int kFusedThreads>
+template <int kPairs, bool kFp8, int kFusedThreads, bool kSeveralItems>
 __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatchParams p, const int tiles) {
     constexpr int kFusedWaves = kFusedThreads / kWaveSize;
     extern __shared__ uint64_t bits[];          // [E_l][words], bit g of row le: token g selects local expert le
+    // Every argument the first loads depend on is asked for in one go, up front: the wavefront starts with one trip to
+    // memory for its arguments, not with one per group of them as they come into use.
+    asm volatile("" ::"s"(p.topk_idx), "s"(p.x), "s"(p.num_tokens_per_src), "s"(p.S), "s"(p.src_token_stride), "s"(p.K), "s"(p.H),
+                 "s"(p.E_l), "s"(tiles));
     const int tid = threadIdx.x, lane = tid & 63;
     const int total_tokens = p.S * p.src_token_stride;
     const int words = (total_tokens + 63) / 64;
 
-    // This wavefront's work item.
-    const unsigned work = blockIdx.x == 0 ? ~0u : wave_work_index(blockIdx.x - 1, kFusedWaves);
-    const bool has_work = work < unsigned(total_tokens) * unsigned(tiles);
-    const unsigned gu = has_work ? work / unsigned(tiles) : 0u;
-    const int64_t g = gu;
-    const int tile = has_work ? int(work - gu * unsigned(tiles)) : 0;
-    const int s = int(gu / unsigned(p.src_token_stride));
-    const int t = int(gu - unsigned(s) * unsigned(p.src_token_stride));
-    const bool live = has_work && t < tokens_of_source(p, s);
+    // This wavefront's first work item; a call with more items than the grid has wavefronts gives every wavefront
+    // several, `item_stride` apart (the grid is held to one workgroup per compute unit, so that the routing pass below
+    // is paid once per compute unit however many tokens there are).
+    const unsigned num_items = unsigned(total_tokens) * unsigned(tiles);
+    const unsigned item_stride = (gridDim.x - 1) * unsigned(kFusedWaves);
+    unsigned work = blockIdx.x == 0 ? ~0u : wave_work_index(blockIdx.x - 1, kFusedWaves);
+    bool has_work = work < num_items;
+    unsigned gu = has_work ? work / unsigned(tiles) : 0u;
+    int64_t g = gu;
+    int tile = has_work ? int(work - gu * unsigned(tiles)) : 0;
+    // token id within its source, and whether the source has that many tokens: worked out here, in the shadow of the
+    // loads, not behind the routing pass
+    auto place_of = [&](unsigned token, int& t_out) {
+        const int src = int(token / unsigned(p.src_token_stride));
+        t_out = int(token - unsigned(src) * unsigned(p.src_token_stride));
+        return t_out < tokens_of_source(p, src);
+    };
+    int t = 0;
+    bool live = place_of(gu, t) && has_work;
 
     // Pass over the whole index table: 16-byte loads (two entries), fully coalesced, a batch of a thread's loads in
     // flight at once (addresses are clamped instead of predicated, so no load waits for another).  The first batch -
@@ -308,7 +324,7 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) v[u] = idx2[min(tid + u * kFusedThreads, pairs_total - 1)];
     // this token's own selections: behind the routing pass they would be one more trip to the L2 on the critical path
-    const int64_t own_loaded = p.topk_idx[g * p.K + min(lane, p.K - 1)];
+    int64_t own_loaded = p.topk_idx[g * p.K + min(lane, p.K - 1)];
     // the payload tile: queued behind the index loads, in flight while the routing pass runs
     vec16 in[kPairs][2];
     ll_load_tile<kPairs, true>(p.x, p.H, g, tile, lane, in);
@@ -403,36 +419,78 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
         }
         return;
     }
-    if (!live) return;
+    const int own_lane = min(lane, p.K - 1);
+    while (has_work) {
+        // Where this item's rows go: needs the routing table and the token's own selections, not the payload, which
+        // may still be on its way.
+        int le = -1, slot = -1, flags = 0;
+        if (live && lane < p.K) {
+            const uint32_t lo = uint32_t(own_loaded), hi = uint32_t(uint64_t(own_loaded) >> 32);
+            if (int32_t(hi) > 0 || (hi == 0u && lo >= uint32_t(p.E))) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
+            if (hi == 0u && lo - uint32_t(p.expert_begin) < uint32_t(p.E_l)) le = int(lo) - p.expert_begin;
+        }
+        // Slot of a selection = rows of its expert that come from tokens [0, g): a prefix popcount over the expert's
+        // words, taken by the whole wavefront for one selection at a time (lane i looks at word i; at most 64 words,
+        // summed in rows of 16 lanes).
+        const int own_word = int(g) >> 6;
+        const uint64_t own_below = lanes_below(int(g) & 63);
+        uint64_t pending = __ballot(le >= 0);
+        while (pending) {
+            const int j = __builtin_ctzll(pending);
+            pending &= pending - 1;
+            const int expert = read_lane(le, j);
+            const uint64_t* row = bits + expert * words;
+            uint64_t wv = lane <= own_word ? row[lane] : 0ull;
+            if (lane == own_word) wv &= own_below;
+            const int sums = row16_sum(__popcll(wv));
+            const int before = read_lane(sums, 0) + read_lane(sums, 16) + read_lane(sums, 32) + read_lane(sums, 48);
+            if (lane == j) slot = before;
+            if (__popcll(__ballot(le == expert)) > 1) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
+        }
+        if (tile == 0 && __ballot(flags != 0) != 0ull) {
+            if (flags != 0) atomicOr(p.status, flags);
+        }
 
-    int le = -1, slot = -1, flags = 0;
-    if (lane < p.K) {
-        const uint32_t lo = uint32_t(own_loaded), hi = uint32_t(uint64_t(own_loaded) >> 32);
-        if (int32_t(hi) > 0 || (hi == 0u && lo >= uint32_t(p.E))) flags |= DEEP_EP_HIP_STATUS_EXPERT_OUT_OF_RANGE;
-        if (hi == 0u && lo - uint32_t(p.expert_begin) < uint32_t(p.E_l)) le = int(lo) - p.expert_begin;
+        // This item's tile has to be in its registers before the next one is requested: the request below sits in a
+        // branch, and behind a branch the compiler waits for every outstanding load at once - this item would wait for
+        // the next item's tile.
+        if constexpr (kSeveralItems) {
+#pragma unroll
+            for (int q = 0; q < kPairs; ++q)
+                asm volatile("" : "+v"(in[q][0].x), "+v"(in[q][0].y), "+v"(in[q][0].z), "+v"(in[q][0].w),
+                                  "+v"(in[q][1].x), "+v"(in[q][1].y), "+v"(in[q][1].z), "+v"(in[q][1].w));
+        }
+        // the next item's tile and selections are requested before this item is converted and stored
+        const unsigned next_work = work + item_stride;
+        const bool has_next = kSeveralItems && next_work < num_items;      // decode sizes: one item per wavefront, no loop
+        const unsigned next_gu = has_next ? next_work / unsigned(tiles) : 0u;
+        const int next_tile = has_next ? int(next_work - next_gu * unsigned(tiles)) : 0;
+        vec16 next_in[kPairs][2];
+        int64_t next_own = -1;
+        int next_t = 0;
+        bool next_live = false;
+        if (has_next) {
+            next_own = p.topk_idx[int64_t(next_gu) * p.K + own_lane];
+            ll_load_tile<kPairs, true>(p.x, p.H, int64_t(next_gu), next_tile, lane, next_in);
+            next_live = place_of(next_gu, next_t);
+        }
+
+        if (live) ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
+
+        has_work = has_next;
+        work = next_work;
+        gu = next_gu;
+        g = next_gu;
+        tile = next_tile;
+        own_loaded = next_own;
+        t = next_t;
+        live = next_live;
+#pragma unroll
+        for (int q = 0; q < kPairs; ++q) {
+            in[q][0] = next_in[q][0];
+            in[q][1] = next_in[q][1];
+        }
     }
-    // Slot of a selection = rows of its expert that come from tokens [0, g): a prefix popcount over the expert's
-    // words, taken by the whole wavefront for one selection at a time (lane i looks at word i; at most 32 words, so
-    // the sum sits in the first two rows of 16 lanes).
-    const int own_word = int(g) >> 6;
-    const uint64_t own_below = lanes_below(int(g) & 63);
-    uint64_t pending = __ballot(le >= 0);
-    while (pending) {
-        const int j = __builtin_ctzll(pending);
-        pending &= pending - 1;
-        const int expert = read_lane(le, j);
-        const uint64_t* row = bits + expert * words;
-        uint64_t wv = lane <= own_word ? row[lane] : 0ull;
-        if (lane == own_word) wv &= own_below;
-        const int sums = row16_sum(__popcll(wv));
-        const int before = read_lane(sums, 0) + read_lane(sums, 16);
-        if (lane == j) slot = before;
-        if (__popcll(__ballot(le == expert)) > 1) flags |= DEEP_EP_HIP_STATUS_DUPLICATE_EXPERT;
-    }
-    if (tile == 0 && __ballot(flags != 0) != 0ull) {
-        if (flags != 0) atomicOr(p.status, flags);
-    }
-    ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
 }
 
 // ---- LogFMT-10, the codec the reference puts the rows of a low-latency combine through on the wire
@@ -489,6 +547,9 @@ __device__ __forceinline__ void logfmt_round_trip(float (&val)[8], const float (
 // of the codec (kVecs = 2 for hidden % 1024 == 0, else 1).
 template <int kVecs, bool kLogFmt = false, int kBlockThreads = kMoveThreads>
 __global__ __launch_bounds__(kBlockThreads) void ll_combine_kernel(const LLCombineParams p, const int tiles) {
+    // all arguments the first loads depend on in one trip to memory (see ll_fused_kernel)
+    asm volatile("" ::"s"(p.topk_idx), "s"(p.topk_weights), "s"(p.lane_slot), "s"(p.x), "s"(p.out), "s"(p.num_tokens_per_src),
+                 "s"(p.S), "s"(p.src_token_stride), "s"(p.K), "s"(p.H), "s"(p.E_l), "s"(p.expert_begin), "s"(p.R), "s"(p.M), "s"(tiles));
     const int lane = threadIdx.x & 63;
     const unsigned work = wave_work_index(blockIdx.x, kBlockThreads / kWaveSize);
     if (work >= unsigned(p.S) * unsigned(p.src_token_stride) * unsigned(tiles)) return;
@@ -679,11 +740,16 @@ hipError_t launch_fused(const LLDispatchParams& p, hipStream_t stream, size_t ld
     constexpr int kFusedWaves = kFusedThreads / kWaveSize;
     const int tiles = (p.H + kPairs * 1024 - 1) / (kPairs * 1024);
     const int64_t waves = int64_t(p.S) * p.src_token_stride * tiles;
-    const unsigned blocks = unsigned((waves + kFusedWaves - 1) / kFusedWaves) + 1;   // workgroup 0 publishes only
-    if (p.use_fp8)
-        hipLaunchKernelGGL((ll_fused_kernel<kPairs, true, kFusedThreads>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
-    else
-        hipLaunchKernelGGL((ll_fused_kernel<kPairs, false, kFusedThreads>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+    // one workgroup per compute unit at most (its wavefronts loop over the work items), plus workgroup 0, which publishes only
+    const unsigned blocks = unsigned(std::min<int64_t>((waves + kFusedWaves - 1) / kFusedWaves, compute_units())) + 1;
+    const bool several = waves > int64_t(blocks - 1) * kFusedWaves;
+    if (p.use_fp8) {
+        if (several) hipLaunchKernelGGL((ll_fused_kernel<kPairs, true, kFusedThreads, true>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+        else hipLaunchKernelGGL((ll_fused_kernel<kPairs, true, kFusedThreads, false>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+    } else {
+        if (several) hipLaunchKernelGGL((ll_fused_kernel<kPairs, false, kFusedThreads, true>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+        else hipLaunchKernelGGL((ll_fused_kernel<kPairs, false, kFusedThreads, false>), dim3(blocks), dim3(kFusedThreads), lds, stream, p, tiles);
+    }
     return hipGetLastError();
 }
 
@@ -707,7 +773,7 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
     // the routing table of the single-kernel path, plus one spare 32-bit word per lane
     const size_t fused_lds = size_t(p.E_l) * ((total_tokens + 63) / 64) * sizeof(uint64_t) + kWaveSize * sizeof(uint32_t);
     const bool table_fits = (reinterpret_cast<uintptr_t>(p.topk_idx) & 15) == 0 && total_tokens * p.K >= 2 && p.H >= 16;
-    if (total_tokens <= 2048 && fused_lds <= 33 * 1024 && table_fits && !p.two_kernels) {
+    if (total_tokens <= 4096 && fused_lds <= 33 * 1024 && table_fits && !p.two_kernels) {
         const int threads = p.threads != 0 ? p.threads : 512;
         if (threads == 256) return launch_fused_by_width<256>(p, stream, fused_lds);
         if (threads == 1024) return launch_fused_by_width<1024>(p, stream, fused_lds);

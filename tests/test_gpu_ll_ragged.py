@@ -24,8 +24,9 @@ def _ragged_case(R, stride, counts, H, E, K, seed):
     (4, 128, (128, 0, 77, 1), 1024, 32, 8, 128, True),             # single kernel, even top-k
     (4, 100, (3, 100, 64, 65), 512, 16, 3, 100, False),            # single kernel, odd top-k, BF16
     (8, 250, (250, 249, 0, 0, 130, 1, 64, 200), 256, 64, 6, 252, True),   # 2000 slots: two words per source boundary
-    (2, 1500, (1499, 700), 256, 16, 4, 1500, True),                # count + move kernels
-], ids=["k8", "k3_bf16", "eight_sources", "two_kernels"])
+    (2, 1500, (1499, 700), 256, 16, 4, 1500, True),                # single kernel, several work items per wavefront
+    (2, 2200, (2199, 900), 256, 16, 4, 2200, True),                # count + move kernels
+], ids=["k8", "k3_bf16", "eight_sources", "several_items", "two_kernels"])
 def test_ragged_sources_match_the_oracle(R, stride, counts, H, E, K, M, use_fp8):
     from deep_ep import _abi
     torch.cuda.set_device(0)

@@ -16,7 +16,8 @@ def _ranges(layout_range):
 
 @pytest.mark.parametrize("R,T,H,E,K,M", [(8, 128, 7168, 256, 8, 128), (2, 40, 1024, 8, 2, 64), (4, 300, 2048, 32, 6, 300),
                                          (1, 17, 512, 4, 3, 20),
-                                         (2, 1500, 256, 16, 9, 1500),      # too many tokens for the single-kernel path
+                                         (2, 1500, 256, 16, 9, 1500),      # single kernel, several work items per wavefront
+                                         (2, 2300, 256, 16, 9, 2300),      # too many tokens for the single-kernel path
                                          (4, 200, 512, 64, 12, 256)])
 @pytest.mark.parametrize("use_fp8", [True, False])
 def test_ll_stacked_sources(R, T, H, E, K, M, use_fp8):

@@ -103,7 +103,7 @@ def _draw_low_latency(seed):
     R = rnd.choice([1, 2, 3, 4, 8])
     E = R * rnd.choice([1, 2, 4, 8, 16])
     K = rnd.randint(1, min(E, rnd.choice([2, 4, 8, 9])))
-    T = rnd.choice([1, 3, 17, 64, 128, 200, 700, 2100])             # 2100 x R tokens: beyond the single-kernel path
+    T = rnd.choice([1, 3, 17, 64, 128, 200, 700, 2100])             # 2100 x R tokens: several work items per wavefront, or beyond the single-kernel path
     ue8m0 = rnd.random() < 0.25
     H = 512 * rnd.randint(1, 4) if ue8m0 else 128 * rnd.randint(1, 16)
     M = (T + rnd.choice([0, 5, 64]) + 3) // 4 * 4                    # rows per expert (R * M) must be a multiple of 4

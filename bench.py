@@ -48,8 +48,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("C2", "compact", "bf16", "dispatch"): 97414801,
     ("C2", "compact", "bf16", "combine"): 96362205,
     # profiles/bench_C5_low_latency_hbm_counters.md
-    ("C5", "packed", "fp8", "ll_dispatch"): 23977605,
-    ("C5", "packed", "fp8", "ll_combine"): 30424088,
+    ("C5", "packed", "fp8", "ll_dispatch"): 23993245,
+    ("C5", "packed", "fp8", "ll_combine"): 30425179,
 }
 
 

@@ -253,26 +253,17 @@ __global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchP
     ll_store_tile<kPairs, kFp8>(p, g, tile, lane, t, le, slot, in);
 }
 
-// Sum over the wavefront of a small non-negative per-lane value (below 2^kBits): one ballot per bit, so the sum is
-// built in scalar registers with no cross-lane data movement.
-template <int kBits>
-__device__ __forceinline__ int wave_sum_small(int v) {
-    int total = 0;
-#pragma unroll
-    for (int b = 0; b < kBits; ++b) total += __popcll(__ballot((v >> b) & 1)) << b;
-    return total;
-}
-
 // Single-kernel path for decode-sized calls.  Every workgroup first rebuilds the complete routing picture in
 // LDS - one bit per (local expert, token), set from its own pass over all topk_idx rows (tens of KB, L2
 // resident) - so slots are prefix popcounts and no workgroup waits for another: no second launch, no ticket,
 // no global scan.  Workgroup 0 only publishes counts and per-source ranges; the wavefronts of the other
-// workgroups each move one (token, column tile).
+// workgroups move (token, column tile) items: one each at decode sizes, several when the call has more items than
+// one workgroup per compute unit can take (kSeveralItems).
 //
 // The kernel is bound by what a compute unit can issue, not by memory: the routing pass costs every workgroup a
 // dozen instructions per index entry.  So the index loads are the first thing on the memory pipeline (the pass can
 // start as soon as they are back), the payload loads queue up behind them and land while the pass runs, and the
-// pass itself is kept short: token ids advance by addition (no division per entry), 32-bit LDS atomics, range and
+// pass itself is kept short: one token id per pair of entries, unpredicated 32-bit LDS atomics, range and
 // duplicate checks left to the wavefront that later moves the token.
 template <int kPairs, bool kFp8, int kFusedThreads, bool kSeveralItems>
 __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatchParams p, const int tiles) {

@@ -260,8 +260,8 @@ __global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchP
 // workgroups move (token, column tile) items: one each at decode sizes, several when the call has more items than
 // one workgroup per compute unit can take (kSeveralItems).
 //
-// The kernel is bound by what a compute unit can issue, not by memory: the routing pass costs every workgroup a
-// dozen instructions per index entry.  So the index loads are the first thing on the memory pipeline (the pass can
+// The kernel is bound by the chain of dependent phases of one wavefront, not by memory bandwidth: the routing pass alone
+// costs every workgroup a dozen instructions per index entry.  So the index loads are the first thing on the memory pipeline (the pass can
 // start as soon as they are back), the payload loads queue up behind them and land while the pass runs, and the
 // pass itself is kept short: one token id per pair of entries, unpredicated 32-bit LDS atomics, range and
 // duplicate checks left to the wavefront that later moves the token.

@@ -66,6 +66,18 @@ class Buffer:
         (deep_ep/buffers/legacy.py:538-551)."""
         self.runtime.clean_low_latency_buffer(num_max_dispatch_tokens_per_rank, hidden, num_experts)
 
+    # ---- mask buffers of the shrink mode (deep_ep/buffers/legacy.py:672-698): a rank is masked when it stops answering.
+    # On one GPU every logical rank lives in the calling process and cannot time out, so no rank is ever masked.
+    def low_latency_update_mask_buffer(self, rank_to_mask: int, mask: bool = False) -> None:
+        if mask:
+            raise NotImplementedError('the HIP backend has no peers to mask: every logical rank runs on this GPU')
+
+    def low_latency_query_mask_buffer(self, mask_status: torch.Tensor) -> None:
+        mask_status.zero_()
+
+    def low_latency_clean_mask_buffer(self) -> None:
+        pass
+
     def internode_dispatch(self, *args, **kwargs):
         return self.runtime.internode_dispatch(*args, **kwargs)        # raises NotImplementedError
 

@@ -193,3 +193,16 @@ def test_low_latency_combine_with_logfmt(hidden):
     assert _calc_diff(out_q.cpu(), out_x.cpu()) > 1e-9, "the codec did nothing"
     with pytest.raises(RuntimeError):
         buf.low_latency_combine(y.cuda(), idx.cuda(), w.cuda(), handle, use_logfmt=True, zero_copy=True)
+
+
+def test_mask_buffer_calls_of_the_reference_surface():
+    """deep_ep/buffers/legacy.py:672-698: on one GPU no logical rank can stop answering, so no rank is ever masked."""
+    import deep_ep
+    buf = deep_ep.Buffer(deep_ep.LogicalGroup(0, 4), low_latency_mode=True)
+    status = torch.full((4,), 7, dtype=torch.int32, device="cuda")
+    buf.low_latency_query_mask_buffer(status)
+    assert status.tolist() == [0, 0, 0, 0]
+    buf.low_latency_update_mask_buffer(2, False)
+    buf.low_latency_clean_mask_buffer()
+    with pytest.raises(NotImplementedError):
+        buf.low_latency_update_mask_buffer(2, True)

@@ -84,6 +84,14 @@ class EPHandle:
         assert self.topk_idx is not None, "a handle always carries the routing it was built from"
         self.cached_recv_src_metadata_before_sort = None        # an instance attribute, as in the reference
 
+    def deterministic_sort(self, do_cpu_sync: bool, is_cached_dispatch: bool, recv_x: torch.Tensor,
+                           recv_sf: Optional[torch.Tensor], recv_topk_idx: Optional[torch.Tensor],
+                           recv_topk_weights: Optional[torch.Tensor], channel_linked_list: Optional[torch.Tensor]) -> None:
+        """The reference sorts what it received by source token to undo its arrival order
+        (deep_ep/buffers/elastic.py:115-207).  Here rows are placed by a scan, in source-token order inside every
+        bucket and every expert region, so the sorted order is the order the tensors already have: nothing moves."""
+        return None
+
     def layout_fields(self) -> tuple:
         """The ten values a cached dispatch hands back to the runtime, in the runtime's argument order."""
         return (self.num_recv_tokens, self.num_expanded_tokens, self.num_recv_tokens_per_expert_list,

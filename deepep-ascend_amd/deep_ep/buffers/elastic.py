@@ -177,6 +177,11 @@ class ElasticBuffer:
     def get_logical_domain_size(self) -> Tuple[int, int]:
         return self.runtime.get_logical_domain_size()
 
+    def get_theoretical_num_qps(self, num_sms: int) -> int:
+        """RDMA queue pairs the reference would recommend (deep_ep/buffers/elastic.py:1371-1389): nothing here crosses
+        a network, so none."""
+        return 0
+
     def get_theoretical_num_sms(self, num_experts: int, num_topk: int, *args, **kwargs) -> int:
         """The routing kernels are bandwidth bound and always launched over the whole GPU."""
         return torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count

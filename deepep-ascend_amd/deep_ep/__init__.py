@@ -7,7 +7,19 @@ from .buffers.elastic import ElasticBuffer, EPHandle, LogicalGroup
 from .buffers.legacy import Buffer
 from .utils.event import EventOverlap
 
+
+def get_physical_domain_size(group):
+    """(RDMA ranks, scale-up ranks) of a group, deep_ep/utils/envs.py:277-295: every logical rank shares this GPU."""
+    return 1, group.size()
+
+
+def get_logical_domain_size(group, allow_hybrid_mode: bool = False):
+    """(scale-out ranks, scale-up ranks), deep_ep/utils/envs.py:298-320; the hybrid (scale-out) mode does not exist here."""
+    if allow_hybrid_mode:
+        raise NotImplementedError("the HIP backend has no hybrid (scale-out) mode")
+    return 1, group.size()
+
 __version__ = "2.0.0+hip"
 
 __all__ = ["ElasticBuffer", "EPHandle", "EventOverlap", "EventHandle", "Buffer", "Config", "LogicalGroup", "topk_idx_t",
-           "tuning", "__version__"]
+           "tuning", "get_physical_domain_size", "get_logical_domain_size", "__version__"]

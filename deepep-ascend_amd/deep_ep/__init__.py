@@ -13,11 +13,11 @@ def get_physical_domain_size(group):
     return 1, group.size()
 
 
-def get_logical_domain_size(group, allow_hybrid_mode: bool = False):
-    """(scale-out ranks, scale-up ranks), deep_ep/utils/envs.py:298-320; the hybrid (scale-out) mode does not exist here."""
-    if allow_hybrid_mode:
-        raise NotImplementedError("the HIP backend has no hybrid (scale-out) mode")
+def get_logical_domain_size(group, allow_hybrid_mode: bool = True):
+    """(scale-out ranks, scale-up ranks), deep_ep/utils/envs.py:298-320: one scale-out domain, whether or not the hybrid
+    mode is allowed, as for a single node in the reference."""
     return 1, group.size()
+
 
 __version__ = "2.0.0+hip"
 

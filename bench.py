@@ -471,6 +471,8 @@ def main():
     x_source = x.clone()
     dist["dispatch_after_input_written"] = distribution(full_dispatch, k, False, before=lambda: x.copy_(x_source))
     del x_source
+    # ... and written in place (what a normalisation leaves behind: no second tensor competes for the cache)
+    dist["dispatch_after_input_rewritten_in_place"] = distribution(full_dispatch, k, False, before=lambda: x.mul_(1.0))
 
     def gbs(nbytes, us):
         return nbytes / us * 1e-3

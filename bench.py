@@ -342,6 +342,8 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--ll-batch-sweep", action="store_true",
+                    help="with --workload C5: also time the low-latency kernels at 64 to 512 tokens per rank")
     ap.add_argument("--expanded", action="store_true", help="expert-major (expanded) receive layout")
     ap.add_argument("--bf16", action="store_true", help="BF16 dispatch instead of the fused FP8 cast")
     ap.add_argument("--launches", type=int, default=0, choices=[0, 1, 2],
@@ -586,8 +588,10 @@ class LowLatencyCalls:
     Buffers allocated once, launches straight through the C ABI."""
     R, T, H, E, K, M = 8, 128, 7168, 256, 8, 128
 
-    def __init__(self, torch, rc, _abi, dev):
+    def __init__(self, torch, rc, _abi, dev, tokens_per_rank=None, two_kernels=False):
         self.torch, self._abi = torch, _abi
+        if tokens_per_rank is not None:
+            self.T = self.M = tokens_per_rank
         R, T, H, E, K, M = self.R, self.T, self.H, self.E, self.K, self.M
         E_l, rows = E // R, R * M
         self.cpu_inputs = x_cpu, idx_cpu, w_cpu = rc.c5_sources(seed=0, R=R, T=T, H=H, E=E, K=K)
@@ -614,6 +618,8 @@ class LowLatencyCalls:
         d.lane_rows = lane_rows.data_ptr()
         d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
         d.tuning = _abi.Tuning.from_env()
+        if two_kernels:
+            d.tuning.ll_two_kernels = 1
         c = self.c = _abi.LLCombineArgs()
         c.num_src_ranks, c.src_rank_begin, c.src_token_stride = R, 0, T
         c.hidden, c.num_topk, c.num_experts, c.expert_begin, c.num_local_experts, c.num_ranks = H, K, E, 0, E_l, R
@@ -658,6 +664,21 @@ def bench_low_latency(args, torch, rc, _abi, dev):
     step_us = ll.loop_us(ll.step, args.steps)
     d_us, c_us = ll.loop_us(ll.dispatch, max(args.steps, 20)), ll.loop_us(ll.combine, max(args.steps, 20))
     d_bytes, c_bytes = ll.dispatch_bytes, ll.combine_bytes
+    sweep = None
+    if args.ll_batch_sweep:
+        # other batch sizes of the same shape: the single-kernel dispatch (one item per wavefront up to 128 tokens per
+        # rank here, several beyond) against the counting + move kernels, and the combine
+        sweep = {}
+        for t in (64, 128, 192, 256, 384, 512):
+            one, two = LowLatencyCalls(torch, rc, _abi, dev, t), LowLatencyCalls(torch, rc, _abi, dev, t, two_kernels=True)
+            for calls in (one, two):
+                for _ in range(5):
+                    calls.step()
+            torch.cuda.synchronize()
+            sweep[f"{R}x{t}"] = {"dispatch_us": round(one.loop_us(one.dispatch, 50), 2),
+                                 "dispatch_two_kernels_us": round(two.loop_us(two.dispatch, 50), 2),
+                                 "combine_us": round(one.loop_us(one.combine, 50), 2)}
+            del one, two
     if args.calibration_copy:
         calibration_copy(torch, dev)
     result = {"metric": "low-latency dispatch+combine us/call, 8 sources x 128 tokens x 7168, top-8 of 256, destination rank 0",
@@ -674,6 +695,8 @@ def bench_low_latency(args, torch, rc, _abi, dev):
             "roofline_combine": {"kernel": "ll_combine_kernel", "bound": "hbm", "achieved": round(c_bytes / c_us * 1e-3, 1),
                                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(c_bytes / c_us * 1e-3 / HBM_PEAK_GBS, 4),
                                  "traffic": MEASURED_TRAFFIC_BYTES.get(("C5", "packed", "fp8", "ll_combine"))}}
+    if sweep is not None:
+        result["low_latency_batch_sweep"] = sweep
     result["us_per_api_call"] = low_latency_api_figures(torch, ll, kernel_us=(d_us, c_us))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_low_latency(*ll.cpu_inputs, R, M, E)

@@ -764,7 +764,7 @@ hipError_t launch_ll_dispatch(const LLDispatchParams& p, hipStream_t stream) {
     // the routing table of the single-kernel path, plus one spare 32-bit word per lane
     const size_t fused_lds = size_t(p.E_l) * ((total_tokens + 63) / 64) * sizeof(uint64_t) + kWaveSize * sizeof(uint32_t);
     const bool table_fits = (reinterpret_cast<uintptr_t>(p.topk_idx) & 15) == 0 && total_tokens * p.K >= 2 && p.H >= 16;
-    if (total_tokens <= 4096 && fused_lds <= 33 * 1024 && table_fits && !p.two_kernels) {
+    if (total_tokens <= 3072 && fused_lds <= 33 * 1024 && table_fits && !p.two_kernels) {      // beyond: the pair is as fast
         const int threads = p.threads != 0 ? p.threads : 512;
         if (threads == 256) return launch_fused_by_width<256>(p, stream, fused_lds);
         if (threads == 1024) return launch_fused_by_width<1024>(p, stream, fused_lds);

@@ -261,9 +261,9 @@ __global__ __launch_bounds__(kMoveThreads) void ll_move_kernel(const LLDispatchP
 // one workgroup per compute unit can take (kSeveralItems).
 //
 // The kernel is bound by the chain of dependent phases of one wavefront, not by memory bandwidth: the routing pass alone
-// costs every workgroup a dozen instructions per index entry.  So the index loads are the first thing on the memory pipeline (the pass can
-// start as soon as they are back), the payload loads queue up behind them and land while the pass runs, and the
-// pass itself is kept short: one token id per pair of entries, unpredicated 32-bit LDS atomics, range and
+// costs every workgroup a dozen instructions per index entry.  So the index loads are the first thing on the memory
+// pipeline (the pass can start as soon as they are back), the payload loads queue up behind them and land while the pass
+// runs, and the pass itself is kept short: one token id per pair of entries, unpredicated 32-bit LDS atomics, range and
 // duplicate checks left to the wavefront that later moves the token.
 template <int kPairs, bool kFp8, int kFusedThreads, bool kSeveralItems>
 __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatchParams p, const int tiles) {
@@ -298,8 +298,7 @@ __global__ __launch_bounds__(kFusedThreads) void ll_fused_kernel(const LLDispatc
     bool live = place_of(gu, t) && has_work;
 
     // Pass over the whole index table: 16-byte loads (two entries), fully coalesced, a batch of a thread's loads in
-    // flight at once (addresses are clamped instead of predicated, so no load waits for another).  The first batch -
-    // for decode sizes the only one - goes out here, ahead of everything else.
+    // flight at once.  The first batch - for decode sizes the only one - goes out here, ahead of everything else.
     // Everything up to the pass is straight-line code without a branch around any load: where control flow merges the
     // compiler can no longer tell how many loads are younger than the one it waits for and waits for all of them - the
     // pass would sit there until the payload had arrived.  So addresses are clamped instead of predicated (the launcher

@@ -362,7 +362,7 @@ def main():
     ap.add_argument("--overlap", action="store_true",
                     help="also time dispatch and combine on a stream of their own while matrix products fill the GPU on another")
     ap.add_argument("--persistent-movers", type=int, default=0,
-                    help="dispatch move phase as a persistent kernel with this many workgroups per compute unit (implies two launches)")
+                    help="dispatch move phase as a persistent kernel with a work queue and this many mover wavefronts per compute unit: 4, 8 or 15 (implies two launches)")
     ap.add_argument("--brief", action="store_true", help="only the headline workload: no other workloads, no API-level figures")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -345,6 +345,8 @@ int dispatch_with_workspace(const deep_ep_hip_dispatch_args* a, void* workspace,
         m.warm_rounds = a->tuning.warm_rounds;
         m.persistent_movers = a->tuning.persistent_movers;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
+        m.gates = reinterpret_cast<uint32_t*>(ws + w.gates);               // a persistent move kernel keeps its item counter there
+        m.gates_finished = reinterpret_cast<uint32_t*>(ws + w.gates_finished);
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 
         hipError_t err = launch_dispatch_move(m, stream);
@@ -676,6 +678,8 @@ int deep_ep_hip_launch_intranode_dispatch(const deep_ep_hip_intranode_dispatch_a
         m.warm_rounds = a->tuning.warm_rounds;
         m.persistent_movers = a->tuning.persistent_movers;
         m.plain_loads = a->tuning.plain_loads; m.xcd_remap = a->tuning.xcd_remap;
+        m.gates = reinterpret_cast<uint32_t*>(ws + w.gates);               // a persistent move kernel keeps its item counter there
+        m.gates_finished = reinterpret_cast<uint32_t*>(ws + w.gates_finished);
         if (plan.fused) fill_fused(m, lay, plan, ws, w);
 
         m.rank_lanes = with_topk ? 0 : 1;

@@ -866,46 +866,92 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
     }
 }
 
-// ---- the same move as a persistent kernel (tuning.persistent_movers) ----
-// A few workgroups per compute unit stay resident and their wavefronts loop over the work items (wavefront w takes items
-// w, w + W, w + 2W, ...), with the loads of the next item - payload tile, top-k ids, weights, position words - issued
-// before the current item is converted and stored.  Kept as a measured alternative, not a default: on MI355X it is
-// slower than one short-lived wavefront per work item (8192 x 7168 FP8, move phase on a finished layout: 96 / 103 / 96 us
-// with four / six / eight workgroups per compute unit against 82 us).  A likely reason: one counter orders a wavefront's
-// loads and stores, so a looping wavefront waits for the acknowledgement of the stores of item i before it can use the
-// loads of item i + 1 that were issued behind them, while a short-lived wavefront hands its stores to the memory system
-// and leaves, and the next one starts with an empty queue.
+// ---- the same move as a persistent kernel with a work queue (tuning.persistent_movers) ----
+// One workgroup per compute unit stays resident: a few mover wavefronts and a feeder.  Items (token, column tile) are
+// handed out in chunks.  A chunk owns sixteen consecutive tickets of the workgroup's ticket counter (LDS) whatever its
+// size; a mover draws a ticket, looks the chunk up in a ring of 64-bit words (chunk number, size, first item) and takes
+// item `first + offset`, or draws again if the offset lies past the chunk's size.  It requests the loads of its next item
+// - payload tile, top-k id, weight, position word, base row of the destination rank - before it converts and stores the
+// current one.  The feeder keeps the ring one chunk ahead of the ticket counter: it asks one global counter for chunks
+// (one atomic per chunk; the chunks shrink towards the end so that the workgroups run dry together) and posts them; a
+// chunk of size zero ends the workgroup.  A feeder that sees the end reports to a wrapping counter at once - its workgroup
+// asks for nothing after that - and the last one to report puts the global counter back to zero for the next launch.
+//
+// Kept as a measured alternative, not a default: on MI355X (8192 x 7168 FP8, move phase on a finished layout) it takes
+// 86-95 us from launch to launch against 81 us for one short-lived wavefront per item.  With a static split of the items
+// instead of the queue the same loop took 95-104 us: wavefronts get through their items at very different speeds, and
+// the slowest ones set the time.  Whether a looping wavefront waits for the acknowledgement of its own stores before it
+// uses the loads it issued ahead made no difference when measured (look-ahead loads issued by hand and waited for by
+// count, the stores left in flight).
+constexpr int kQueueSlot = 16;               // tickets per chunk
+constexpr int kQueueStatic = 2;              // chunks a workgroup owns by index (no atomic)
+constexpr int kQueueRing = 16;
+constexpr int kQueueCounterLine = 128;       // the gate line (kernels.h) that serves as the global item counter
+
+__device__ __forceinline__ unsigned long long queue_word(unsigned chunk, unsigned size, unsigned base) {
+    return ((unsigned long long)(((chunk + 1u) << 8) | size) << 32) | base;
+}
+
+// Everything a mover needs of one item, requested together.
 template <int kPairs>
-struct CastItem {
+struct QueuedItem {
     vec16 in[kPairs][2];
-    RouteInputs route_in;
-    uint32_t word;
+    int64_t raw;         // topk_idx entry of routing lane min(lane, K - 1)
+    float w;             // its weight
+    uint32_t word;       // its position word
+    int base;            // base row of (rank min(lane, R - 1), the token's chunk)
 };
 
 template <int kPairs>
-__device__ __forceinline__ void load_cast_item(const MoveParams& p, unsigned work, int lane, CastItem<kPairs>& item) {
+__device__ __forceinline__ void load_queued_item(const MoveParams& p, unsigned work, int lane, QueuedItem<kPairs>& item) {
     const int t = int(work / unsigned(p.tiles));
     const int tile = int(work - unsigned(t) * unsigned(p.tiles));
+    const int64_t at = int64_t(t) * p.K + min(lane, p.K - 1);
+    item.raw = p.topk_idx[at];
+    item.word = p.pos[at];
+    item.w = p.topk_weights != nullptr ? p.topk_weights[at] : 0.f;
+    item.base = layout_word(p.tab.rank_bases + int64_t(min(lane, p.R - 1)) * p.tab.chunks_padded + t / kLayoutChunk);
     const uint8_t* src = p.x + int64_t(t) * p.row_bytes;
 #pragma unroll
     for (int q = 0; q < kPairs; ++q) {
-        const int elem = (tile * kPairs + q) * 1024 + lane * 16;
-        item.in[q][0] = vec16{0, 0, 0, 0};
-        item.in[q][1] = vec16{0, 0, 0, 0};
-        if (elem < p.H) {
-            item.in[q][0] = load16_stream(src + int64_t(elem) * 2);
-            item.in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
-        }
+        // a segment past the end of the row reads the row's last 32 bytes instead (never stored)
+        const int elem = min((tile * kPairs + q) * 1024 + lane * 16, p.H - 16);
+        item.in[q][0] = load16_stream(src + int64_t(elem) * 2);
+        item.in[q][1] = load16_stream(src + int64_t(elem) * 2 + 16);
     }
-    item.route_in = load_route_inputs(p, t, lane);
-    item.word = load_position_word(p, t, lane);
 }
 
+// Routes, converts and stores one item: resolve_route for the one case this kernel is launched for (compact layout, no
+// cached handle, top-k routing, at most 64 ranks), with every word it needs already requested.
 template <int kPairs>
-__device__ __forceinline__ void finish_cast_item(const MoveParams& p, unsigned work, int lane, const CastItem<kPairs>& item) {
+__device__ __forceinline__ void finish_queued_item(const MoveParams& p, unsigned work, int lane, const QueuedItem<kPairs>& item,
+                                                   int start_of_rank) {
     const int t = int(work / unsigned(p.tiles));
     const int tile = int(work - unsigned(t) * unsigned(p.tiles));
-    const Route r = resolve_route<false>(p, item.route_in, item.word, nullptr, 0, t, lane, tile == 0);
+    Route r{-1, -1, -1, -1, -1, lane < p.K ? item.w : 0.f};
+    int slot = -1;
+    if (lane < p.K) {
+        if (item.raw >= 0 && item.raw < p.E) r.e = int(item.raw);
+        slot = (item.word & kNoPosition) == kNoPosition ? -1 : int(item.word & kNoPosition);
+    }
+    if (r.e >= 0) r.d = small_div(r.e, p.rcp_E_l);
+    else slot = -1;
+    {
+        const int from = r.d >= 0 ? r.d : 0;
+        const int base = __shfl(item.base, from, kWaveSize);
+        const int start = __shfl(start_of_rank, from, kWaveSize);
+        if (r.d >= 0 && slot >= 0) {
+            r.row_c = base + slot;
+            slot = r.row_c - start;             // slot inside the destination bucket
+        }
+    }
+    if (tile == 0 && lane < p.K && p.dst_buffer_slot_idx != nullptr)
+        p.dst_buffer_slot_idx[int64_t(t) * p.K + lane] = (r.e >= 0 && slot >= 0) ? p.rank_idx * p.M + slot : -1;
+    for (int j = 0; j < p.K; ++j) {
+        const int dj = read_lane(r.d, j);
+        const int rj = read_lane(r.row_c, j);
+        if (r.d >= 0 && dj == r.d && rj >= 0) r.my_row = rj;
+    }
     if (tile == 0) write_token_metadata(p, r, t, lane);
     vec16 out[kPairs];
     float my_scale = 0.f;
@@ -933,25 +979,100 @@ __device__ __forceinline__ void finish_cast_item(const MoveParams& p, unsigned w
     }
 }
 
-template <int kPairs>
-__global__ __launch_bounds__(kThreads) void dispatch_cast_persistent_kernel(const MoveParams p) {
+template <int kPairs, int kQueueThreads>
+__global__ __launch_bounds__(kQueueThreads) void dispatch_cast_queue_kernel(const MoveParams p) {
+    constexpr int kQueueWaves = kQueueThreads / kWaveSize;
+    __shared__ unsigned ticket;
+    __shared__ unsigned long long ring[kQueueRing];
     const int lane = threadIdx.x & 63;
     const unsigned total = unsigned(p.T) * unsigned(p.tiles);
-    const unsigned stride = gridDim.x * unsigned(kWavesPerBlock);
-    unsigned work = wave_work_index(blockIdx.x, kWavesPerBlock);
+    const unsigned static_items = gridDim.x * unsigned(kQueueStatic * kQueueSlot);
+    uint32_t* counter = p.gates + kQueueCounterLine * kDispatchGateStride;
+    if (threadIdx.x < kQueueRing) {
+        const unsigned c = threadIdx.x;
+        unsigned long long word = 0ull;
+        if (c < unsigned(kQueueStatic)) {
+            const unsigned base = (blockIdx.x * unsigned(kQueueStatic) + c) * unsigned(kQueueSlot);
+            word = queue_word(c, base < total ? min(unsigned(kQueueSlot), total - base) : 0u, base);
+        }
+        ring[c] = word;
+        if (c == 0) ticket = 0u;
+    }
+    __syncthreads();
+
+    if ((threadIdx.x >> 6) == kQueueWaves - 1) {
+        // ---- the feeder (one lane) ----
+        if (lane != 0) return;
+        unsigned posted = kQueueStatic;
+        bool ended = (blockIdx.x * unsigned(kQueueStatic) + unsigned(kQueueStatic) - 1u) * unsigned(kQueueSlot) >= total;
+        unsigned size = kQueueSlot;
+        unsigned polls = 0;
+        while (!ended) {
+            const unsigned drawing = __hip_atomic_load(&ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) / unsigned(kQueueSlot);
+            if (posted > drawing + 1u) {                    // the chunk being drawn and one more are there
+                __builtin_amdgcn_s_sleep(8);
+                if (++polls > (1u << 26)) {                 // movers that never draw again: give up, and say so
+                    atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+                    break;
+                }
+                continue;
+            }
+            const unsigned base = static_items + atomicAdd(counter, size);
+            if (base >= total) {
+                __hip_atomic_store(&ring[posted % kQueueRing], queue_word(posted, 0u, total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                ended = true;
+            } else {
+                __hip_atomic_store(&ring[posted % kQueueRing], queue_word(posted, min(size, total - base), base), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+                ++posted;
+                const unsigned left = total - base;
+                size = left > total / 4u ? 16u : left > total / 16u ? 8u : 4u;
+            }
+        }
+        if (atomicInc(p.gates_finished, gridDim.x - 1u) == gridDim.x - 1u) atomicExch(counter, 0u);
+        return;
+    }
+
+    // ---- a mover ----
+    // The wavefront's next item, or `total` for none.
+    auto draw = [&]() {
+        for (;;) {
+            unsigned n = 0;
+            if (lane == 0) n = __hip_atomic_fetch_add(&ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            n = unsigned(__builtin_amdgcn_readfirstlane(int(n)));
+            const unsigned c = n / unsigned(kQueueSlot), o = n % unsigned(kQueueSlot);
+            unsigned long long word;
+            unsigned spins = 0;
+            for (;;) {
+                word = __hip_atomic_load(&ring[c % kQueueRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (unsigned(word >> 40) == c + 1u) break;
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > (1u << 24)) {                 // cannot happen while the feeder makes progress
+                    if (lane == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
+                    return total;
+                }
+            }
+            const unsigned size = unsigned(word >> 32) & 0xffu;
+            if (size == 0u) return total;
+            if (o < size) return unsigned(word) + o;
+        }
+    };
+
+    unsigned work = draw();
     if (work >= total) return;
-    CastItem<kPairs> a, b;
-    load_cast_item<kPairs>(p, work, lane, a);
-    for (;;) {                                         // every wavefront leaves through one of the two breaks
-        unsigned next = work + stride;
-        if (next < total) load_cast_item<kPairs>(p, next, lane, b);
-        finish_cast_item<kPairs>(p, work, lane, a);
-        if (next >= total) break;
-        work = next;
-        next = work + stride;
-        if (next < total) load_cast_item<kPairs>(p, next, lane, a);
-        finish_cast_item<kPairs>(p, work, lane, b);
-        if (next >= total) break;
+    const int start_of_rank = layout_word(p.tab.rank_bases + int64_t(min(lane, p.R - 1)) * p.tab.chunks_padded);
+    QueuedItem<kPairs> cur;
+    load_queued_item<kPairs>(p, work, lane, cur);
+    for (;;) {                                              // every mover leaves through the first branch
+        const unsigned next = draw();
+        if (next >= total) {
+            finish_queued_item<kPairs>(p, work, lane, cur, start_of_rank);
+            return;
+        }
+        QueuedItem<kPairs> ahead;
+        load_queued_item<kPairs>(p, next, lane, ahead);
+        finish_queued_item<kPairs>(p, work, lane, cur, start_of_rank);
+        cur = ahead;
         work = next;
     }
 }
@@ -1159,9 +1280,14 @@ hipError_t launch_cast(MoveParams p, hipStream_t stream) {
     }
     if (p.fused) return hipErrorInvalidConfiguration;      // the launch plan keeps wider tiles out of the single launch
     if constexpr (kPairs <= 2) {
-        if (p.persistent_movers > 0) {
-            const unsigned resident = unsigned(compute_units()) * unsigned(p.persistent_movers > 8 ? 8 : p.persistent_movers);
-            hipLaunchKernelGGL((dispatch_cast_persistent_kernel<kPairs>), dim3(resident < blocks ? resident : blocks), dim3(kThreads), 0, stream, p);
+        if (p.persistent_movers > 0 && !p.cached && !p.do_expand && p.route_mask == nullptr && p.R <= kWaveSize &&
+            p.send_head == nullptr && p.H >= 16 && p.gates != nullptr && p.gates_finished != nullptr) {
+            const int64_t items = int64_t(p.T) * p.tiles;
+            const int64_t wanted = (items + kQueueSlot * kQueueStatic - 1) / (kQueueSlot * kQueueStatic);
+            const unsigned grid = unsigned(std::min<int64_t>(wanted, compute_units()));
+            if (p.persistent_movers <= 4) hipLaunchKernelGGL((dispatch_cast_queue_kernel<kPairs, 320>), dim3(grid), dim3(320), 0, stream, p);
+            else if (p.persistent_movers <= 8) hipLaunchKernelGGL((dispatch_cast_queue_kernel<kPairs, 576>), dim3(grid), dim3(576), 0, stream, p);
+            else hipLaunchKernelGGL((dispatch_cast_queue_kernel<kPairs, 1024>), dim3(grid), dim3(1024), 0, stream, p);
             return hipGetLastError();
         }
     }

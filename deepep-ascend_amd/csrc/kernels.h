@@ -9,7 +9,9 @@
 namespace deep_ep_hip {
 
 // Single-launch dispatch: number of completion counters ("gates") the movers spread over, and the distance between
-// two of them in 32-bit words (one cache line each).
+// two of them in 32-bit words (one cache line each).  A persistent move kernel (never part of a single launch) keeps its
+// item counter in one of these lines and counts its workgroups out on `gates_finished`; every launch leaves all of them
+// at zero.
 constexpr int kDispatchGates = 256;
 constexpr int kDispatchGateStride = 32;
 constexpr int kMaxCountBlocks = 1024;
@@ -164,7 +166,7 @@ struct MoveParams {
     unsigned mover_spin_limit;   // reads a mover repeats for a word of the layout before it gives up (set from the tuning block)
     int move_workgroups_per_cu;  // forced residency of a move kernel on a finished layout, 0 = choose (tuning block)
     int warm_rounds;             // rounds ahead the first movers of a single launch warm the caches, 0 = choose, < 0 = none (tuning block)
-    int persistent_movers;       // fused-cast move kernel on a finished layout as a persistent kernel with this many workgroups per CU, 0 = off (tuning block)
+    int persistent_movers;       // fused-cast move kernel on a finished layout as a persistent kernel with a work queue and this many mover wavefronts per CU, 0 = off (tuning block)
     uint32_t* generation;        // see WorkspaceLayout
     uint32_t* tagged;            // the tagged tables, tagged_words long: cleared by the launch that uses the last tag
     int tagged_words;

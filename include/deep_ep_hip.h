@@ -97,10 +97,12 @@ typedef struct {
                                   load, into the caches only, the tiles of the work items this many rounds of resident
                                   workgroups ahead of their own (0 = 2, or 1 in launches of one and a half to two rounds;
                                   negative = none) */
-    int32_t persistent_movers; /* fused-cast dispatch: > 0 = the move phase as a persistent kernel, this many workgroups per
-                                  compute unit (1..8), whose wavefronts loop over the work items with the next item's loads
-                                  issued before the current item's stores; implies layout kernel + move kernel.  A measured
-                                  alternative (slower on MI355X), not a default */
+    int32_t persistent_movers; /* fused-cast dispatch, compact layout: > 0 = the move phase as a persistent kernel with a
+                                  work queue - one resident workgroup per compute unit with this many mover wavefronts (4, 8
+                                  or 15 are built; other values take the next larger) that draw their items from a counter and
+                                  request the next item's loads before the current item's stores; implies layout kernel +
+                                  move kernel.  Calls it does not cover (expanded layout, cached handle, mask routing) run
+                                  as if it were 0.  A measured alternative (slower on MI355X), not a default */
     int32_t reserved[2];
 } deep_ep_hip_tuning;
 

@@ -15,7 +15,7 @@ KNOBS = [
     ("cast_pairs", 1), ("cast_pairs", 4), ("cast_pairs", 7), ("cast_pairs", 8), ("copy_vecs", 1), ("copy_vecs", 2),
     ("copy_vecs", 7), ("copy_vecs", 8), ("combine_vecs", 1), ("combine_vecs", 4),
     ("move_workgroups_per_cu", 3), ("move_workgroups_per_cu", 8), ("warm_rounds", -1), ("warm_rounds", 1),
-    ("persistent_movers", 1), ("persistent_movers", 6),
+    ("persistent_movers", 4), ("persistent_movers", 8), ("persistent_movers", 15),
 ]
 
 
@@ -56,6 +56,30 @@ def test_dispatch_and_combine_under_knob(knob):
     assert_equal(out + 0.0, ref_out + 0.0, "combined_x")
     assert_equal(out_w, ref_w, "combined_topk_weights")
     buf.check_device_status()
+
+
+@pytest.mark.parametrize("tokens,hidden", [(1, 1024), (37, 2304), (5000, 7168)], ids=["one_token", "under_one_chunk", "dynamic_chunks"])
+def test_persistent_movers_work_queue(tokens, hidden, monkeypatch):
+    """The persistent move kernel draws its items from counters that it has to leave at zero, and it shares them with the
+    single-launch dispatch: launches of both kinds, one after the other on one buffer, from a call smaller than one chunk
+    to one that goes round the global counter many times."""
+    import deep_ep
+    case = rc.small("queue", tokens, hidden, 64, 8, 6, seed=44, masked_ratio=0.1)
+    buf = _buffer(case)
+    x, idx, w = case.x.cuda(), case.topk_idx.cuda(), case.topk_weights.cuda()
+    q = oracle.per_token_cast_to_fp8(case.x)
+    ref = oracle.dispatch(q, case.topk_idx, case.topk_weights, case.E, case.R, 0, case.M)
+    n = ref.num_recv_tokens
+    for movers in (8, 0, 15, 4, 0, 8):
+        monkeypatch.setattr(deep_ep.tuning, "persistent_movers", movers)
+        (rx, rsf), ridx, rw, handle, _ = buf.dispatch(x, idx, w, num_experts=case.E, cast_to_fp8=True, do_cpu_sync=False)
+        assert_equal(rx[:n], ref.recv_x, f"fused FP8 payload, {movers} movers")
+        assert_equal(rsf[:n], ref.recv_sf, f"fused FP8 scales, {movers} movers")
+        assert_equal(ridx[:n], ref.recv_topk_idx, f"recv_topk_idx, {movers} movers")
+        assert_equal(rw[:n], ref.recv_topk_weights, f"recv_topk_weights, {movers} movers")
+        assert_equal(handle.dst_buffer_slot_idx, ref.dst_buffer_slot_idx, f"dst_buffer_slot_idx, {movers} movers")
+        assert_equal(handle.recv_src_metadata[:n], ref.recv_src_metadata, f"recv_src_metadata, {movers} movers")
+        buf.check_device_status()
 
 
 LL_KNOBS = [("ll_threads", 256), ("ll_threads", 1024), ("ll_pairs", 1), ("ll_pairs", 2), ("ll_two_kernels", 1),

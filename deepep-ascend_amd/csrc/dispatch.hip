@@ -1047,7 +1047,7 @@ __global__ __launch_bounds__(kQueueThreads) void dispatch_cast_queue_kernel(cons
                 word = __hip_atomic_load(&ring[c % kQueueRing], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 if (unsigned(word >> 40) == c + 1u) break;
                 __builtin_amdgcn_s_sleep(2);
-                if (++spins > (1u << 24)) {                 // cannot happen while the feeder makes progress
+                if (++spins > (1u << 24)) {                 // a feeder that makes no progress, or a slot that went on to a later chunk
                     if (lane == 0) atomicOr(p.status, DEEP_EP_HIP_STATUS_LAYOUT_TIMEOUT);
                     return total;
                 }

@@ -26,7 +26,7 @@ def _draw(seed):
                 expand=rnd.random() < 0.5, alignment=rnd.choice([1, 1, 4, 16, 128]), zero_pad=rnd.random() < 0.5,
                 cpu_sync=rnd.random() < 0.5, rank=rnd.randrange(R), launches=rnd.choice([0, 1, 2]),
                 col_major=rnd.random() < 0.3, weights=rnd.random() < 0.8, biases=rnd.choice([0, 1, 2]),
-                multi_red=rnd.random() < 0.5)
+                multi_red=rnd.random() < 0.5, persistent=rnd.choice([0, 0, 0, 4, 8, 15]))
 
 
 @pytest.mark.parametrize("seed", range(int(os.environ.get("DEEP_EP_TEST_RANDOM_CASES", "60"))))    # more for a longer hunt
@@ -34,6 +34,7 @@ def test_random_configuration(seed, monkeypatch):
     import deep_ep
     c = _draw(1000 + seed)
     monkeypatch.setattr(deep_ep.tuning, "dispatch_launches", c["launches"])
+    monkeypatch.setattr(deep_ep.tuning, "persistent_movers", c["persistent"])      # takes effect on compact fused-cast dispatches
     case = rc.small(f"rnd{seed}", c["T"], c["H"], c["E"], c["R"], c["K"], seed=seed, masked_ratio=c["masked"])
     M = case.M + (seed % 3) * 17                      # capacity above the token count on two of three cases
     buf = deep_ep.ElasticBuffer(deep_ep.LogicalGroup(c["rank"], c["R"]), num_max_tokens_per_rank=M, hidden=c["H"],

@@ -363,11 +363,22 @@ def main():
                     help="also time dispatch and combine on a stream of their own while matrix products fill the GPU on another")
     ap.add_argument("--persistent-movers", type=int, default=0,
                     help="dispatch move phase as a persistent kernel with a work queue and this many mover wavefronts per compute unit: 4, 8 or 15 (implies two launches)")
+    ap.add_argument("--wave-spans", action="store_true",
+                    help="fused-cast compact dispatch only: load the measurement build of the library (mover wavefronts record "
+                         "their start and end) and report the span of a launch's wavefronts beside its launch-to-launch time")
     ap.add_argument("--brief", action="store_true", help="only the headline workload: no other workloads, no API-level figures")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (logical ranks share its HBM); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.wave_spans:
+        stamps_lib = os.path.join(ROOT, "deepep-ascend_amd", "deep_ep", "libdeep_ep_hip_stamps.so")
+        if not os.path.exists(stamps_lib) or args.bf16 or args.expanded or args.workload == "C5" or args.persistent_movers:
+            print("bench.py: --wave-spans needs libdeep_ep_hip_stamps.so (python deepep-ascend_amd/build.py) and the fused-cast "
+                  "compact dispatch", file=sys.stderr)
+            sys.exit(2)
+        os.environ["DEEP_EP_HIP_LIBRARY"] = stamps_lib
 
     import torch
     import routing_cases as rc
@@ -527,6 +538,9 @@ def main():
     if args.overlap:
         result["under_compute_load"] = under_compute_load(torch, dev, rt)
 
+    if args.wave_spans:
+        result["wave_spans_us"] = wave_spans(torch, _abi, rt, timed, k)
+
     headline = (args.workload == "C3" and fp8 and not expanded and args.routing == "case" and not args.l2_flush and
                 not args.fresh_input and args.persistent_movers == 0)
     if headline and not args.brief:
@@ -537,6 +551,33 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens, fp8, expanded)
     print(json.dumps(result))
+
+
+def wave_spans(torch, _abi, rt, timed, iters):
+    """With the measurement build of the library: for the whole dispatch (one launch) and for its move phase on a finished
+    layout, the launch-to-launch time of a hot loop, and for the loop's last launch the time from the start of its first
+    mover wavefront to the moment the last one had issued its stores / had them acknowledged (100 MHz wall clock).  The
+    stamps cost every wavefront a wait for its own stores, so the launches are a little longer than the library's."""
+    import numpy as np
+    pairs = rt.d.tuning.cast_pairs if rt.d.tuning.cast_pairs in (1, 2) else (1 if rt.H <= 1024 else 2)
+    waves = rt.T * ((rt.H + pairs * 1024 - 1) // (pairs * 1024))
+    out = {"wavefronts": waves}
+    for name, phases in (("dispatch", _abi.PHASE_LAYOUT | _abi.PHASE_MOVE), ("dispatch_move", _abi.PHASE_MOVE)):
+        for _ in range(10):                              # the loop below starts from the state its own launches leave behind
+            rt.dispatch(phases)
+        period = timed(lambda: rt.dispatch(phases), iters)
+        torch.cuda.synchronize()
+        raw = (ctypes.c_longlong * (3 * waves))()
+        if _abi.lib.deep_ep_hip_debug_wave_stamps(raw, waves) != 0:
+            raise RuntimeError("reading the wavefront stamps failed")
+        a = np.frombuffer(raw, dtype=np.int64).reshape(waves, 3)
+        first = a[:, 0].min()
+        out[name] = {"launch_to_launch": round(period, 2),
+                     "first_start_to_last_store_issued": round(float(a[:, 1].max() - first) / 100.0, 2),
+                     "first_start_to_last_store_acknowledged": round(float(a[:, 2].max() - first) / 100.0, 2),
+                     "last_wavefront_start": round(float(a[:, 0].max() - first) / 100.0, 2),
+                     "median_wavefront_lifetime": round(float(np.median(a[:, 2] - a[:, 0])) / 100.0, 2)}
+    return out
 
 
 def calibration_copy(torch, dev):

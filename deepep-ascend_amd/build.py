@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "deep_ep")
 LIB_NAME = "libdeep_ep_hip.so"
+STAMPS_LIB_NAME = "libdeep_ep_hip_stamps.so"     # measurement build: mover wavefronts record their start and end (bench.py --wave-spans)
 SOURCES = ["layout.hip", "dispatch.hip", "combine.hip", "low_latency.hip", "api.hip"]
 
 HIPCC_FLAGS = [
@@ -25,6 +26,10 @@ HIPCC_FLAGS = [
 
 def lib_path() -> str:
     return os.path.join(OUT_DIR, LIB_NAME)
+
+
+def stamps_lib_path() -> str:
+    return os.path.join(OUT_DIR, STAMPS_LIB_NAME)
 
 
 def _hipcc() -> str:
@@ -44,8 +49,10 @@ def build_library(force: bool = True, software_fp8: bool = False, verbose: bool 
     hipcc = _hipcc()
 
     def compile_one(src):
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        stamped = src.startswith("stamps:")
+        src = src.split(":")[-1]
+        obj = os.path.join(obj_dir, src.replace(".hip", "_stamps.o" if stamped else ".o"))
+        cmd = [hipcc, *flags, *(["-DDEEP_EP_HIP_WAVE_STAMPS"] if stamped else []), "-c", os.path.join(CSRC, src), "-o", obj]
         res = subprocess.run(cmd, capture_output=True, text=True)
         # the host pass does not know the packed-fp32 feature and says so; that note is harmless
         err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -55,15 +62,17 @@ def build_library(force: bool = True, software_fp8: bool = False, verbose: bool 
             print(err, file=sys.stderr)
         return obj
 
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(len(SOURCES), 8)) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(len(SOURCES) + 1, 8)) as pool:
+        objs = list(pool.map(compile_one, SOURCES + ["stamps:dispatch.hip"]))
+    stamped_dispatch = objs.pop()
     out = lib_path()
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"link failed:\n{res.stderr}")
-    if verbose:
-        print(f"built {out}")
+    for target, members in ((out, objs), (stamps_lib_path(), [stamped_dispatch if o.endswith("dispatch.o") else o for o in objs])):
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *members, "-o", target]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"link failed:\n{res.stderr}")
+        if verbose:
+            print(f"built {target}")
     return out
 
 

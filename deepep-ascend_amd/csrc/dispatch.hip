@@ -751,6 +751,15 @@ __device__ __forceinline__ void dispatch_copy(const MoveParams& p) {
     }
 }
 
+// Measurement build only (-DDEEP_EP_HIP_WAVE_STAMPS, a library of its own that bench.py --wave-spans loads): every mover
+// wavefront of the fused-cast kernels records when it started, when it had issued its last store and when its stores
+// were acknowledged, on the 100 MHz wall clock: the span of a launch's wavefronts beside its launch-to-launch time, the
+// lifetime of a wavefront, how long before the end the last one starts.
+#ifdef DEEP_EP_HIP_WAVE_STAMPS
+constexpr int kMaxStampedWaves = 65536;
+__device__ long long wave_stamps[3 * kMaxStampedWaves];
+#endif
+
 // ---- fused BF16 -> e4m3 cast: lane owns 16 consecutive channels, 8 lanes own one 128-group ----
 template <int kPairs, bool kFused>
 __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
@@ -762,6 +771,9 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
         }
     }
     const int lane = threadIdx.x & 63;
+#ifdef DEEP_EP_HIP_WAVE_STAMPS
+    const long long stamp_start = wall_clock64();
+#endif
     const unsigned mover = blockIdx.x - (kFused ? unsigned(p.count_blocks) + 1u : 0u);
     const unsigned block = p.xcd_remap ? xcd_contiguous_block(mover, p.num_movers) : mover;
     const unsigned work = wave_work_index(block, kWavesPerBlock);
@@ -864,6 +876,16 @@ __device__ __forceinline__ void dispatch_cast(const MoveParams& p) {
         if (owns_scale)
             p.recv_sf[int64_t(row) * p.rsf_ts + int64_t(group) * p.rsf_hs] = __float_as_uint(my_scale);
     }
+#ifdef DEEP_EP_HIP_WAVE_STAMPS
+    if (lane == 0 && work < unsigned(kMaxStampedWaves)) {
+        const long long issued = wall_clock64();
+        wait_for_own_stores();
+        long long* at = wave_stamps + size_t(work) * 3;
+        at[0] = stamp_start;
+        at[1] = issued;
+        at[2] = wall_clock64();
+    }
+#endif
 }
 
 // ---- the same move as a persistent kernel with a work queue (tuning.persistent_movers) ----
@@ -1387,3 +1409,11 @@ hipError_t launch_cast_kernel(const CastParams& p, hipStream_t stream) {
 }
 
 }  // namespace deep_ep_hip
+
+#ifdef DEEP_EP_HIP_WAVE_STAMPS
+// Copies the stamps of the first `waves` mover wavefronts of the last fused-cast launch to `out` (3 * waves values).
+extern "C" int deep_ep_hip_debug_wave_stamps(long long* out, int waves) {
+    if (out == nullptr || waves < 0 || waves > deep_ep_hip::kMaxStampedWaves) return 1;
+    return int(hipMemcpyFromSymbol(out, HIP_SYMBOL(deep_ep_hip::wave_stamps), size_t(waves) * 3 * sizeof(long long)));
+}
+#endif

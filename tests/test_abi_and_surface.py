@@ -34,6 +34,18 @@ def test_library_exports_every_declared_symbol():
     assert _abi.lib.deep_ep_hip_abi_version() == _abi.ABI_VERSION == 4
 
 
+def test_measurement_build_exports_the_same_abi_plus_the_stamp_reader():
+    """libdeep_ep_hip_stamps.so (bench.py --wave-spans) is the product's sources with time stamps in the mover wavefronts:
+    the declared ABI and one more function to read the stamps, which the product library does not have."""
+    import ctypes
+    import os
+    stamps = ctypes.CDLL(os.path.join(os.path.dirname(_abi.library_path()), "libdeep_ep_hip_stamps.so"))
+    for name in header_functions():
+        assert hasattr(stamps, name), f"{name} is missing from the measurement build"
+    assert hasattr(stamps, "deep_ep_hip_debug_wave_stamps")
+    assert not hasattr(_abi.lib, "deep_ep_hip_debug_wave_stamps")
+
+
 def test_ctypes_structs_match_the_header_layout():
     structs = {"deep_ep_hip_layout_args": _abi.LayoutArgs, "deep_ep_hip_dispatch_args": _abi.DispatchArgs,
                "deep_ep_hip_combine_args": _abi.CombineArgs,

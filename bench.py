@@ -379,6 +379,7 @@ def main():
                   "compact dispatch", file=sys.stderr)
             sys.exit(2)
         os.environ["DEEP_EP_HIP_LIBRARY"] = stamps_lib
+        args.brief = True                 # the API-level figures go through the compiled extension, which holds the product library
 
     import torch
     import routing_cases as rc

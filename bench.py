@@ -576,6 +576,8 @@ def wave_spans(torch, _abi, rt, timed, iters):
         out[name] = {"launch_to_launch": round(period, 2),
                      "first_start_to_last_store_issued": round(float(a[:, 1].max() - first) / 100.0, 2),
                      "first_start_to_last_store_acknowledged": round(float(a[:, 2].max() - first) / 100.0, 2),
+                     "first_wavefront_done": round(float(a[:, 2].min() - first) / 100.0, 2),
+                     "wavefronts_done_after_10_us": int((a[:, 2] - first <= 1000).sum()),
                      "last_wavefront_start": round(float(a[:, 0].max() - first) / 100.0, 2),
                      "median_wavefront_lifetime": round(float(np.median(a[:, 2] - a[:, 0])) / 100.0, 2)}
     return out

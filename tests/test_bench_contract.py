@@ -2,9 +2,12 @@
 algorithmic-byte formulas behind `value` and `roofline.achieved` against the per-unit figures of the survey
 (hand-expanded at the headline shape), and that every traffic constant names a committed profile."""
 import importlib.util
+import json
 import os
 import subprocess
 import sys
+
+import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -53,3 +56,22 @@ def test_traffic_constants_point_at_committed_profiles():
     ab = b.algorithmic_bytes(8192, 7168, 8, 256, 8, 43456, 65536)
     measured = b.MEASURED_TRAFFIC_BYTES[("C3", "compact", "fp8", "combine")]
     assert 1.0 <= measured / ab["combine"] < 1.05
+
+
+@pytest.mark.gpu
+def test_wave_spans_through_the_measurement_build():
+    """`bench.py --wave-spans` (the command of profiles/dispatch_wave_spans_C3.md): the measurement build runs the same
+    dispatch, and what it records is consistent - every mover wavefront stamped, the span of the wavefronts inside the
+    launch-to-launch time, the single launch's head later than that of a move on a finished layout."""
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--no-cpu-baseline", "--wave-spans", "--steps", "3",
+                          "--warmup", "2"], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0, res.stderr[-2000:]
+    line = json.loads(res.stdout.strip().splitlines()[-1])
+    spans = line["wave_spans_us"]
+    assert spans["wavefronts"] == 8192 * 4
+    for name in ("dispatch", "dispatch_move"):
+        s = spans[name]
+        assert 0 < s["first_wavefront_done"] < s["last_wavefront_start"] < s["first_start_to_last_store_acknowledged"]
+        assert s["first_start_to_last_store_issued"] <= s["first_start_to_last_store_acknowledged"] < s["launch_to_launch"] + 10
+        assert 1 < s["median_wavefront_lifetime"] < 60
+    assert spans["dispatch"]["first_wavefront_done"] > spans["dispatch_move"]["first_wavefront_done"]

@@ -1,5 +1,5 @@
 """bench.py's side of the driver contract that can be checked without a GPU: the refusal of more than one GPU, the
-algorithmic-byte formulas behind `value` and `roofline.achieved` against the per-unit figures of the survey
+algorithmic-byte formulas behind `value` and `roofline.achieved` against the per-row and per-token byte counts
 (hand-expanded at the headline shape), and that every traffic constant names a committed profile."""
 import importlib.util
 import json
